@@ -1,0 +1,192 @@
+// extern "C" boundary of libbam_hip.so: argument validation + kernel launches.
+// The declarations (with the reference call sites they replace) are in include/bam_hip.h.
+#include "../../include/bam_hip.h"
+
+#include <cstdarg>
+#include <cstdio>
+
+#include "bam_launch.h"
+
+namespace {
+
+thread_local char g_error[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+int check_half_tensor(const char* name, const void* ptr, int64_t sb, int64_t ss, int64_t sh) {
+    if (ptr == nullptr) return fail(BAM_ERR_INVALID_ARGUMENT, "%s: null pointer", name);
+    if (!aligned16(ptr)) return fail(BAM_ERR_INVALID_ARGUMENT, "%s: pointer is not 16-byte aligned", name);
+    if ((sb % 8) || (ss % 8) || (sh % 8))
+        return fail(BAM_ERR_INVALID_ARGUMENT, "%s: strides (%lld, %lld, %lld) must be multiples of 8 elements", name,
+                    (long long)sb, (long long)ss, (long long)sh);
+    return BAM_OK;
+}
+
+int check_f32_tensor(const char* name, const void* ptr, int64_t sb, int64_t ss, int64_t sh) {
+    if (ptr == nullptr) return fail(BAM_ERR_INVALID_ARGUMENT, "%s: null pointer", name);
+    if (!aligned16(ptr)) return fail(BAM_ERR_INVALID_ARGUMENT, "%s: pointer is not 16-byte aligned", name);
+    if ((sb % 4) || (ss % 4) || (sh % 4))
+        return fail(BAM_ERR_INVALID_ARGUMENT, "%s: strides (%lld, %lld, %lld) must be multiples of 4 elements", name,
+                    (long long)sb, (long long)ss, (long long)sh);
+    return BAM_OK;
+}
+
+int check_problem(int B, int S, int Hq, int Hkv, int D, int dtype) {
+    if (B <= 0 || S <= 0 || Hq <= 0 || Hkv <= 0)
+        return fail(BAM_ERR_INVALID_ARGUMENT, "B, S, Hq, Hkv must be positive (got %d, %d, %d, %d)", B, S, Hq, Hkv);
+    if (Hq % Hkv) return fail(BAM_ERR_INVALID_ARGUMENT, "Hq (%d) must be a multiple of Hkv (%d)", Hq, Hkv);
+    if (D != 32 && D != 64 && D != 128)
+        return fail(BAM_ERR_UNSUPPORTED, "head dimension %d is not supported (32, 64 or 128)", D);
+    if (dtype != BAM_DTYPE_F16 && dtype != BAM_DTYPE_BF16)
+        return fail(BAM_ERR_INVALID_ARGUMENT, "dtype %d is neither BAM_DTYPE_F16 nor BAM_DTYPE_BF16", dtype);
+    if (S > BAM_MAX_SEQLEN) return fail(BAM_ERR_UNSUPPORTED, "S = %d exceeds BAM_MAX_SEQLEN = %d", S, BAM_MAX_SEQLEN);
+    return BAM_OK;
+}
+
+int launched(int hip_err, const char* what) {
+    if (hip_err != 0)
+        return fail(BAM_ERR_LAUNCH, "%s: launch failed: %s", what, hipGetErrorString((hipError_t)hip_err));
+    return BAM_OK;
+}
+
+void fill_sizes(bam::AttnParams& p, int B, int S, int Hq, int Hkv, int D, float scale) {
+    p.B = B;
+    p.S = S;
+    p.Hq = Hq;
+    p.Hkv = Hkv;
+    p.D = D;
+    p.num_m = (S + 127) / 128;
+    p.num_n = (S + 31) / 32;
+    p.S_rounded = p.num_m * 128;
+    p.scale = scale;
+}
+
+}  // namespace
+
+#define BAM_TRY(expr)             \
+    do {                          \
+        int rc_ = (expr);         \
+        if (rc_ != BAM_OK) return rc_; \
+    } while (0)
+
+extern "C" {
+
+const char* bam_last_error(void) { return g_error; }
+
+int bam_abi_version(void) { return 1; }
+
+int bam_tile_flags(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int64_t flags_stride_b,
+                   int64_t flags_stride_m, int B, int S, void* stream) {
+    if (bf == nullptr || flags == nullptr) return fail(BAM_ERR_INVALID_ARGUMENT, "bam_tile_flags: null pointer");
+    if (B <= 0 || S <= 0) return fail(BAM_ERR_INVALID_ARGUMENT, "bam_tile_flags: B and S must be positive");
+    if (B > 65535 || (S + 127) / 128 > 65535)
+        return fail(BAM_ERR_UNSUPPORTED, "bam_tile_flags: grid too large (B = %d, S = %d)", B, S);
+    return launched(bam::launch_tile_flags(bf, bf_stride_b, flags, flags_stride_b, flags_stride_m, B, S,
+                                           (hipStream_t)stream),
+                    "bam_tile_flags");
+}
+
+int bam_materialize_mask(const int64_t* bf, int64_t bf_stride_b, uint8_t* out, int B, int S, void* stream) {
+    if (bf == nullptr || out == nullptr) return fail(BAM_ERR_INVALID_ARGUMENT, "bam_materialize_mask: null pointer");
+    if (B <= 0 || S <= 0) return fail(BAM_ERR_INVALID_ARGUMENT, "bam_materialize_mask: B and S must be positive");
+    if (B > 65535 || S > 65535)
+        return fail(BAM_ERR_UNSUPPORTED, "bam_materialize_mask: B and S are limited to 65535 (got %d, %d)", B, S);
+    return launched(bam::launch_materialize_mask(bf, bf_stride_b, out, B, S, (hipStream_t)stream),
+                    "bam_materialize_mask");
+}
+
+int bam_fwd(const void* q, const void* k, const void* v, void* o, float* lse, const int64_t* bf,
+            const int8_t* flags, int64_t q_stride_b, int64_t q_stride_s, int64_t q_stride_h,
+            int64_t k_stride_b, int64_t k_stride_s, int64_t k_stride_h, int64_t v_stride_b,
+            int64_t v_stride_s, int64_t v_stride_h, int64_t o_stride_b, int64_t o_stride_s,
+            int64_t o_stride_h, int64_t bf_stride_b, int64_t flags_stride_b, int64_t flags_stride_m, int B,
+            int S, int Hq, int Hkv, int D, float scale, int dtype, void* stream) {
+    BAM_TRY(check_problem(B, S, Hq, Hkv, D, dtype));
+    BAM_TRY(check_half_tensor("q", q, q_stride_b, q_stride_s, q_stride_h));
+    BAM_TRY(check_half_tensor("k", k, k_stride_b, k_stride_s, k_stride_h));
+    BAM_TRY(check_half_tensor("v", v, v_stride_b, v_stride_s, v_stride_h));
+    BAM_TRY(check_half_tensor("o", o, o_stride_b, o_stride_s, o_stride_h));
+    if (lse == nullptr || bf == nullptr || flags == nullptr)
+        return fail(BAM_ERR_INVALID_ARGUMENT, "bam_fwd: lse, bf and flags must not be null");
+    if (!(scale > 0.f)) return fail(BAM_ERR_INVALID_ARGUMENT, "bam_fwd: softmax scale must be > 0 (got %g)", scale);
+    if ((int64_t)((S + 127) / 128) * B * Hq > 0x7FFFFFFFll) return fail(BAM_ERR_UNSUPPORTED, "bam_fwd: grid too large");
+    bam::AttnParams p = {};
+    p.q = {q, q_stride_b, q_stride_s, q_stride_h};
+    p.k = {k, k_stride_b, k_stride_s, k_stride_h};
+    p.v = {v, v_stride_b, v_stride_s, v_stride_h};
+    p.o = {o, o_stride_b, o_stride_s, o_stride_h};
+    p.lse = lse;
+    p.bf = bf;
+    p.bf_sb = bf_stride_b;
+    p.flags = flags;
+    p.flags_sb = flags_stride_b;
+    p.flags_sm = flags_stride_m;
+    fill_sizes(p, B, S, Hq, Hkv, D, scale);
+    return launched(bam::launch_fwd(p, dtype, (hipStream_t)stream), "bam_fwd");
+}
+
+int bam_bwd_preprocess(const void* o, const void* dout, float* delta, int64_t o_stride_b, int64_t o_stride_s,
+                       int64_t o_stride_h, int64_t do_stride_b, int64_t do_stride_s, int64_t do_stride_h,
+                       int B, int S, int Hq, int D, int dtype, void* stream) {
+    BAM_TRY(check_problem(B, S, Hq, Hq, D, dtype));
+    BAM_TRY(check_half_tensor("o", o, o_stride_b, o_stride_s, o_stride_h));
+    BAM_TRY(check_half_tensor("do", dout, do_stride_b, do_stride_s, do_stride_h));
+    if (delta == nullptr) return fail(BAM_ERR_INVALID_ARGUMENT, "bam_bwd_preprocess: delta must not be null");
+    bam::AttnParams p = {};
+    p.o = {o, o_stride_b, o_stride_s, o_stride_h};
+    p.dout = {dout, do_stride_b, do_stride_s, do_stride_h};
+    p.delta = delta;
+    fill_sizes(p, B, S, Hq, Hq, D, 1.f);
+    return launched(bam::launch_bwd_preprocess(p, dtype, (hipStream_t)stream), "bam_bwd_preprocess");
+}
+
+int bam_bwd(const void* q, const void* k, const void* v, const void* dout, const float* lse,
+            const float* delta, float* dq, float* dk, float* dv, const int64_t* bf, const int8_t* flags,
+            int64_t q_stride_b, int64_t q_stride_s, int64_t q_stride_h, int64_t k_stride_b,
+            int64_t k_stride_s, int64_t k_stride_h, int64_t v_stride_b, int64_t v_stride_s,
+            int64_t v_stride_h, int64_t do_stride_b, int64_t do_stride_s, int64_t do_stride_h,
+            int64_t dq_stride_b, int64_t dq_stride_s, int64_t dq_stride_h, int64_t dk_stride_b,
+            int64_t dk_stride_s, int64_t dk_stride_h, int64_t dv_stride_b, int64_t dv_stride_s,
+            int64_t dv_stride_h, int64_t bf_stride_b, int64_t flags_stride_b, int64_t flags_stride_m, int B,
+            int S, int Hq, int Hkv, int D, float scale, int dtype, void* stream) {
+    BAM_TRY(check_problem(B, S, Hq, Hkv, D, dtype));
+    BAM_TRY(check_half_tensor("q", q, q_stride_b, q_stride_s, q_stride_h));
+    BAM_TRY(check_half_tensor("k", k, k_stride_b, k_stride_s, k_stride_h));
+    BAM_TRY(check_half_tensor("v", v, v_stride_b, v_stride_s, v_stride_h));
+    BAM_TRY(check_half_tensor("do", dout, do_stride_b, do_stride_s, do_stride_h));
+    BAM_TRY(check_f32_tensor("dq", dq, dq_stride_b, dq_stride_s, dq_stride_h));
+    BAM_TRY(check_f32_tensor("dk", dk, dk_stride_b, dk_stride_s, dk_stride_h));
+    BAM_TRY(check_f32_tensor("dv", dv, dv_stride_b, dv_stride_s, dv_stride_h));
+    if (lse == nullptr || delta == nullptr || bf == nullptr || flags == nullptr)
+        return fail(BAM_ERR_INVALID_ARGUMENT, "bam_bwd: lse, delta, bf and flags must not be null");
+    if (!(scale > 0.f)) return fail(BAM_ERR_INVALID_ARGUMENT, "bam_bwd: softmax scale must be > 0 (got %g)", scale);
+    if ((int64_t)((S + 127) / 128) * B * Hq > 0x7FFFFFFFll) return fail(BAM_ERR_UNSUPPORTED, "bam_bwd: grid too large");
+    bam::AttnParams p = {};
+    p.q = {q, q_stride_b, q_stride_s, q_stride_h};
+    p.k = {k, k_stride_b, k_stride_s, k_stride_h};
+    p.v = {v, v_stride_b, v_stride_s, v_stride_h};
+    p.dout = {dout, do_stride_b, do_stride_s, do_stride_h};
+    p.dq = {dq, dq_stride_b, dq_stride_s, dq_stride_h};
+    p.dk = {dk, dk_stride_b, dk_stride_s, dk_stride_h};
+    p.dv = {dv, dv_stride_b, dv_stride_s, dv_stride_h};
+    p.lse = const_cast<float*>(lse);
+    p.delta = const_cast<float*>(delta);
+    p.bf = bf;
+    p.bf_sb = bf_stride_b;
+    p.flags = flags;
+    p.flags_sb = flags_stride_b;
+    p.flags_sm = flags_stride_m;
+    fill_sizes(p, B, S, Hq, Hkv, D, scale);
+    BAM_TRY(launched(bam::launch_bwd_dkdv(p, dtype, (hipStream_t)stream), "bam_bwd (dk/dv)"));
+    return launched(bam::launch_bwd_dq(p, dtype, (hipStream_t)stream), "bam_bwd (dq)");
+}
+
+}  // extern "C"

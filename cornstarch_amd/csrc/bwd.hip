@@ -1,0 +1,486 @@
+// Backward kernels of bitfield-masked attention for gfx950.
+// Reference semantics: cornstarch/kernel/bitfield_attention.py:527-572 (delta) and :598-929
+// (dQ, dK, dV).  The reference accumulates dQ, dK and dV with fp32 atomics; here every output
+// element has exactly one owner, so nothing is atomic and the sums are deterministic:
+//   dkdv kernel : one workgroup per (batch, kv head, 128-key tile); it loops over the q heads
+//                 of the group and over the query blocks its flag column lists.
+//   dq kernel   : one workgroup per (batch, q head, 128-query block), looping over key tiles
+//                 exactly like the forward kernel.
+// Both recompute P = exp(scale * s - lse) from the saved log-sum-exp.
+#include "bam_common.h"
+#include "bam_launch.h"
+#include "bam_tiles.h"
+
+namespace bam {
+
+// ---------------------------------------------------------------------------------------
+// delta[b,h,i] = sum_d o * do   (fp32).  D/8 lanes per row, 16 bytes per lane per tensor.
+template <typename T, int D>
+__global__ __launch_bounds__(256) void bwd_preprocess_kernel(const AttnParams p) {
+    constexpr int LPR = D / 8;
+    const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t row = gid / LPR;
+    const int c = (int)(gid % LPR);
+    const int64_t total = (int64_t)p.B * p.S * p.Hq;
+    const bool valid = row < total;
+    int h = 0, i = 0, b = 0;
+    float acc = 0.f;
+    if (valid) {
+        h = (int)(row % p.Hq);
+        const int64_t bi = row / p.Hq;
+        i = (int)(bi % p.S);
+        b = (int)(bi / p.S);
+        const u32x4 ov = *(const u32x4*)((const char*)p.o.ptr +
+                                         2 * ((int64_t)b * p.o.sb + (int64_t)i * p.o.ss + (int64_t)h * p.o.sh) + c * 16);
+        const u32x4 gv = *(const u32x4*)((const char*)p.dout.ptr +
+                                         2 * ((int64_t)b * p.dout.sb + (int64_t)i * p.dout.ss + (int64_t)h * p.dout.sh) + c * 16);
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+            acc += T::to_float((unsigned short)(ov[x] & 0xFFFFu)) * T::to_float((unsigned short)(gv[x] & 0xFFFFu));
+            acc += T::to_float((unsigned short)(ov[x] >> 16)) * T::to_float((unsigned short)(gv[x] >> 16));
+        }
+    }
+#pragma unroll
+    for (int off = LPR / 2; off > 0; off >>= 1) acc += __shfl_xor(acc, off);
+    if (valid && c == 0) p.delta[((int64_t)b * p.Hq + h) * p.S_rounded + i] = acc;
+}
+
+// ---------------------------------------------------------------------------------------
+// dK, dV.  Wave w owns keys [32w, 32w+32) of the 128-key tile: K and V of those keys stay in
+// registers as MFMA B operands for the whole kernel, dK^T and dV^T (d x keys) stay in
+// accumulators.  Query rows arrive in 32-row tiles of Q and dO through LDS (double buffered).
+// With S = Q K^T computed as queries x keys, a lane of the C fragment owns ONE key and 16
+// query rows, so P and dS feed dV^T = dO^T P and dK^T = Q^T dS as B operands from registers;
+// Q^T and dO^T come from the transposing LDS read of the same row-major tiles.
+constexpr int DKDV_QT = 32;
+constexpr int DKDV_THREADS = 256;
+
+template <typename T, int D>
+__global__ __launch_bounds__(DKDV_THREADS, 1) void bwd_dkdv_kernel(const AttnParams p) {
+    constexpr int NCH = D / 8, KK = D / 16, DB = D / 32;
+    __shared__ u32x4 sQ[2][DKDV_QT * NCH];
+    __shared__ u32x4 sDO[2][DKDV_QT * NCH];
+    __shared__ __attribute__((aligned(16))) float sLse[2][DKDV_QT];
+    __shared__ __attribute__((aligned(16))) float sDelta[2][DKDV_QT];
+    __shared__ __attribute__((aligned(16))) unsigned sQlo[2][DKDV_QT];
+    __shared__ __attribute__((aligned(16))) unsigned sQhi[2][DKDV_QT];
+    __shared__ __attribute__((aligned(16))) int sQlim[2][DKDV_QT];
+    __shared__ int sList[MAX_LIST];
+    __shared__ int sCount;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int hi = lane >> 5, l32 = lane & 31, half16 = (lane >> 4) & 1;
+    const int S = p.S;
+    const int G = p.Hq / p.Hkv;
+
+    const int unit = blockIdx.x;
+    const int hk = unit % p.Hkv;
+    const int ub = unit / p.Hkv;
+    const int b = ub % p.B;
+    const int nt = ub / p.B;  // early key tiles (most queries under causality) first
+
+    if (wave == 0)
+        build_query_block_list(p.flags + (int64_t)b * p.flags_sb, p.flags_sm, p.num_m, p.num_n, nt, lane, sList,
+                               &sCount);
+
+    // ---- per-lane key state ---------------------------------------------------------------
+    const int key = nt * 128 + wave * 32 + l32;
+    const bool kvalid = key < S;
+    u32x4 kreg[KK], vreg[KK];
+    {
+        const char* kp = (const char*)p.k.ptr + 2 * ((int64_t)b * p.k.sb + (int64_t)key * p.k.ss + (int64_t)hk * p.k.sh);
+        const char* vp = (const char*)p.v.ptr + 2 * ((int64_t)b * p.v.sb + (int64_t)key * p.v.ss + (int64_t)hk * p.v.sh);
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) {
+            u32x4 zk = {0u, 0u, 0u, 0u}, zv = {0u, 0u, 0u, 0u};
+            if (kvalid) {
+                zk = *(const u32x4*)(kp + (16 * kk + 8 * hi) * 2);
+                zv = *(const u32x4*)(vp + (16 * kk + 8 * hi) * 2);
+            }
+            kreg[kk] = zk;
+            vreg[kk] = zv;
+        }
+    }
+    const int64_t kf = kvalid ? p.bf[(int64_t)b * p.bf_sb + key] : 0;
+    const unsigned klo = (unsigned)(kf & 0xFFFFFFFFll);
+    const unsigned khi = ((unsigned)((uint64_t)kf >> 32)) & HI_MODALITY_MASK;
+
+    f32x16 dk[DB], dv[DB];
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            dk[db][i] = 0.f;
+            dv[db][i] = 0.f;
+        }
+    const float c2 = p.scale * LOG2E;
+    const int64_t* bfrow = p.bf + (int64_t)b * p.bf_sb;
+
+    TileStage<D, DKDV_QT, DKDV_THREADS> stQ, stDO;
+    float lse_stage = 0.f, delta_stage = 0.f;
+    int64_t qf_stage = 0;
+
+    // iteration `it` -> (q head of the group, list entry, 32-row sub block)
+    auto stage_load = [&](int it, int n) {
+        const int g = it / (4 * n);
+        const int rem = it - g * 4 * n;
+        const int entry = sList[rem >> 2];
+        const int row0 = (entry >> 8) * BLOCK_M + (rem & 3) * DKDV_QT;
+        const int h = hk * G + g;
+        const char* qbase = (const char*)p.q.ptr + 2 * ((int64_t)b * p.q.sb + (int64_t)h * p.q.sh);
+        const char* gbase = (const char*)p.dout.ptr + 2 * ((int64_t)b * p.dout.sb + (int64_t)h * p.dout.sh);
+        stQ.load(qbase, 2 * p.q.ss, row0, S, tid);
+        stDO.load(gbase, 2 * p.dout.ss, row0, S, tid);
+        if (tid < DKDV_QT) {
+            const int r = row0 + tid;
+            const bool ok = r < S;
+            const int64_t off = ((int64_t)b * p.Hq + h) * p.S_rounded + r;
+            const float l = ok ? p.lse[off] : -INFINITY;
+            // rows past the end, and rows that allow no key (lse = -inf), must give P = 0
+            lse_stage = (l == -INFINITY) ? INFINITY : l * LOG2E;
+            delta_stage = ok ? p.delta[off] : 0.f;
+            qf_stage = ok ? bfrow[r] : 0;
+        }
+    };
+    auto stage_store = [&](int it, int n, int buf) {
+        stQ.store(sQ[buf], tid);
+        stDO.store(sDO[buf], tid);
+        if (tid < DKDV_QT) {
+            const int rem = it % (4 * n);
+            const int row0 = (sList[rem >> 2] >> 8) * BLOCK_M + (rem & 3) * DKDV_QT;
+            const QueryBits qb = make_query_bits(qf_stage, row0 + tid);
+            sLse[buf][tid] = lse_stage;
+            sDelta[buf][tid] = delta_stage;
+            sQlo[buf][tid] = qb.lo;
+            sQhi[buf][tid] = qb.hi;
+            sQlim[buf][tid] = qb.lim;
+        }
+    };
+
+    __syncthreads();
+    const int n = sCount;
+    const int total = n * 4 * G;
+    if (total > 0) {
+        stage_load(0, n);
+        stage_store(0, n, 0);
+        __syncthreads();
+        for (int it = 0; it < total; ++it) {
+            const int cur = it & 1;
+            const bool more = it + 1 < total;
+            if (more) stage_load(it + 1, n);
+
+            const int rem = it % (4 * n);
+            const int entry = sList[rem >> 2];
+            const int cls = (entry >> (2 * wave)) & 3;  // this wave's own 128x32 flag
+            if (cls != 0) {
+                // ---- S = Q K^T and dP = dO V^T : 32 queries x 32 keys ---------------------
+                f32x16 s, dp;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    s[i] = 0.f;
+                    dp[i] = 0.f;
+                }
+#pragma unroll
+                for (int kk = 0; kk < KK; ++kk) {
+                    const u32x4 a = lds_read_chunk<D>(sQ[cur], l32, 2 * kk + hi);
+                    s = T::mfma(a, kreg[kk], s);
+                }
+#pragma unroll
+                for (int kk = 0; kk < KK; ++kk) {
+                    const u32x4 a = lds_read_chunk<D>(sDO[cur], l32, 2 * kk + hi);
+                    dp = T::mfma(a, vreg[kk], dp);
+                }
+                // ---- P, dS (C fragment: register i <-> query row 8*(i/4) + 4*hi + i%4) --------
+#pragma unroll
+                for (int grp = 0; grp < 4; ++grp) {
+                    const int roff = 8 * grp + 4 * hi;
+                    const f32x4 l4 = *(const f32x4*)&sLse[cur][roff];
+                    const f32x4 d4 = *(const f32x4*)&sDelta[cur][roff];
+#pragma unroll
+                    for (int x = 0; x < 4; ++x) {
+                        const float e = __builtin_amdgcn_exp2f(fmaf(s[4 * grp + x], c2, -l4[x]));
+                        s[4 * grp + x] = e;
+                        dp[4 * grp + x] = e * (dp[4 * grp + x] - d4[x]) * p.scale;
+                    }
+                }
+                if (cls == 1) {
+#pragma unroll
+                    for (int grp = 0; grp < 4; ++grp) {
+                        const int roff = 8 * grp + 4 * hi;
+                        const u32x4 qlo = *(const u32x4*)&sQlo[cur][roff];
+                        const u32x4 qhi = *(const u32x4*)&sQhi[cur][roff];
+                        const u32x4 qlim = *(const u32x4*)&sQlim[cur][roff];
+#pragma unroll
+                        for (int x = 0; x < 4; ++x) {
+                            QueryBits qb;
+                            qb.lo = qlo[x];
+                            qb.hi = qhi[x];
+                            qb.lim = (int)qlim[x];
+                            qb.text = (qlo[x] & 1u) != 0;
+                            const bool a = allow_pair(qb, klo, khi, key);
+                            s[4 * grp + x] = a ? s[4 * grp + x] : 0.f;
+                            dp[4 * grp + x] = a ? dp[4 * grp + x] : 0.f;
+                        }
+                    }
+                }
+                u32x4 pb[2], dsb[2];
+#pragma unroll
+                for (int t = 0; t < 2; ++t) {
+                    pb[t] = pack8<T>(s, 8 * t);
+                    dsb[t] = pack8<T>(dp, 8 * t);
+                }
+                // ---- dV^T += dO^T P ; dK^T += Q^T dS -------------------------------------------
+#pragma unroll
+                for (int db = 0; db < DB; ++db)
+#pragma unroll
+                    for (int t = 0; t < 2; ++t) {
+                        const u32x4 a = lds_read_transposed<D>(sDO[cur], lane, 16 * t + 4 * hi, 32 * db + 16 * half16);
+                        dv[db] = T::mfma(a, pb[t], dv[db]);
+                    }
+#pragma unroll
+                for (int db = 0; db < DB; ++db)
+#pragma unroll
+                    for (int t = 0; t < 2; ++t) {
+                        const u32x4 a = lds_read_transposed<D>(sQ[cur], lane, 16 * t + 4 * hi, 32 * db + 16 * half16);
+                        dk[db] = T::mfma(a, dsb[t], dk[db]);
+                    }
+            }
+            if (more) stage_store(it + 1, n, cur ^ 1);
+            __syncthreads();
+        }
+    }
+
+    // ---- epilogue: accumulate into the caller's fp32 buffers (sole owner of these rows) -----
+    if (kvalid) {
+        float* dkp = (float*)p.dk.ptr + ((int64_t)b * p.dk.sb + (int64_t)key * p.dk.ss + (int64_t)hk * p.dk.sh);
+        float* dvp = (float*)p.dv.ptr + ((int64_t)b * p.dv.sb + (int64_t)key * p.dv.ss + (int64_t)hk * p.dv.sh);
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int grp = 0; grp < 4; ++grp) {
+                const int d0 = 32 * db + 8 * grp + 4 * hi;
+                f32x4 a = *(f32x4*)(dkp + d0), c = *(f32x4*)(dvp + d0);
+#pragma unroll
+                for (int x = 0; x < 4; ++x) {
+                    a[x] += dk[db][4 * grp + x];
+                    c[x] += dv[db][4 * grp + x];
+                }
+                *(f32x4*)(dkp + d0) = a;
+                *(f32x4*)(dvp + d0) = c;
+            }
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// dQ.  Same decomposition and S^T layout as the forward kernel: a lane owns one query, so
+// lse and delta are per-lane scalars; dS^T feeds dQ^T = K^T dS^T from registers and K^T comes
+// from the transposing LDS read of the K tile that also serves S^T = K Q^T.
+constexpr int DQ_KT = 64;
+constexpr int DQ_THREADS = 256;
+
+template <typename T, int D>
+__global__ __launch_bounds__(DQ_THREADS, 2) void bwd_dq_kernel(const AttnParams p) {
+    constexpr int NCH = D / 8, KK = D / 16, DB = D / 32;
+    __shared__ u32x4 sK[2][DQ_KT * NCH];
+    __shared__ u32x4 sV[2][DQ_KT * NCH];
+    __shared__ __attribute__((aligned(16))) unsigned sKlo[2][DQ_KT];
+    __shared__ __attribute__((aligned(16))) unsigned sKhi[2][DQ_KT];
+    __shared__ int sList[MAX_LIST];
+    __shared__ int sCount;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int hi = lane >> 5, l32 = lane & 31, half16 = (lane >> 4) & 1;
+    const int S = p.S;
+    const int G = p.Hq / p.Hkv;
+
+    int unit, g;
+    xcd_group_map(blockIdx.x, p.num_m * p.B * p.Hkv, G, unit, g);
+    const int hk = unit % p.Hkv;
+    const int ub = unit / p.Hkv;
+    const int b = ub % p.B;
+    const int m = p.num_m - 1 - ub / p.B;
+    const int h = hk * G + g;
+
+    if (wave == 0)
+        build_key_tile_list(p.flags + (int64_t)b * p.flags_sb + (int64_t)m * p.flags_sm, p.num_n, S, lane,
+                            sList, &sCount);
+
+    const int qrow = m * BLOCK_M + wave * 32 + l32;
+    const bool qvalid = qrow < S;
+    u32x4 qreg[KK], greg[KK];
+    {
+        const char* qp = (const char*)p.q.ptr + 2 * ((int64_t)b * p.q.sb + (int64_t)qrow * p.q.ss + (int64_t)h * p.q.sh);
+        const char* gp = (const char*)p.dout.ptr + 2 * ((int64_t)b * p.dout.sb + (int64_t)qrow * p.dout.ss + (int64_t)h * p.dout.sh);
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) {
+            u32x4 zq = {0u, 0u, 0u, 0u}, zg = {0u, 0u, 0u, 0u};
+            if (qvalid) {
+                zq = *(const u32x4*)(qp + (16 * kk + 8 * hi) * 2);
+                zg = *(const u32x4*)(gp + (16 * kk + 8 * hi) * 2);
+            }
+            qreg[kk] = zq;
+            greg[kk] = zg;
+        }
+    }
+    const int64_t qf = qvalid ? p.bf[(int64_t)b * p.bf_sb + qrow] : 0;
+    const QueryBits qb = make_query_bits(qf, qrow);
+    float lse2 = INFINITY, dlt = 0.f;
+    if (qvalid) {
+        const int64_t off = ((int64_t)b * p.Hq + h) * p.S_rounded + qrow;
+        const float l = p.lse[off];
+        lse2 = (l == -INFINITY) ? INFINITY : l * LOG2E;
+        dlt = p.delta[off];
+    }
+
+    f32x16 dq[DB];
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) dq[db][i] = 0.f;
+    const float c2 = p.scale * LOG2E;
+
+    const char* kbase = (const char*)p.k.ptr + 2 * ((int64_t)b * p.k.sb + (int64_t)hk * p.k.sh);
+    const char* vbase = (const char*)p.v.ptr + 2 * ((int64_t)b * p.v.sb + (int64_t)hk * p.v.sh);
+    const int64_t k_rs = 2 * p.k.ss, v_rs = 2 * p.v.ss;
+    const int64_t* bfrow = p.bf + (int64_t)b * p.bf_sb;
+
+    TileStage<D, DQ_KT, DQ_THREADS> stK, stV;
+    int64_t kf_stage = 0;
+
+    __syncthreads();
+    const int n = sCount;
+    if (n > 0) {
+        {
+            const int kt = sList[0] >> 2;
+            stK.load(kbase, k_rs, kt * DQ_KT, S, tid);
+            stV.load(vbase, v_rs, kt * DQ_KT, S, tid);
+            if (tid < DQ_KT) kf_stage = (kt * DQ_KT + tid < S) ? bfrow[kt * DQ_KT + tid] : 0;
+            stK.store(sK[0], tid);
+            stV.store(sV[0], tid);
+            if (tid < DQ_KT) {
+                sKlo[0][tid] = (unsigned)(kf_stage & 0xFFFFFFFFll);
+                sKhi[0][tid] = ((unsigned)((uint64_t)kf_stage >> 32)) & HI_MODALITY_MASK;
+            }
+        }
+        __syncthreads();
+        for (int it = 0; it < n; ++it) {
+            const int cur = it & 1;
+            const int entry = sList[it];
+            const int kt = entry >> 2, cls = entry & 3;
+            const bool more = it + 1 < n;
+            if (more) {
+                const int kt1 = sList[it + 1] >> 2;
+                stK.load(kbase, k_rs, kt1 * DQ_KT, S, tid);
+                stV.load(vbase, v_rs, kt1 * DQ_KT, S, tid);
+                if (tid < DQ_KT) kf_stage = (kt1 * DQ_KT + tid < S) ? bfrow[kt1 * DQ_KT + tid] : 0;
+            }
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb) {
+                f32x16 s, dp;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    s[i] = 0.f;
+                    dp[i] = 0.f;
+                }
+#pragma unroll
+                for (int kk = 0; kk < KK; ++kk) {
+                    const u32x4 a = lds_read_chunk<D>(sK[cur], 32 * kb + l32, 2 * kk + hi);
+                    s = T::mfma(a, qreg[kk], s);
+                }
+#pragma unroll
+                for (int kk = 0; kk < KK; ++kk) {
+                    const u32x4 a = lds_read_chunk<D>(sV[cur], 32 * kb + l32, 2 * kk + hi);
+                    dp = T::mfma(a, greg[kk], dp);
+                }
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const float e = __builtin_amdgcn_exp2f(fmaf(s[i], c2, -lse2));
+                    dp[i] = e * (dp[i] - dlt) * p.scale;
+                }
+                if (cls == 1) {
+                    const int kt0 = kt * DQ_KT;
+#pragma unroll
+                    for (int grp = 0; grp < 4; ++grp) {
+                        const int koff = 32 * kb + 8 * grp + 4 * hi;
+                        const u32x4 klo = *(const u32x4*)&sKlo[cur][koff];
+                        const u32x4 khi = *(const u32x4*)&sKhi[cur][koff];
+#pragma unroll
+                        for (int x = 0; x < 4; ++x)
+                            dp[4 * grp + x] = allow_pair(qb, klo[x], khi[x], kt0 + koff + x) ? dp[4 * grp + x] : 0.f;
+                    }
+                }
+                u32x4 dsb[2];
+#pragma unroll
+                for (int t = 0; t < 2; ++t) dsb[t] = pack8<T>(dp, 8 * t);
+#pragma unroll
+                for (int db = 0; db < DB; ++db)
+#pragma unroll
+                    for (int t = 0; t < 2; ++t) {
+                        const u32x4 a =
+                            lds_read_transposed<D>(sK[cur], lane, 32 * kb + 16 * t + 4 * hi, 32 * db + 16 * half16);
+                        dq[db] = T::mfma(a, dsb[t], dq[db]);
+                    }
+            }
+            if (more) {
+                stK.store(sK[cur ^ 1], tid);
+                stV.store(sV[cur ^ 1], tid);
+                if (tid < DQ_KT) {
+                    sKlo[cur ^ 1][tid] = (unsigned)(kf_stage & 0xFFFFFFFFll);
+                    sKhi[cur ^ 1][tid] = ((unsigned)((uint64_t)kf_stage >> 32)) & HI_MODALITY_MASK;
+                }
+            }
+            __syncthreads();
+        }
+    }
+
+    if (qvalid) {
+        float* dqp = (float*)p.dq.ptr + ((int64_t)b * p.dq.sb + (int64_t)qrow * p.dq.ss + (int64_t)h * p.dq.sh);
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int grp = 0; grp < 4; ++grp) {
+                const int d0 = 32 * db + 8 * grp + 4 * hi;
+                f32x4 a = *(f32x4*)(dqp + d0);
+#pragma unroll
+                for (int x = 0; x < 4; ++x) a[x] += dq[db][4 * grp + x];
+                *(f32x4*)(dqp + d0) = a;
+            }
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+template <typename T, int D>
+static int launch_pre_t(const AttnParams& p, hipStream_t stream) {
+    const int64_t threads = (int64_t)p.B * p.S * p.Hq * (D / 8);
+    const int64_t blocks = (threads + 255) / 256;
+    hipLaunchKernelGGL((bwd_preprocess_kernel<T, D>), dim3((unsigned)blocks), dim3(256), 0, stream, p);
+    return (int)hipGetLastError();
+}
+template <typename T, int D>
+static int launch_dkdv_t(const AttnParams& p, hipStream_t stream) {
+    const int blocks = p.num_m * p.B * p.Hkv;  // ceil(S/128) key tiles
+    hipLaunchKernelGGL((bwd_dkdv_kernel<T, D>), dim3(blocks), dim3(DKDV_THREADS), 0, stream, p);
+    return (int)hipGetLastError();
+}
+template <typename T, int D>
+static int launch_dq_t(const AttnParams& p, hipStream_t stream) {
+    const int blocks = p.num_m * p.B * p.Hq;
+    hipLaunchKernelGGL((bwd_dq_kernel<T, D>), dim3(blocks), dim3(DQ_THREADS), 0, stream, p);
+    return (int)hipGetLastError();
+}
+
+#define BAM_DISPATCH(fn)                                       \
+    if (dtype == 1) {                                          \
+        if (p.D == 128) return fn<BF16, 128>(p, stream);       \
+        if (p.D == 64) return fn<BF16, 64>(p, stream);         \
+        return fn<BF16, 32>(p, stream);                        \
+    }                                                          \
+    if (p.D == 128) return fn<F16, 128>(p, stream);            \
+    if (p.D == 64) return fn<F16, 64>(p, stream);              \
+    return fn<F16, 32>(p, stream);
+
+int launch_bwd_preprocess(const AttnParams& p, int dtype, hipStream_t stream) { BAM_DISPATCH(launch_pre_t) }
+int launch_bwd_dkdv(const AttnParams& p, int dtype, hipStream_t stream) { BAM_DISPATCH(launch_dkdv_t) }
+int launch_bwd_dq(const AttnParams& p, int dtype, hipStream_t stream) { BAM_DISPATCH(launch_dq_t) }
+
+}  // namespace bam

@@ -1,0 +1,81 @@
+// Tile-summary kernel: int64 bitfields -> int8 flag per (128-row, 32-column) tile, and the
+// dense-mask utility.  Integer work only; results are bit exact by construction.
+// Reference: cornstarch/kernel/bitfield_attention.py:60-156.
+#include "bam_common.h"
+#include "bam_launch.h"
+
+namespace bam {
+
+// One workgroup = one 128-row block x FLAG_COLS_PER_BLOCK key tiles.  Each wave takes one
+// 128x32 tile at a time: lane l owns key column (l & 31) and the 64 query rows of half
+// (l >> 5); the per-lane counts are summed over the wave.
+constexpr int FLAG_WAVES = 4;
+constexpr int FLAG_TILES_PER_WAVE = 8;
+constexpr int FLAG_COLS_PER_BLOCK = FLAG_WAVES * FLAG_TILES_PER_WAVE;
+
+__global__ __launch_bounds__(FLAG_WAVES * 64) void tile_flags_kernel(const int64_t* __restrict__ bf,
+                                                                    int64_t bf_stride_b,
+                                                                    int8_t* __restrict__ flags,
+                                                                    int64_t flags_stride_b,
+                                                                    int64_t flags_stride_m, int S, int num_n) {
+    __shared__ int64_t q_bits[BLOCK_M];
+    const int b = blockIdx.z, m = blockIdx.y;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int64_t* row = bf + (int64_t)b * bf_stride_b;
+    if (tid < BLOCK_M) {
+        const int i = m * BLOCK_M + tid;
+        q_bits[tid] = (i < S) ? row[i] : 0;  // out-of-range positions read 0 (reference :86-87)
+    }
+    __syncthreads();
+    const int rows_in_range = min(BLOCK_M, S - m * BLOCK_M);
+    const int half = lane >> 5;
+    for (int t = 0; t < FLAG_TILES_PER_WAVE; ++t) {
+        const int n = blockIdx.x * FLAG_COLS_PER_BLOCK + wave * FLAG_TILES_PER_WAVE + t;
+        if (n >= num_n) break;  // wave-uniform
+        const int j = n * BLOCK_N + (lane & 31);
+        const int64_t kf = (j < S) ? row[j] : 0;
+        int cnt = 0;
+#pragma unroll 8
+        for (int r = 0; r < 64; ++r) {
+            const int ri = half * 64 + r;
+            cnt += allow_rule(q_bits[ri], kf, (int64_t)m * BLOCK_M + ri, j) ? 1 : 0;
+        }
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) cnt += __shfl_xor(cnt, off);
+        if (lane == 0) {
+            const int cols_in_range = min(BLOCK_N, S - n * BLOCK_N);
+            int8_t f = 0;
+            if (cnt > 0) f = 1;
+            if (cnt == rows_in_range * cols_in_range) f = 2;  // full over in-range cells (:149-153)
+            flags[(int64_t)b * flags_stride_b + (int64_t)m * flags_stride_m + n] = f;
+        }
+    }
+}
+
+__global__ __launch_bounds__(256) void materialize_mask_kernel(const int64_t* __restrict__ bf,
+                                                               int64_t bf_stride_b,
+                                                               uint8_t* __restrict__ out, int S) {
+    const int b = blockIdx.z, i = blockIdx.y;
+    const int64_t* row = bf + (int64_t)b * bf_stride_b;
+    const int64_t qf = row[i];
+    for (int j = blockIdx.x * blockDim.x + threadIdx.x; j < S; j += gridDim.x * blockDim.x)
+        out[((int64_t)b * S + i) * S + j] = allow_rule(qf, row[j], i, j) ? 1 : 0;
+}
+
+int launch_tile_flags(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int64_t flags_stride_b,
+                      int64_t flags_stride_m, int B, int S, hipStream_t stream) {
+    const int num_m = (S + BLOCK_M - 1) / BLOCK_M, num_n = (S + BLOCK_N - 1) / BLOCK_N;
+    dim3 grid((num_n + FLAG_COLS_PER_BLOCK - 1) / FLAG_COLS_PER_BLOCK, num_m, B);
+    hipLaunchKernelGGL(tile_flags_kernel, grid, dim3(FLAG_WAVES * 64), 0, stream, bf, bf_stride_b, flags,
+                       flags_stride_b, flags_stride_m, S, num_n);
+    return (int)hipGetLastError();
+}
+
+int launch_materialize_mask(const int64_t* bf, int64_t bf_stride_b, uint8_t* out, int B, int S,
+                            hipStream_t stream) {
+    dim3 grid(min((S + 255) / 256, 64), S, B);
+    hipLaunchKernelGGL(materialize_mask_kernel, grid, dim3(256), 0, stream, bf, bf_stride_b, out, S);
+    return (int)hipGetLastError();
+}
+
+}  // namespace bam

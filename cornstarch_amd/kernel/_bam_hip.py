@@ -1,0 +1,69 @@
+"""ctypes binding of ``libbam_hip.so`` (declarations: ``include/bam_hip.h``).
+
+There is no fallback: if the library is missing or a call fails, an exception is raised.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+
+_PKG_DIR = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+LIB_PATH = os.path.join(_PKG_DIR, "libbam_hip.so")
+
+BAM_DTYPE_F16 = 0
+BAM_DTYPE_BF16 = 1
+BAM_MAX_SEQLEN = 131072
+ABI_VERSION = 1
+
+_i64 = ctypes.c_int64
+_int = ctypes.c_int
+_ptr = ctypes.c_void_p
+_f32 = ctypes.c_float
+
+# name -> argtypes, exactly the prototypes of include/bam_hip.h
+SIGNATURES = {
+    "bam_tile_flags": [_ptr, _i64, _ptr, _i64, _i64, _int, _int, _ptr],
+    "bam_materialize_mask": [_ptr, _i64, _ptr, _int, _int, _ptr],
+    "bam_fwd": [_ptr] * 7 + [_i64] * 15 + [_int] * 5 + [_f32, _int, _ptr],
+    "bam_bwd_preprocess": [_ptr] * 3 + [_i64] * 6 + [_int] * 5 + [_ptr],
+    "bam_bwd": [_ptr] * 11 + [_i64] * 24 + [_int] * 5 + [_f32, _int, _ptr],
+}
+
+_lib = None
+
+
+class BamError(RuntimeError):
+    pass
+
+
+def load() -> ctypes.CDLL:
+    """Load the HIP library (once).  Raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise BamError(
+            f"{LIB_PATH} is missing: the HIP kernels have not been built "
+            "(run `python -m cornstarch_amd.build`); there is no fallback path"
+        )
+    lib = ctypes.CDLL(LIB_PATH)
+    lib.bam_last_error.restype = ctypes.c_char_p
+    lib.bam_last_error.argtypes = []
+    lib.bam_abi_version.restype = _int
+    lib.bam_abi_version.argtypes = []
+    for name, argtypes in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.argtypes = argtypes
+        fn.restype = _int
+    if lib.bam_abi_version() != ABI_VERSION:
+        raise BamError(f"libbam_hip.so has ABI {lib.bam_abi_version()}, this binding expects {ABI_VERSION}")
+    _lib = lib
+    return lib
+
+
+def call(name: str, *args) -> None:
+    lib = load()
+    rc = getattr(lib, name)(*args)
+    if rc != 0:
+        raise BamError(f"{name} failed ({rc}): {lib.bam_last_error().decode()}")

@@ -1,0 +1,313 @@
+"""Bitfield-masked attention on MI355X: host side of the reference's
+``cornstarch/kernel/bitfield_attention.py`` with the same names, argument order and
+defaults, backed by hand-written gfx950 HIP kernels reached through ``libbam_hip.so``.
+
+Every token carries an int64 bitfield; the attention mask is derived from those bitfields
+inside the kernels (text tokens: causal over tokens sharing a bit; modality tokens:
+bidirectional inside their own modality).  There is no PyTorch/CPU fallback: tensors must
+live on the GPU and the HIP library must be built.
+"""
+
+from __future__ import annotations
+
+import math
+from typing import Optional
+
+import torch
+import torch.nn.functional as F
+
+from . import _bam_hip
+
+BLOCK_M = 128  # rows of a flag tile (reference bitfield_attention.py:53)
+BLOCK_N = 32  # columns of a flag tile (reference bitfield_attention.py:54)
+NUM_TOKENS_TO_COMPUTE_PER_BLOCK = 4096  # kept for importers; the HIP forward is single pass
+NUM_KV_BLOCKS_PER_BLOCK = NUM_TOKENS_TO_COMPUTE_PER_BLOCK // BLOCK_N
+
+_SUPPORTED_HEAD_DIMS = (32, 64, 128)
+
+
+def _stream_ptr(device: torch.device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def _dtype_code(dtype: torch.dtype) -> int:
+    return _bam_hip.BAM_DTYPE_BF16 if dtype == torch.bfloat16 else _bam_hip.BAM_DTYPE_F16
+
+
+def _kernel_ready(x: torch.Tensor, elems_per_16b: int) -> torch.Tensor:
+    """Kernels read 16 bytes at a time: unit last stride, 16-byte aligned rows."""
+    ok = (
+        x.stride(-1) == 1
+        and x.data_ptr() % 16 == 0
+        and all(s % elems_per_16b == 0 for s in x.stride()[:-1])
+    )
+    return x if ok else x.contiguous()
+
+
+def _padded_head_dim(d: int) -> int:
+    for cand in _SUPPORTED_HEAD_DIMS:
+        if d <= cand:
+            return cand
+    raise AssertionError("FlashAttention only support head dimensions up to 128")
+
+
+def materialize_bitfield_mask(bitfield_mask: torch.Tensor) -> torch.Tensor:
+    """bool (B, S, S): the allow rule for every (query, key) pair, evaluated on the GPU.
+
+    Host-callable counterpart of the reference's Triton device function
+    ``_materialize_bitfield_mask_block`` (bitfield_attention.py:60-101), which its test
+    wraps in a kernel (tests/test_kernel/test_bitfield_attention.py:16-52)."""
+    assert bitfield_mask.is_cuda and bitfield_mask.dtype == torch.int64 and bitfield_mask.dim() == 2
+    if bitfield_mask.stride(1) != 1:
+        bitfield_mask = bitfield_mask.contiguous()
+    B, S = bitfield_mask.shape
+    out = torch.empty((B, S, S), dtype=torch.uint8, device=bitfield_mask.device)
+    with torch.cuda.device(bitfield_mask.device):
+        _bam_hip.call(
+            "bam_materialize_mask", bitfield_mask.data_ptr(), bitfield_mask.stride(0), out.data_ptr(), B, S,
+            _stream_ptr(bitfield_mask.device),
+        )
+    return out.bool()
+
+
+class BitfieldUtils:
+    """Cache of the tile flags ("compressed mask") of the current bitfield mask.
+
+    compressed_mask_cache: int8 (batch, ceil(S / BLOCK_M), ceil(S / BLOCK_N));
+        0: every pair of the tile is masked, the tile is skipped
+        1: some pairs are allowed, the mask is evaluated
+        2: every in-range pair is allowed, the mask is not evaluated
+    Same API as the reference (bitfield_attention.py:159-212).  The reference returns
+    whatever the cache holds until ``clear_cache()``; here the cache is also keyed on the
+    identity of the bitfield tensor, so a different mask can never pick up stale flags.
+    """
+
+    compressed_mask_cache: Optional[torch.Tensor] = None
+    _cache_key = None
+
+    @classmethod
+    def clear_cache(cls):
+        cls.compressed_mask_cache = None
+        cls._cache_key = None
+
+    @classmethod
+    def materialize_compressed_mask_from_bitfield_mask(cls, bitfield_mask: torch.Tensor) -> torch.Tensor:
+        key = (
+            bitfield_mask.data_ptr(),
+            tuple(bitfield_mask.shape),
+            tuple(bitfield_mask.stride()),
+            bitfield_mask._version,
+            bitfield_mask.device,
+        )
+        if cls.compressed_mask_cache is not None and cls._cache_key == key:
+            return cls.compressed_mask_cache
+
+        assert bitfield_mask.is_cuda, "bitfield attention runs on the GPU only"
+        assert bitfield_mask.dtype == torch.int64 and bitfield_mask.dim() == 2
+        bf = bitfield_mask if bitfield_mask.stride(1) == 1 else bitfield_mask.contiguous()
+        batch_size, seq_len = bf.shape
+        out = torch.empty(
+            (batch_size, -(-seq_len // BLOCK_M), -(-seq_len // BLOCK_N)),
+            dtype=torch.int8,
+            device=bf.device,
+        )
+        with torch.cuda.device(bf.device):
+            _bam_hip.call(
+                "bam_tile_flags", bf.data_ptr(), bf.stride(0), out.data_ptr(), out.stride(0), out.stride(1),
+                batch_size, seq_len, _stream_ptr(bf.device),
+            )
+        cls.compressed_mask_cache = out
+        cls._cache_key = key
+        return out
+
+
+def _check_unsupported(offsets_q, offsets_k, bias):
+    if offsets_q is not None or offsets_k is not None:
+        raise NotImplementedError("offsets_q / offsets_k (context-parallel index tensors) are not implemented yet")
+    if bias is not None:
+        raise NotImplementedError("attention bias is not implemented (no caller of the reference passes one)")
+
+
+def _bitfield_attn_forward(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    bitfield_mask: torch.Tensor,
+    compressed_mask: torch.Tensor,
+    offsets_q: Optional[torch.Tensor] = None,
+    offsets_k: Optional[torch.Tensor] = None,
+    bias: Optional[torch.Tensor] = None,
+    softmax_scale: Optional[float] = None,
+):
+    """q (B, S, Hq, D), k/v (B, S, Hkv, D) -> (o like q, lse fp32 (B, Hq, ceil(S/128)*128),
+    softmax_scale).  Contract of the reference's ``_bitfield_attn_forward``
+    (bitfield_attention.py:932-1069)."""
+    batch, seqlen_q, nheads, d = q.shape
+    _, seqlen_k, nheads_k, _ = k.shape
+    assert d <= 128, "FlashAttention only support head dimensions up to 128"
+    assert q.dtype == k.dtype == v.dtype, "All tensors must have the same type"
+    assert q.dtype in [torch.float16, torch.bfloat16], "Only support fp16 and bf16"
+    assert q.is_cuda and k.is_cuda and v.is_cuda
+    assert seqlen_q == seqlen_k, "self-attention only: query and key sequence lengths must match"
+    assert k.shape == v.shape and k.shape[0] == batch and k.shape[3] == d
+    assert nheads % nheads_k == 0
+    assert bitfield_mask.dtype == torch.int64 and bitfield_mask.shape == (batch, seqlen_k)
+    _check_unsupported(offsets_q, offsets_k, bias)
+    softmax_scale = softmax_scale or 1.0 / math.sqrt(d)
+
+    dp = _padded_head_dim(d)
+    if dp != d:  # zero columns change neither q.k nor the first d columns of p.v
+        q, k, v = (F.pad(x, (0, dp - d)) for x in (q, k, v))
+    qk, kk, vk = (_kernel_ready(x, 8) for x in (q, k, v))
+    bf = bitfield_mask if bitfield_mask.stride(1) == 1 else bitfield_mask.contiguous()
+    flags = compressed_mask if compressed_mask.stride(-1) == 1 else compressed_mask.contiguous()
+    num_m, num_n = -(-seqlen_q // BLOCK_M), -(-seqlen_k // BLOCK_N)
+    assert flags.dtype == torch.int8 and flags.shape == (batch, num_m, num_n)
+
+    seqlen_q_rounded = num_m * BLOCK_M
+    lse = torch.empty((batch, nheads, seqlen_q_rounded), device=q.device, dtype=torch.float32)
+    o = torch.empty_like(qk)
+    with torch.cuda.device(q.device):
+        _bam_hip.call(
+            "bam_fwd",
+            qk.data_ptr(), kk.data_ptr(), vk.data_ptr(), o.data_ptr(), lse.data_ptr(), bf.data_ptr(), flags.data_ptr(),
+            qk.stride(0), qk.stride(1), qk.stride(2),
+            kk.stride(0), kk.stride(1), kk.stride(2),
+            vk.stride(0), vk.stride(1), vk.stride(2),
+            o.stride(0), o.stride(1), o.stride(2),
+            bf.stride(0), flags.stride(0), flags.stride(1),
+            batch, seqlen_q, nheads, nheads_k, dp, float(softmax_scale), _dtype_code(q.dtype),
+            _stream_ptr(q.device),
+        )
+    if dp != d:
+        o = o[..., :d].contiguous()
+    return o, lse, softmax_scale
+
+
+def _bitfield_attn_backward(
+    do: torch.Tensor,
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    o: torch.Tensor,
+    bitfield_mask: torch.Tensor,
+    compressed_mask: torch.Tensor,
+    lse: torch.Tensor,
+    dq: torch.Tensor,
+    dk: torch.Tensor,
+    dv: torch.Tensor,
+    offsets_q: Optional[torch.Tensor] = None,
+    offsets_k: Optional[torch.Tensor] = None,
+    bias: Optional[torch.Tensor] = None,
+    softmax_scale: Optional[float] = None,
+):
+    """Accumulates the gradients into the caller's fp32 ``dq``, ``dk``, ``dv``.  Contract of
+    the reference's ``_bitfield_attn_backward`` (bitfield_attention.py:1073-1199)."""
+    if do.stride(-1) != 1:
+        do = do.contiguous()
+    batch, seqlen_q, nheads, d = q.shape
+    _, seqlen_k, nheads_k, _ = k.shape
+    assert d <= 128
+    seqlen_q_rounded = math.ceil(seqlen_q / BLOCK_M) * BLOCK_M
+    assert lse.shape == (batch, nheads, seqlen_q_rounded)
+    assert q.stride(-1) == k.stride(-1) == v.stride(-1) == o.stride(-1) == 1
+    assert dq.stride(-1) == dk.stride(-1) == dv.stride(-1) == 1
+    assert dq.dtype == dk.dtype == dv.dtype == torch.float32
+    assert q.is_cuda and seqlen_q == seqlen_k
+    _check_unsupported(offsets_q, offsets_k, bias)
+    softmax_scale = softmax_scale or 1.0 / math.sqrt(d)
+
+    dp = _padded_head_dim(d)
+    acc = (dq, dk, dv)
+    if dp != d:
+        q, k, v, o, do = (F.pad(x, (0, dp - d)) for x in (q, k, v, o, do))
+        acc = tuple(torch.zeros(x.shape[:-1] + (dp,), dtype=torch.float32, device=x.device) for x in (dq, dk, dv))
+    qk, kk, vk, ok, gk = (_kernel_ready(x, 8) for x in (q, k, v, o, do))
+    work = tuple(_kernel_ready(x, 4) for x in acc)
+    lse = lse.contiguous()
+    bf = bitfield_mask if bitfield_mask.stride(1) == 1 else bitfield_mask.contiguous()
+    flags = compressed_mask if compressed_mask.stride(-1) == 1 else compressed_mask.contiguous()
+    delta = torch.empty_like(lse)
+    code = _dtype_code(q.dtype)
+    stream = _stream_ptr(q.device)
+    with torch.cuda.device(q.device):
+        _bam_hip.call(
+            "bam_bwd_preprocess",
+            ok.data_ptr(), gk.data_ptr(), delta.data_ptr(),
+            ok.stride(0), ok.stride(1), ok.stride(2),
+            gk.stride(0), gk.stride(1), gk.stride(2),
+            batch, seqlen_q, nheads, dp, code, stream,
+        )
+        wq, wk, wv = work
+        _bam_hip.call(
+            "bam_bwd",
+            qk.data_ptr(), kk.data_ptr(), vk.data_ptr(), gk.data_ptr(), lse.data_ptr(), delta.data_ptr(),
+            wq.data_ptr(), wk.data_ptr(), wv.data_ptr(), bf.data_ptr(), flags.data_ptr(),
+            qk.stride(0), qk.stride(1), qk.stride(2),
+            kk.stride(0), kk.stride(1), kk.stride(2),
+            vk.stride(0), vk.stride(1), vk.stride(2),
+            gk.stride(0), gk.stride(1), gk.stride(2),
+            wq.stride(0), wq.stride(1), wq.stride(2),
+            wk.stride(0), wk.stride(1), wk.stride(2),
+            wv.stride(0), wv.stride(1), wv.stride(2),
+            bf.stride(0), flags.stride(0), flags.stride(1),
+            batch, seqlen_q, nheads, nheads_k, dp, float(softmax_scale), code, stream,
+        )
+    # the kernels accumulated into `work`; hand the sums back if those were copies
+    for dst, mid, w in zip((dq, dk, dv), acc, work):
+        if dp != d:
+            dst += w[..., :d]
+        elif w is not mid:
+            dst.copy_(w)
+
+
+class BitfieldAttentionFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(
+        ctx,
+        q: torch.Tensor,
+        k: torch.Tensor,
+        v: torch.Tensor,
+        bitfield_mask: torch.Tensor,
+        bias: Optional[torch.Tensor] = None,
+        softmax_scale: Optional[float] = None,
+    ):
+        """
+        q: (batch_size, seqlen_q, nheads, headdim)
+        k, v: (batch_size, seqlen_k, nheads_k, headdim)
+        bitfield_mask: (batch_size, seqlen) int64
+        """
+        q, k, v = [x if x.stride(-1) == 1 else x.contiguous() for x in [q, k, v]]
+
+        compressed_mask = BitfieldUtils.materialize_compressed_mask_from_bitfield_mask(bitfield_mask)
+
+        o, lse, ctx.softmax_scale = _bitfield_attn_forward(
+            q, k, v, bitfield_mask, compressed_mask, bias=bias, softmax_scale=softmax_scale
+        )
+        ctx.save_for_backward(q, k, v, o, lse, bias, bitfield_mask, compressed_mask)
+        return o
+
+    @staticmethod
+    def backward(ctx, do: torch.Tensor):
+        q, k, v, o, lse, bias, bitfield_mask, compressed_mask = ctx.saved_tensors
+        assert not ctx.needs_input_grad[3], "the bitfield mask is not differentiable"
+        with torch.no_grad():
+            dq = torch.zeros_like(q, dtype=torch.float32)
+            dk = torch.zeros_like(k, dtype=torch.float32)
+            dv = torch.zeros_like(v, dtype=torch.float32)
+            _bitfield_attn_backward(
+                do, q, k, v, o, bitfield_mask, compressed_mask, lse, dq, dk, dv,
+                bias=bias, softmax_scale=ctx.softmax_scale,
+            )
+        return dq.to(dtype=q.dtype), dk.to(dtype=k.dtype), dv.to(dtype=v.dtype), None, None, None
+
+
+def bitfield_attn_func(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    bitfield_mask: torch.Tensor,
+    bias: Optional[torch.Tensor] = None,
+    softmax_scale: Optional[float] = None,
+) -> torch.Tensor:
+    return BitfieldAttentionFunction.apply(q, k, v, bitfield_mask, bias, softmax_scale)

@@ -1,0 +1,104 @@
+/*
+ * C ABI of libbam_hip.so: bitfield-masked attention for AMD MI355X (gfx950).
+ *
+ * Every entry point replaces one Triton launch site of the reference file
+ * cornstarch/kernel/bitfield_attention.py (cited per function).  Conventions:
+ *   - all pointers are DEVICE pointers owned by the caller; nothing is allocated or freed;
+ *   - work is enqueued on `stream` (a hipStream_t passed as void*); no call synchronizes;
+ *   - q/k/v/o/do/dq/dk/dv are logically (B, S, H, D) with element strides for b, s, h and
+ *     unit stride along D; 16-bit tensors need 16-byte aligned rows (pointer % 16 == 0,
+ *     strides % 8 == 0), fp32 gradient buffers need pointer % 16 == 0, strides % 4 == 0;
+ *   - D is 32, 64 or 128; Hq % Hkv == 0; kv head of q head h is h / (Hq / Hkv);
+ *   - dtype: BAM_DTYPE_F16 or BAM_DTYPE_BF16;
+ *   - flags: int8 (B, ceil(S/128), ceil(S/32)), unit stride along the last axis,
+ *     0 = empty, 1 = partial, 2 = every in-range pair allowed;
+ *   - lse / delta: fp32 (B, Hq, S_rounded), S_rounded = ceil(S/128)*128, contiguous;
+ *   - return value: BAM_OK or a negative BAM_ERR_* code; bam_last_error() gives the text
+ *     of the calling thread's last failure.
+ */
+#ifndef BAM_HIP_H
+#define BAM_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define BAM_OK 0
+#define BAM_ERR_INVALID_ARGUMENT (-1) /* shape / stride / alignment / dtype violation */
+#define BAM_ERR_UNSUPPORTED (-2)      /* valid request this build does not implement */
+#define BAM_ERR_LAUNCH (-3)           /* the HIP runtime refused the launch */
+
+#define BAM_DTYPE_F16 0
+#define BAM_DTYPE_BF16 1
+
+/* Upper bound on S accepted by the attention kernels (tile lists live in LDS). */
+#define BAM_MAX_SEQLEN 131072
+
+const char* bam_last_error(void);
+
+/* ABI version of this library (bumped on any signature change). */
+int bam_abi_version(void);
+
+/*
+ * Tile flags ("compressed mask").  Replaces the `_materialize_compressed_mask[shape](...)`
+ * launch in BitfieldUtils.materialize_compressed_mask_from_bitfield_mask
+ * (bitfield_attention.py:105-156, 176-212).
+ *   bf: int64 (B, S), row stride bf_stride_b, unit column stride.
+ *   flags: int8, strides flags_stride_b / flags_stride_m, unit stride along key tiles.
+ */
+int bam_tile_flags(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int64_t flags_stride_b,
+                   int64_t flags_stride_m, int B, int S, void* stream);
+
+/*
+ * Dense bool mask, uint8 (B, S, S) contiguous: the allow rule for every pair
+ * (device function `_materialize_bitfield_mask_block`, bitfield_attention.py:60-101,
+ * which the reference's test wraps in a kernel of its own,
+ * tests/test_kernel/test_bitfield_attention.py:16-52).  Test/diagnostic utility.
+ */
+int bam_materialize_mask(const int64_t* bf, int64_t bf_stride_b, uint8_t* out, int B, int S, void* stream);
+
+/*
+ * Forward.  Replaces `_fwd_kernel[grid]` + `_aggregate_partial_outputs[grid]` in
+ * `_bitfield_attn_forward` (bitfield_attention.py:236-523, 932-1069, 1292-1436):
+ *   o = softmax_allowed(scale * q k^T) v,  lse = log sum_allowed exp(scale * q k^T);
+ *   rows that allow no key give o = 0, lse = -inf.
+ * o has q's dtype.  scale must be > 0.
+ */
+int bam_fwd(const void* q, const void* k, const void* v, void* o, float* lse, const int64_t* bf,
+            const int8_t* flags, int64_t q_stride_b, int64_t q_stride_s, int64_t q_stride_h,
+            int64_t k_stride_b, int64_t k_stride_s, int64_t k_stride_h, int64_t v_stride_b,
+            int64_t v_stride_s, int64_t v_stride_h, int64_t o_stride_b, int64_t o_stride_s,
+            int64_t o_stride_h, int64_t bf_stride_b, int64_t flags_stride_b, int64_t flags_stride_m, int B,
+            int S, int Hq, int Hkv, int D, float scale, int dtype, void* stream);
+
+/*
+ * delta[b,h,i] = sum_d o[b,i,h,d] * do[b,i,h,d] in fp32.  Replaces
+ * `_bwd_preprocess_do_o_dot[grid]` (bitfield_attention.py:527-572, 1105-1122).
+ */
+int bam_bwd_preprocess(const void* o, const void* dout, float* delta, int64_t o_stride_b, int64_t o_stride_s,
+                       int64_t o_stride_h, int64_t do_stride_b, int64_t do_stride_s, int64_t do_stride_h,
+                       int B, int S, int Hq, int D, int dtype, void* stream);
+
+/*
+ * Backward.  Replaces `_bwd_kernel[grid]` (bitfield_attention.py:598-929, 1145-1199).
+ * dq, dk, dv are fp32 and are ACCUMULATED INTO (the caller zeroes them,
+ * bitfield_attention.py:1248-1250); dk/dv receive the sum over the q heads of a group.
+ * No atomics are used: each output element is owned by exactly one workgroup, so the
+ * result is deterministic.
+ */
+int bam_bwd(const void* q, const void* k, const void* v, const void* dout, const float* lse,
+            const float* delta, float* dq, float* dk, float* dv, const int64_t* bf, const int8_t* flags,
+            int64_t q_stride_b, int64_t q_stride_s, int64_t q_stride_h, int64_t k_stride_b,
+            int64_t k_stride_s, int64_t k_stride_h, int64_t v_stride_b, int64_t v_stride_s,
+            int64_t v_stride_h, int64_t do_stride_b, int64_t do_stride_s, int64_t do_stride_h,
+            int64_t dq_stride_b, int64_t dq_stride_s, int64_t dq_stride_h, int64_t dk_stride_b,
+            int64_t dk_stride_s, int64_t dk_stride_h, int64_t dv_stride_b, int64_t dv_stride_s,
+            int64_t dv_stride_h, int64_t bf_stride_b, int64_t flags_stride_b, int64_t flags_stride_m, int B,
+            int S, int Hq, int Hkv, int D, float scale, int dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BAM_HIP_H */

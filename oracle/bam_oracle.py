@@ -1,0 +1,229 @@
+"""CPU oracle for bitfield-masked attention (BAM).  TEST INFRASTRUCTURE ONLY.
+
+This module is a restatement, in plain torch tensor ops, of the algorithm of the
+reference hot path ``cornstarch/kernel/bitfield_attention.py``.  It is the checker
+the parity tests, the smoke test and the CPU-baseline leg of the benchmark compare
+the HIP kernels against.  Nothing in the shipped package imports it, and the
+shipped package never falls back to it.
+
+What pins each function (the pins live in ``tests/test_oracle.py``):
+
+* ``allow_rows`` / ``materialize_mask`` -- the closed-form masks held by the
+  reference's own test (``tests/test_kernel/test_bitfield_attention.py:55-110``:
+  lower-triangular with modality rows replaced by same-segment squares), plus the
+  degenerate cases all-text == causal and all-one-modality == dense.
+* ``tile_flags`` -- its definition over the pinned mask
+  (``bitfield_attention.py:118-126,143-153``), the analytic tile histogram of the
+  1024-token plumbing layout (124 full / 24 partial / 108 empty, 557440 pairs) and
+  the per-row-block non-empty counts the reference's context-parallel test expects
+  (``tests/test_shardformer/test_context_parallel.py:30-63,258-272``).
+* ``attention_sdpa`` -- is the library routine the reference's tests use as ground
+  truth (``tests/test_kernel/test_bitfield_attention.py:188-190,287-293``).
+* ``attention_forward`` (explicit softmax, also yields LSE) -- pinned against
+  ``attention_sdpa`` and against ``torch.logsumexp``.
+* ``attention_backward`` -- ``torch.autograd.grad`` through the explicit forward,
+  pinned against autograd through SDPA (``test_bitfield_attention.py:198-204``)
+  and against the closed-form C restatement in ``bam_oracle.c``.
+* ``create_bitfield_attention_mask`` -- golden vectors of
+  ``tests/test_models/test_multimodal_merge_outputs.py:94-110``.
+
+All functions are device agnostic torch code: the parity tests run them on the CPU
+at small sizes and, for the full-size configurations, on whatever device the
+inputs live on (fp32 library math, never the HIP kernels).
+"""
+
+from __future__ import annotations
+
+import math
+from typing import Optional
+
+import torch
+import torch.nn.functional as F
+
+BLOCK_M = 128  # bitfield_attention.py:53
+BLOCK_N = 32  # bitfield_attention.py:54
+MODALITY_MASK = (1 << 62) - 1  # bitfield_attention.py:92-93
+
+
+# --------------------------------------------------------------------------- mask
+def _gather_bits(bf_row: torch.Tensor, pos: torch.Tensor) -> torch.Tensor:
+    """bitfield at global positions ``pos``; positions >= S read 0
+    (bitfield_attention.py:86-87)."""
+    S = bf_row.shape[0]
+    ok = pos < S
+    return torch.where(ok, bf_row[pos.clamp(max=S - 1)], torch.zeros_like(pos))
+
+
+def allow_rows(
+    bf_row: torch.Tensor,
+    r0: int,
+    r1: int,
+    idx_q: Optional[torch.Tensor] = None,
+    idx_k: Optional[torch.Tensor] = None,
+) -> torch.Tensor:
+    """Allow rule for query rows [r0, r1) of ONE sequence -> bool (r1-r0, Sk).
+
+    ``bf_row``: int64 (S_total,).  Without index tensors the query/key positions
+    are the row/column numbers; with them they are ``idx_q[row]`` / ``idx_k[col]``
+    (global positions, bitfield_attention.py:71-81).
+    Rule (bitfield_attention.py:86-101), M = 2**62 - 1:
+        allow(i, j) = (i >= j and text_i and (q & k & M) != 0)
+                   or (not text_i and (q & M) == (k & M) and (q & M) != 0)
+    """
+    S = bf_row.shape[0]
+    dev = bf_row.device
+    if idx_q is None:
+        pos_q = torch.arange(r0, r1, device=dev, dtype=torch.int64)
+    else:
+        pos_q = idx_q[r0:r1].to(torch.int64)
+    if idx_k is None:
+        pos_k = torch.arange(0, S, device=dev, dtype=torch.int64)
+    else:
+        pos_k = idx_k.to(torch.int64)
+    qf = _gather_bits(bf_row, pos_q)
+    kf = _gather_bits(bf_row, pos_k)
+    text = (qf & 1) != 0
+    qb = (qf & MODALITY_MASK)[:, None]
+    kb = (kf & MODALITY_MASK)[None, :]
+    causal = pos_q[:, None] >= pos_k[None, :]
+    return (causal & text[:, None] & ((qb & kb) != 0)) | (
+        (~text)[:, None] & (qb == kb) & (qb != 0)
+    )
+
+
+def materialize_mask(bitfield: torch.Tensor) -> torch.Tensor:
+    """bool (B, S, S) attention mask of a (B, S) int64 bitfield tensor."""
+    B, S = bitfield.shape
+    return torch.stack([allow_rows(bitfield[b], 0, S) for b in range(B)])
+
+
+def tile_flags(bitfield: torch.Tensor) -> torch.Tensor:
+    """int8 (B, ceil(S/128), ceil(S/32)): 0 empty, 1 partial, 2 full.
+
+    A tile is full when every IN-RANGE cell is allowed; the ragged last row/column
+    tile counts ``S % 128`` rows / ``S % 32`` columns
+    (bitfield_attention.py:143-153).
+    """
+    B, S = bitfield.shape
+    nm, nn = -(-S // BLOCK_M), -(-S // BLOCK_N)
+    out = torch.zeros((B, nm, nn), dtype=torch.int8, device=bitfield.device)
+    cols = torch.full((nn,), BLOCK_N, dtype=torch.int64, device=bitfield.device)
+    if S % BLOCK_N:
+        cols[-1] = S % BLOCK_N
+    for b in range(B):
+        for m in range(nm):
+            r0, r1 = m * BLOCK_M, min((m + 1) * BLOCK_M, S)
+            a = allow_rows(bitfield[b], r0, r1)  # (rows, S)
+            a = F.pad(a, (0, nn * BLOCK_N - S))
+            cnt = a.view(r1 - r0, nn, BLOCK_N).sum(dim=(0, 2))
+            full = cnt == (r1 - r0) * cols
+            out[b, m] = torch.where(cnt == 0, 0, torch.where(full, 2, 1)).to(torch.int8)
+    return out
+
+
+def unmasked_pairs(bitfield: torch.Tensor) -> int:
+    """Number of allowed (query, key) pairs over the whole batch."""
+    B, S = bitfield.shape
+    total = 0
+    step = 2048
+    for b in range(B):
+        for r0 in range(0, S, step):
+            total += int(allow_rows(bitfield[b], r0, min(r0 + step, S)).sum())
+    return total
+
+
+def create_bitfield_attention_mask(input_ids: torch.Tensor, token_ids: dict) -> torch.Tensor:
+    """Bitfield format (cornstarch/kernel/interface.py:13-30): modality number n in
+    ``token_ids`` order gets bit n+1; text gets bit 62, bit 0 and every modality bit."""
+    text = (1 << 62) | 1
+    bits = {}
+    for n, key in enumerate(token_ids):
+        bits[key] = 1 << (n + 1)
+        text |= bits[key]
+    out = torch.full(input_ids.shape, text, dtype=torch.int64, device=input_ids.device)
+    for key, tok in token_ids.items():
+        out = torch.where(input_ids == tok, torch.full_like(out, bits[key]), out)
+    return out
+
+
+# ---------------------------------------------------------------------- attention
+def attention_sdpa(q, k, v, bitfield, softmax_scale=None):
+    """Materialized-mask attention exactly as the reference's tests build their
+    ground truth (test_bitfield_attention.py:188-190,287-293): library SDPA with the
+    bool mask, GQA by ``enable_gqa``.  q (B,S,Hq,D), k/v (B,S,Hkv,D) -> (B,S,Hq,D).
+    Rows that allow no key come out as NaN from the library; the reference kernel
+    defines them as 0 (bitfield_attention.py:441-444,493-495), so they are zeroed."""
+    mask = materialize_mask(bitfield).unsqueeze(1)
+    o = F.scaled_dot_product_attention(
+        q.transpose(1, 2),
+        k.transpose(1, 2),
+        v.transpose(1, 2),
+        attn_mask=mask,
+        scale=softmax_scale,
+        enable_gqa=q.shape[2] != k.shape[2],
+    ).transpose(1, 2)
+    dead = ~mask.any(dim=-1)  # (B,1,S)
+    return torch.where(dead.transpose(1, 2).unsqueeze(-1), torch.zeros_like(o), o)
+
+
+def _chunk_forward(qc, kb, vb, allow, scale):
+    """qc (rows,Hq,D), kb/vb (S,Hkv,D), allow (rows,S) -> o (rows,Hq,D), lse (Hq,rows).
+    s = scale * q.k ; lse = log sum_allowed exp(s) ; o = sum_allowed exp(s-lse) v
+    (bitfield_attention.py:389-390,435-495); GQA h -> h // (Hq//Hkv) (:292-293)."""
+    Hq, Hkv = qc.shape[1], kb.shape[1]
+    g = Hq // Hkv
+    kk = kb.repeat_interleave(g, dim=1) if g > 1 else kb
+    vv = vb.repeat_interleave(g, dim=1) if g > 1 else vb
+    s = torch.einsum("ihd,jhd->hij", qc, kk) * scale
+    s = s.masked_fill(~allow[None], float("-inf"))
+    lse = torch.logsumexp(s, dim=-1)  # -inf where nothing is allowed
+    p = torch.exp(s - torch.where(torch.isinf(lse), torch.zeros_like(lse), lse)[..., None])
+    o = torch.einsum("hij,jhd->ihd", p, vv)
+    return o, lse
+
+
+def attention_forward(q, k, v, bitfield, softmax_scale=None, row_chunk=1024, dtype=torch.float32):
+    """Explicit masked softmax attention -> (o (B,S,Hq,D), lse (B,Hq,S)) in ``dtype``."""
+    B, S, Hq, D = q.shape
+    scale = softmax_scale or 1.0 / math.sqrt(D)
+    q, k, v = q.to(dtype), k.to(dtype), v.to(dtype)
+    o = torch.empty((B, S, Hq, D), dtype=dtype, device=q.device)
+    lse = torch.empty((B, Hq, S), dtype=dtype, device=q.device)
+    for b in range(B):
+        for r0 in range(0, S, row_chunk):
+            r1 = min(r0 + row_chunk, S)
+            allow = allow_rows(bitfield[b], r0, r1)
+            oc, lc = _chunk_forward(q[b, r0:r1], k[b], v[b], allow, scale)
+            o[b, r0:r1] = oc
+            lse[b, :, r0:r1] = lc
+    return o, lse
+
+
+def attention_backward(q, k, v, bitfield, do, softmax_scale=None, row_chunk=1024, dtype=torch.float32):
+    """dq, dk, dv of sum(o * do) by autograd through the explicit forward, one row
+    chunk at a time (bounded memory).  Matches the reference's gradient contract
+    (bitfield_attention.py:840-886): dk/dv are summed over the q-heads of a group."""
+    B, S, Hq, D = q.shape
+    scale = softmax_scale or 1.0 / math.sqrt(D)
+    q, k, v, do = q.to(dtype), k.to(dtype), v.to(dtype), do.to(dtype)
+    dq = torch.zeros_like(q)
+    dk = torch.zeros_like(k)
+    dv = torch.zeros_like(v)
+    for b in range(B):
+        for r0 in range(0, S, row_chunk):
+            r1 = min(r0 + row_chunk, S)
+            allow = allow_rows(bitfield[b], r0, r1)
+            qc = q[b, r0:r1].detach().requires_grad_(True)
+            kb = k[b].detach().requires_grad_(True)
+            vb = v[b].detach().requires_grad_(True)
+            oc, _ = _chunk_forward(qc, kb, vb, allow, scale)
+            gq, gk, gv = torch.autograd.grad(oc, (qc, kb, vb), do[b, r0:r1])
+            dq[b, r0:r1] = gq
+            dk[b] += gk
+            dv[b] += gv
+    return dq, dk, dv
+
+
+def delta(o, do):
+    """delta[b,h,i] = sum_d o*do in fp32 (bitfield_attention.py:527-572)."""
+    return (o.float() * do.float()).sum(-1).transpose(1, 2).contiguous()

@@ -1,0 +1,221 @@
+"""Pins of the oracle: every check here compares the oracle with something that is NOT the
+oracle's own formula -- the closed-form masks and expectations held by the reference's own
+tests, library routines (SDPA, logsumexp, autograd), analytic counts, or a second,
+independently written restatement (C scalar loops vs vectorized torch)."""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import bam_oracle as O
+from oracle import c_oracle as C
+from tests.helpers import random_bitfield, reference_mask_kat, reference_test_bitfield, rel_l2
+
+
+# ------------------------------------------------------------------ allow rule / mask
+@pytest.mark.parametrize("size", ["small", "large"])
+def test_mask_matches_reference_kat(size):
+    bf, expected = reference_mask_kat(size)
+    assert torch.equal(O.materialize_mask(bf), expected)
+    assert np.array_equal(C.mask(bf.numpy()), expected.numpy())
+
+
+@pytest.mark.parametrize("S", [57, 128, 283])
+def test_mask_matches_reference_fwd_test_layout(S):
+    bf, expected = reference_test_bitfield(2, S)
+    assert torch.equal(O.materialize_mask(bf), expected)
+    assert np.array_equal(C.mask(bf.numpy()), expected.numpy())
+
+
+def test_mask_degenerate_layouts():
+    S = 96
+    tril = torch.tril(torch.ones((1, S, S), dtype=torch.bool))
+    # all text == causal (tests/test_shardformer/utils.py:388-391), with or without the
+    # decorative bit 62 and whatever bit 63 holds
+    for text in [(1 << 62) | 1, 1, -(1 << 63) | 1, (1 << 62) | 1 | 6]:
+        bf = torch.full((1, S), text, dtype=torch.int64)
+        assert torch.equal(O.materialize_mask(bf), tril)
+        assert np.array_equal(C.mask(bf.numpy()), tril.numpy())
+    # one modality everywhere == dense; padding (0) == nothing
+    bf = torch.full((1, S), 1 << 1, dtype=torch.int64)
+    assert O.materialize_mask(bf).all() and C.mask(bf.numpy()).all()
+    bf = torch.zeros((1, S), dtype=torch.int64)
+    assert not O.materialize_mask(bf).any() and not C.mask(bf.numpy()).any()
+    # bits 62/63 alone carry no modality: such tokens see nothing and are seen by nobody
+    bf = torch.full((1, S), 1 << 62, dtype=torch.int64)
+    assert not O.materialize_mask(bf).any() and not C.mask(bf.numpy()).any()
+
+
+def test_mask_text_without_modality_bit_cannot_see_that_modality():
+    # text carries bit 1 only; a modality-2 segment is invisible to it, modality-1 visible
+    S = 32
+    bf = torch.full((1, S), (1 << 62) | 1 | 2, dtype=torch.int64)
+    bf[0, 4:8] = 2
+    bf[0, 12:16] = 4
+    m = O.materialize_mask(bf)[0]
+    assert m[20, 4:8].all() and not m[20, 12:16].any()
+    assert m[12:16, 12:16].all() and not m[12:16, :12].any() and not m[12:16, 16:].any()
+
+
+@pytest.mark.parametrize("seed", [0, 1, 2])
+@pytest.mark.parametrize("wide", [False, True])
+def test_two_restatements_agree_on_random_bitfields(seed, wide):
+    bf = random_bitfield(2, 200, seed, pad=7, wide=wide)
+    assert np.array_equal(O.materialize_mask(bf).numpy(), C.mask(bf.numpy()))
+    assert np.array_equal(O.tile_flags(bf).numpy(), C.tile_flags(bf.numpy()))
+
+
+def test_indexed_mask_is_a_gather_of_the_global_mask():
+    # context-parallel callers evaluate the rule on global positions (reference :71-81)
+    bf = random_bitfield(1, 160, 3)
+    full = O.materialize_mask(bf)[0]
+    g = torch.Generator().manual_seed(0)
+    idx_q = torch.randperm(160, generator=g)[:48].sort().values
+    idx_k = torch.arange(160)
+    got = O.allow_rows(bf[0], 0, 48, idx_q=idx_q, idx_k=idx_k)
+    assert torch.equal(got, full[idx_q][:, idx_k])
+    c = C.mask_indexed(bf.numpy(), idx_q.numpy(), idx_k.numpy())[0]
+    assert np.array_equal(c, got.numpy())
+    # an out-of-range index behaves like padding
+    idx_k2 = torch.cat([idx_k[:10], torch.tensor([160])])
+    got2 = O.allow_rows(bf[0], 0, 48, idx_q=idx_q, idx_k=idx_k2)
+    assert not got2[:, -1].any()
+    assert np.array_equal(C.mask_indexed(bf.numpy(), idx_q.numpy(), idx_k2.numpy())[0], got2.numpy())
+
+
+# ------------------------------------------------------------------------- tile flags
+def test_flags_plumbing_layout_analytic_histogram():
+    # tokens 0-255 one image (bit 1), 256-1023 text: derived by hand -> 124 full, 24 partial,
+    # 108 empty tiles of 128x32 and 557440 allowed pairs
+    bf = torch.full((1, 1024), (1 << 62) | 1 | 2, dtype=torch.int64)
+    bf[0, :256] = 2
+    for flags in (O.tile_flags(bf), torch.from_numpy(C.tile_flags(bf.numpy()))):
+        assert flags.shape == (1, 8, 32) and flags.dtype == torch.int8
+        assert [(flags == v).sum().item() for v in (0, 1, 2)] == [108, 24, 124]
+    assert O.unmasked_pairs(bf) == 256 * 256 + sum(range(257, 1025)) == 557440
+
+
+@pytest.mark.parametrize("S", [57, 256, 335, 684, 1024, 2003, 3712])
+def test_flags_rowblock_workloads_of_context_parallel_test(S):
+    # tests/test_shardformer/test_context_parallel.py:192-274 relies on these per-row-block
+    # counts of non-empty tiles: causal -> 4(m+1) capped at ceil(S/32); dense -> ceil(S/32)
+    nn = -(-S // 32)
+    causal = O.tile_flags(torch.full((1, S), (1 << 62) | 1, dtype=torch.int64))[0]
+    assert [(row > 0).sum().item() for row in causal] == [min(4 * (m + 1), nn) for m in range(causal.shape[0])]
+    dense = O.tile_flags(torch.full((1, S), 1 << 1, dtype=torch.int64))[0]
+    assert (dense == 2).all()  # ragged edge tiles count only in-range cells (reference :149-153)
+    # below the diagonal causal tiles are full, on it partial, above it empty
+    m = causal.shape[0] - 1
+    if S % 128 == 0:
+        assert (causal[m, : 4 * m] == 2).all() and (causal[m, 4 * m :] == 1).all()
+
+
+def test_flags_classification_vs_mask_bruteforce():
+    bf = random_bitfield(2, 300, 5, pad=9)
+    mask = O.materialize_mask(bf)
+    flags = C.tile_flags(bf.numpy())
+    for b in range(2):
+        for m in range(3):
+            for n in range(10):
+                t = mask[b, 128 * m : 128 * m + 128, 32 * n : 32 * n + 32]
+                want = 0 if t.sum() == 0 else (2 if t.all() else 1)
+                assert flags[b, m, n] == want
+
+
+# ------------------------------------------------------------------- bitfield format
+def test_bitfield_format_golden_vectors():
+    # tests/test_models/test_multimodal_merge_outputs.py:94-110: vision -> 1<<1, audio -> 1<<2,
+    # text -> (1<<62) | 1 | 2 | 4
+    from cornstarch_amd.kernel.interface import create_bitfield_attention_mask as product_fn
+
+    vid, aid = 44, 55
+    for vis, aud in [([2, 3, 4, 5], [9, 10, 11]), ([0, 1], []), ([], [13, 14, 15])]:
+        ids = torch.arange(16).unsqueeze(0).clone()
+        want = torch.full((1, 16), (1 << 62) | 1 | 2 | 4, dtype=torch.int64)
+        ids[0, vis] = vid
+        want[0, vis] = 1 << 1
+        ids[0, aud] = aid
+        want[0, aud] = 1 << 2
+        tok = {"vision": vid, "audio": aid}
+        assert torch.equal(O.create_bitfield_attention_mask(ids, tok), want)
+        assert torch.equal(product_fn(ids, tok), want)
+
+
+# --------------------------------------------------------------- forward / backward
+def _rand(B, S, Hq, Hkv, D, seed=0, dtype=torch.float32):
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn(B, S, Hq, D, generator=g, dtype=dtype) * 0.5
+    k = torch.randn(B, S, Hkv, D, generator=g, dtype=dtype) * 0.5
+    v = torch.randn(B, S, Hkv, D, generator=g, dtype=dtype) * 0.5
+    do = torch.randn(B, S, Hq, D, generator=g, dtype=dtype)
+    return q, k, v, do
+
+
+@pytest.mark.parametrize("S,Hq,Hkv,D", [(57, 6, 6, 32), (144, 6, 2, 64), (283, 6, 3, 16)])
+def test_forward_against_library_sdpa_and_c_loops(S, Hq, Hkv, D):
+    # the reference's ground truth: SDPA with the materialized mask, enable_gqa
+    bf, full = reference_test_bitfield(2, S)
+    q, k, v, _ = _rand(2, S, Hq, Hkv, D, dtype=torch.float64)
+    want = F.scaled_dot_product_attention(
+        q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), attn_mask=full.unsqueeze(1), enable_gqa=True
+    ).transpose(1, 2)
+    o, lse = O.attention_forward(q, k, v, bf, dtype=torch.float64)
+    assert torch.allclose(o, want, atol=1e-10, rtol=0)
+    assert torch.allclose(O.attention_sdpa(q, k, v, bf), want, atol=1e-10, rtol=0)
+    # LSE against library logsumexp over independently built (repeat_interleave) scores
+    g = Hq // Hkv
+    s = torch.einsum("bihd,bjhd->bhij", q, k.repeat_interleave(g, dim=2)) / math.sqrt(D)
+    want_lse = torch.logsumexp(s.masked_fill(~full.unsqueeze(1), float("-inf")), dim=-1)
+    assert torch.allclose(lse, want_lse, atol=1e-10, rtol=0)
+    co, clse = C.attn_fwd(q.float().numpy(), k.float().numpy(), v.float().numpy(), bf.numpy())
+    assert np.allclose(co, want.float().numpy(), atol=2e-6) and np.allclose(clse, want_lse.float().numpy(), atol=2e-6)
+
+
+@pytest.mark.parametrize("S,Hq,Hkv,D", [(57, 6, 6, 32), (144, 6, 2, 64), (130, 4, 1, 16)])
+def test_backward_against_autograd_through_sdpa(S, Hq, Hkv, D):
+    bf, full = reference_test_bitfield(2, S)
+    q, k, v, do = _rand(2, S, Hq, Hkv, D, seed=1, dtype=torch.float64)
+    qr, kr, vr = (x.clone().requires_grad_(True) for x in (q, k, v))
+    ref = F.scaled_dot_product_attention(
+        qr.transpose(1, 2), kr.transpose(1, 2), vr.transpose(1, 2), attn_mask=full.unsqueeze(1), enable_gqa=True
+    ).transpose(1, 2)
+    wq, wk, wv = torch.autograd.grad(ref, (qr, kr, vr), do)
+    dq, dk, dv = O.attention_backward(q, k, v, bf, do, row_chunk=50, dtype=torch.float64)
+    for got, want in ((dq, wq), (dk, wk), (dv, wv)):
+        assert torch.allclose(got, want, atol=1e-10, rtol=0)
+    # closed-form restatement (P, dS formulas of the reference's backward) in C
+    o, lse = O.attention_forward(q, k, v, bf, dtype=torch.float64)
+    dlt = C.delta(o.float().numpy(), do.float().numpy())
+    assert np.allclose(dlt, O.delta(o, do).numpy(), atol=1e-5)
+    cq, ck, cv = C.attn_bwd(*(x.float().numpy() for x in (q, k, v, do)), lse.float().numpy(), dlt, bf.numpy())
+    for got, want in ((cq, wq), (ck, wk), (cv, wv)):
+        assert rel_l2(torch.from_numpy(got), want) < 1e-5
+
+
+def test_rows_without_any_allowed_key_give_zero_output_and_minus_inf_lse():
+    # right padding = bitfield 0 (reference modeling_multimodal_language_model.py:947-948);
+    # the reference kernel defines o = 0, lse = -inf there (bitfield_attention.py:441-444,493-495)
+    bf = random_bitfield(1, 90, 2, pad=11)
+    q, k, v, do = _rand(1, 90, 2, 2, 16, seed=3)
+    o, lse = O.attention_forward(q, k, v, bf)
+    assert (o[0, -11:] == 0).all() and torch.isinf(lse[0, :, -11:]).all() and (lse[0, :, -11:] < 0).all()
+    assert torch.isfinite(o).all()
+    co, clse = C.attn_fwd(q.numpy(), k.numpy(), v.numpy(), bf.numpy())
+    assert (co[0, -11:] == 0).all() and np.isneginf(clse[0, :, -11:]).all()
+    dq, dk, dv = O.attention_backward(q, k, v, bf, do)
+    assert torch.isfinite(dq).all() and (dq[0, -11:] == 0).all() and (dk[0, -11:] == 0).all()
+    assert torch.allclose(O.attention_sdpa(q, k, v, bf), o, atol=1e-5)
+
+
+def test_all_text_bitfield_is_plain_causal_attention():
+    S = 77
+    bf = torch.full((1, S), (1 << 62) | 1, dtype=torch.int64)
+    q, k, v, _ = _rand(1, S, 4, 4, 32, seed=4)
+    want = F.scaled_dot_product_attention(
+        q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), is_causal=True
+    ).transpose(1, 2)
+    o, _ = O.attention_forward(q, k, v, bf)
+    assert torch.allclose(o, want, atol=1e-5)
