@@ -1,0 +1,203 @@
+#!/usr/bin/env python3
+"""Benchmark of bitfield-masked attention on one MI355X.
+
+A step is one pass of the hot path over one batch of synthetic input that is already
+resident in HBM: tile flags -> forward -> zeroed fp32 gradient buffers -> delta -> dK/dV ->
+dQ -> cast of the gradients to the input dtype, i.e. everything
+``bitfield_attn_func(...).backward(dO)`` launches.  The figure of merit is effective
+TFLOP/s over UNMASKED (query, key) pairs: fwd 4*D*Hq*pairs, bwd 10*D*Hq*pairs.
+
+Prints one JSON line (see --help for the knobs).  The CPU baseline leg times the oracle's
+materialized-mask SDPA in fp32 on the host cores on a bounded sample (one KV group).
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_BF16_DENSE_TFLOPS = 2500.0  # MI355X published dense bf16 MFMA peak
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="C2", choices=["C2", "C3", "C4", "C5"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--traffic", default=None, help="JSON file with measured HBM bytes per launch (from rocprofv3 --pmc)")
+    return ap.parse_args()
+
+
+def cpu_baseline(name):
+    """Oracle (port of the reference tests' ground truth): bool mask from the bitfields +
+    library SDPA in fp32 on the host, fwd+bwd, on the first KV group of the workload."""
+    import torch
+
+    from cornstarch_amd import workloads as W
+    from oracle import bam_oracle as O
+
+    w = W.WORKLOADS[name]
+    G = w.Hq // w.Hkv
+    q, k, v, do = (t.float() for t in W.make_tensors(name, heads=(0, G)))
+    bf = W.make_bitfields(name)
+    if name == "C4":  # one sequence of the packed batch
+        q, k, v, do, bf = q[:1], k[:1], v[:1], do[:1], bf[:1]
+    pairs = O.unmasked_pairs(bf)
+    flops = 14 * w.D * G * pairs
+    torch.set_num_threads(min(os.cpu_count() or 1, 16))
+    times = []
+    for _ in range(2):
+        t0 = time.perf_counter()
+        O.sdpa_forward_backward(q, k, v, bf, do, row_chunk=2048)
+        times.append(time.perf_counter() - t0)
+    t = min(times)
+    return {
+        "value": flops / t / 1e12,
+        "unit": "TFLOP/s",
+        "cores": torch.get_num_threads(),
+        "kind": "port",
+        "seconds": t,
+        "sample": f"{name} q-heads 0..{G - 1} + kv-head 0" + (", sequence 0" if name == "C4" else "")
+        + ", fwd+bwd fp32 materialized-mask SDPA, best of 2",
+    }
+
+
+def main():
+    args = parse()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from cornstarch_amd import workloads as W
+    from cornstarch_amd.kernel import bitfield_attention as BA
+    from oracle import bam_oracle as O  # checker / baseline only
+
+    assert torch.cuda.is_available(), "bench.py needs the GPU"
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    name = args.workload
+    w = W.WORKLOADS[name]
+
+    q, k, v, do = (t.to(dev) for t in W.make_tensors(name))
+    bf_cpu = W.make_bitfields(name)
+    bf = bf_cpu.to(dev)
+    pairs = O.unmasked_pairs(bf)  # exact, on the GPU through torch ops (setup, untimed)
+    f_fwd = 4 * w.D * w.Hq * pairs
+    f_bwd = 10 * w.D * w.Hq * pairs
+    scale = 1.0 / math.sqrt(w.D)
+
+    stages = ["flags", "fwd", "zero", "delta", "dkdv", "dq", "cast"]
+    n_ev = len(stages) + 1
+
+    def step(ev=None):
+        def mark(i):
+            if ev is not None:
+                ev[i].record()
+
+        mark(0)
+        BA.BitfieldUtils.clear_cache()
+        flags = BA.BitfieldUtils.materialize_compressed_mask_from_bitfield_mask(bf)
+        mark(1)
+        o, lse, _ = BA._bitfield_attn_forward(q, k, v, bf, flags, softmax_scale=scale)
+        mark(2)
+        dq = torch.zeros_like(q, dtype=torch.float32)
+        dk = torch.zeros_like(k, dtype=torch.float32)
+        dv = torch.zeros_like(v, dtype=torch.float32)
+        delta = torch.empty_like(lse)
+        mark(3)
+        BA._launch_bwd_preprocess(o, do, delta)
+        mark(4)
+        BA._launch_bwd_dkdv(q, k, v, do, lse, delta, dk, dv, bf, flags, scale)
+        mark(5)
+        BA._launch_bwd_dq(q, k, v, do, lse, delta, dq, bf, flags, scale)
+        mark(6)
+        out = dq.to(q.dtype), dk.to(k.dtype), dv.to(v.dtype)
+        mark(7)
+        return o, out
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+
+    events = [[torch.cuda.Event(enable_timing=True) for _ in range(n_ev)] for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(events[i])
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+
+    ms_per_step = wall * 1e3 / args.steps
+    stage_ms = {}
+    for si, s in enumerate(stages):
+        stage_ms[s] = sum(ev[si].elapsed_time(ev[si + 1]) for ev in events) / args.steps
+    fwd_ms = stage_ms["flags"] + stage_ms["fwd"]
+    bwd_ms = stage_ms["zero"] + stage_ms["delta"] + stage_ms["dkdv"] + stage_ms["dq"] + stage_ms["cast"]
+
+    # dominant kernel and its algorithmic FLOPs per launch (5-GEMM accounting of the
+    # backward: the dK/dV kernel owns S, dP, dV, dK; the dQ kernel owns dQ)
+    algo = {"fwd": f_fwd, "dkdv": 8 * w.D * w.Hq * pairs, "dq": 2 * w.D * w.Hq * pairs}
+    kname = {"fwd": "fwd_kernel", "dkdv": "bwd_dkdv_kernel", "dq": "bwd_dq_kernel"}
+    dom = max(algo, key=lambda s: stage_ms[s])
+    achieved = algo[dom] / (stage_ms[dom] * 1e-3) / 1e12
+    traffic = None
+    if args.traffic and os.path.exists(args.traffic):
+        with open(args.traffic) as f:
+            traffic = json.load(f).get(kname[dom])
+
+    value = (f_fwd + f_bwd) / (ms_per_step * 1e-3) / 1e12
+    result = {
+        "metric": "bitfield attention fwd+bwd effective TFLOP/s over unmasked pairs (S=8192 GQA bf16)"
+        if name == "C2"
+        else f"bitfield attention fwd+bwd effective TFLOP/s over unmasked pairs ({name})",
+        "value": round(value, 3),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": f"{name}: B={w.B} S={w.S} Hq={w.Hq} Hkv={w.Hkv} D={w.D} bf16 fwd+bwd, {w.description}",
+            "unmasked_pairs": pairs,
+            "flops_fwd": f_fwd,
+            "flops_bwd": f_bwd,
+        },
+        "fwd_ms": round(fwd_ms, 4),
+        "bwd_ms": round(bwd_ms, 4),
+        "fwd_tflops": round(f_fwd / (fwd_ms * 1e-3) / 1e12, 3),
+        "mfma_util_unmasked": round(value / PEAK_BF16_DENSE_TFLOPS, 4),
+        "stage_ms": {s: round(x, 4) for s, x in stage_ms.items()},
+        "roofline": {
+            "kernel": kname[dom],
+            "bound": "mfma",
+            "achieved": round(achieved, 3),
+            "peak": PEAK_BF16_DENSE_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": round(achieved / PEAK_BF16_DENSE_TFLOPS, 4),
+            "traffic": traffic,
+            "avg_launch_ms": round(stage_ms[dom], 4),
+        },
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(name)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

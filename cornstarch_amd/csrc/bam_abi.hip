@@ -148,6 +148,47 @@ int bam_bwd_preprocess(const void* o, const void* dout, float* delta, int64_t o_
     return launched(bam::launch_bwd_preprocess(p, dtype, (hipStream_t)stream), "bam_bwd_preprocess");
 }
 
+static int bwd_params(bam::AttnParams& p, const void* q, const void* k, const void* v, const void* dout,
+                      const float* lse, const float* delta, float* dq, float* dk, float* dv, const int64_t* bf,
+                      const int8_t* flags, const int64_t* st, int B, int S, int Hq, int Hkv, int D, float scale,
+                      int dtype, bool need_dq, bool need_dkdv) {
+    BAM_TRY(check_problem(B, S, Hq, Hkv, D, dtype));
+    BAM_TRY(check_half_tensor("q", q, st[0], st[1], st[2]));
+    BAM_TRY(check_half_tensor("k", k, st[3], st[4], st[5]));
+    BAM_TRY(check_half_tensor("v", v, st[6], st[7], st[8]));
+    BAM_TRY(check_half_tensor("do", dout, st[9], st[10], st[11]));
+    if (need_dq) BAM_TRY(check_f32_tensor("dq", dq, st[12], st[13], st[14]));
+    if (need_dkdv) {
+        BAM_TRY(check_f32_tensor("dk", dk, st[15], st[16], st[17]));
+        BAM_TRY(check_f32_tensor("dv", dv, st[18], st[19], st[20]));
+    }
+    if (lse == nullptr || delta == nullptr || bf == nullptr || flags == nullptr)
+        return fail(BAM_ERR_INVALID_ARGUMENT, "bam_bwd: lse, delta, bf and flags must not be null");
+    if (!(scale > 0.f)) return fail(BAM_ERR_INVALID_ARGUMENT, "bam_bwd: softmax scale must be > 0 (got %g)", scale);
+    if ((int64_t)((S + 127) / 128) * B * Hq > 0x7FFFFFFFll) return fail(BAM_ERR_UNSUPPORTED, "bam_bwd: grid too large");
+    p.q = {q, st[0], st[1], st[2]};
+    p.k = {k, st[3], st[4], st[5]};
+    p.v = {v, st[6], st[7], st[8]};
+    p.dout = {dout, st[9], st[10], st[11]};
+    p.dq = {dq, st[12], st[13], st[14]};
+    p.dk = {dk, st[15], st[16], st[17]};
+    p.dv = {dv, st[18], st[19], st[20]};
+    p.lse = const_cast<float*>(lse);
+    p.delta = const_cast<float*>(delta);
+    p.bf = bf;
+    p.bf_sb = st[21];
+    p.flags = flags;
+    p.flags_sb = st[22];
+    p.flags_sm = st[23];
+    fill_sizes(p, B, S, Hq, Hkv, D, scale);
+    return BAM_OK;
+}
+
+#define BAM_BWD_STRIDES                                                                                      \
+    {q_stride_b,  q_stride_s,  q_stride_h,  k_stride_b,  k_stride_s,  k_stride_h,  v_stride_b,  v_stride_s,  \
+     v_stride_h,  do_stride_b, do_stride_s, do_stride_h, dq_stride_b, dq_stride_s, dq_stride_h, dk_stride_b, \
+     dk_stride_s, dk_stride_h, dv_stride_b, dv_stride_s, dv_stride_h, bf_stride_b, flags_stride_b, flags_stride_m}
+
 int bam_bwd(const void* q, const void* k, const void* v, const void* dout, const float* lse,
             const float* delta, float* dq, float* dk, float* dv, const int64_t* bf, const int8_t* flags,
             int64_t q_stride_b, int64_t q_stride_s, int64_t q_stride_h, int64_t k_stride_b,
@@ -157,36 +198,44 @@ int bam_bwd(const void* q, const void* k, const void* v, const void* dout, const
             int64_t dk_stride_s, int64_t dk_stride_h, int64_t dv_stride_b, int64_t dv_stride_s,
             int64_t dv_stride_h, int64_t bf_stride_b, int64_t flags_stride_b, int64_t flags_stride_m, int B,
             int S, int Hq, int Hkv, int D, float scale, int dtype, void* stream) {
-    BAM_TRY(check_problem(B, S, Hq, Hkv, D, dtype));
-    BAM_TRY(check_half_tensor("q", q, q_stride_b, q_stride_s, q_stride_h));
-    BAM_TRY(check_half_tensor("k", k, k_stride_b, k_stride_s, k_stride_h));
-    BAM_TRY(check_half_tensor("v", v, v_stride_b, v_stride_s, v_stride_h));
-    BAM_TRY(check_half_tensor("do", dout, do_stride_b, do_stride_s, do_stride_h));
-    BAM_TRY(check_f32_tensor("dq", dq, dq_stride_b, dq_stride_s, dq_stride_h));
-    BAM_TRY(check_f32_tensor("dk", dk, dk_stride_b, dk_stride_s, dk_stride_h));
-    BAM_TRY(check_f32_tensor("dv", dv, dv_stride_b, dv_stride_s, dv_stride_h));
-    if (lse == nullptr || delta == nullptr || bf == nullptr || flags == nullptr)
-        return fail(BAM_ERR_INVALID_ARGUMENT, "bam_bwd: lse, delta, bf and flags must not be null");
-    if (!(scale > 0.f)) return fail(BAM_ERR_INVALID_ARGUMENT, "bam_bwd: softmax scale must be > 0 (got %g)", scale);
-    if ((int64_t)((S + 127) / 128) * B * Hq > 0x7FFFFFFFll) return fail(BAM_ERR_UNSUPPORTED, "bam_bwd: grid too large");
+    const int64_t st[24] = BAM_BWD_STRIDES;
     bam::AttnParams p = {};
-    p.q = {q, q_stride_b, q_stride_s, q_stride_h};
-    p.k = {k, k_stride_b, k_stride_s, k_stride_h};
-    p.v = {v, v_stride_b, v_stride_s, v_stride_h};
-    p.dout = {dout, do_stride_b, do_stride_s, do_stride_h};
-    p.dq = {dq, dq_stride_b, dq_stride_s, dq_stride_h};
-    p.dk = {dk, dk_stride_b, dk_stride_s, dk_stride_h};
-    p.dv = {dv, dv_stride_b, dv_stride_s, dv_stride_h};
-    p.lse = const_cast<float*>(lse);
-    p.delta = const_cast<float*>(delta);
-    p.bf = bf;
-    p.bf_sb = bf_stride_b;
-    p.flags = flags;
-    p.flags_sb = flags_stride_b;
-    p.flags_sm = flags_stride_m;
-    fill_sizes(p, B, S, Hq, Hkv, D, scale);
+    BAM_TRY(bwd_params(p, q, k, v, dout, lse, delta, dq, dk, dv, bf, flags, st, B, S, Hq, Hkv, D, scale, dtype, true, true));
     BAM_TRY(launched(bam::launch_bwd_dkdv(p, dtype, (hipStream_t)stream), "bam_bwd (dk/dv)"));
     return launched(bam::launch_bwd_dq(p, dtype, (hipStream_t)stream), "bam_bwd (dq)");
+}
+
+int bam_bwd_dkdv(const void* q, const void* k, const void* v, const void* dout, const float* lse,
+                 const float* delta, float* dk, float* dv, const int64_t* bf, const int8_t* flags,
+                 int64_t q_stride_b, int64_t q_stride_s, int64_t q_stride_h, int64_t k_stride_b,
+                 int64_t k_stride_s, int64_t k_stride_h, int64_t v_stride_b, int64_t v_stride_s,
+                 int64_t v_stride_h, int64_t do_stride_b, int64_t do_stride_s, int64_t do_stride_h,
+                 int64_t dk_stride_b, int64_t dk_stride_s, int64_t dk_stride_h, int64_t dv_stride_b,
+                 int64_t dv_stride_s, int64_t dv_stride_h, int64_t bf_stride_b, int64_t flags_stride_b,
+                 int64_t flags_stride_m, int B, int S, int Hq, int Hkv, int D, float scale, int dtype,
+                 void* stream) {
+    float* dq = nullptr;
+    const int64_t dq_stride_b = 0, dq_stride_s = 0, dq_stride_h = 0;
+    const int64_t st[24] = BAM_BWD_STRIDES;
+    bam::AttnParams p = {};
+    BAM_TRY(bwd_params(p, q, k, v, dout, lse, delta, dq, dk, dv, bf, flags, st, B, S, Hq, Hkv, D, scale, dtype, false, true));
+    return launched(bam::launch_bwd_dkdv(p, dtype, (hipStream_t)stream), "bam_bwd_dkdv");
+}
+
+int bam_bwd_dq(const void* q, const void* k, const void* v, const void* dout, const float* lse,
+               const float* delta, float* dq, const int64_t* bf, const int8_t* flags, int64_t q_stride_b,
+               int64_t q_stride_s, int64_t q_stride_h, int64_t k_stride_b, int64_t k_stride_s,
+               int64_t k_stride_h, int64_t v_stride_b, int64_t v_stride_s, int64_t v_stride_h,
+               int64_t do_stride_b, int64_t do_stride_s, int64_t do_stride_h, int64_t dq_stride_b,
+               int64_t dq_stride_s, int64_t dq_stride_h, int64_t bf_stride_b, int64_t flags_stride_b,
+               int64_t flags_stride_m, int B, int S, int Hq, int Hkv, int D, float scale, int dtype,
+               void* stream) {
+    float *dk = nullptr, *dv = nullptr;
+    const int64_t dk_stride_b = 0, dk_stride_s = 0, dk_stride_h = 0, dv_stride_b = 0, dv_stride_s = 0, dv_stride_h = 0;
+    const int64_t st[24] = BAM_BWD_STRIDES;
+    bam::AttnParams p = {};
+    BAM_TRY(bwd_params(p, q, k, v, dout, lse, delta, dq, dk, dv, bf, flags, st, B, S, Hq, Hkv, D, scale, dtype, true, false));
+    return launched(bam::launch_bwd_dq(p, dtype, (hipStream_t)stream), "bam_bwd_dq");
 }
 
 }  // extern "C"

@@ -184,6 +184,47 @@ def _bitfield_attn_forward(
     return o, lse, softmax_scale
 
 
+def _strides3(*tensors):
+    out = []
+    for t in tensors:
+        out += [t.stride(0), t.stride(1), t.stride(2)]
+    return out
+
+
+def _launch_bwd_preprocess(o, do, delta):
+    """delta = rowsum(o * do); tensors must already satisfy the kernels' layout rules."""
+    B, S, Hq, D = o.shape
+    with torch.cuda.device(o.device):
+        _bam_hip.call(
+            "bam_bwd_preprocess", o.data_ptr(), do.data_ptr(), delta.data_ptr(), *_strides3(o, do),
+            B, S, Hq, D, _dtype_code(o.dtype), _stream_ptr(o.device),
+        )
+
+
+def _launch_bwd_dkdv(q, k, v, do, lse, delta, dk, dv, bf, flags, softmax_scale):
+    B, S, Hq, D = q.shape
+    with torch.cuda.device(q.device):
+        _bam_hip.call(
+            "bam_bwd_dkdv",
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), do.data_ptr(), lse.data_ptr(), delta.data_ptr(),
+            dk.data_ptr(), dv.data_ptr(), bf.data_ptr(), flags.data_ptr(),
+            *_strides3(q, k, v, do, dk, dv), bf.stride(0), flags.stride(0), flags.stride(1),
+            B, S, Hq, k.shape[2], D, float(softmax_scale), _dtype_code(q.dtype), _stream_ptr(q.device),
+        )
+
+
+def _launch_bwd_dq(q, k, v, do, lse, delta, dq, bf, flags, softmax_scale):
+    B, S, Hq, D = q.shape
+    with torch.cuda.device(q.device):
+        _bam_hip.call(
+            "bam_bwd_dq",
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), do.data_ptr(), lse.data_ptr(), delta.data_ptr(),
+            dq.data_ptr(), bf.data_ptr(), flags.data_ptr(),
+            *_strides3(q, k, v, do, dq), bf.stride(0), flags.stride(0), flags.stride(1),
+            B, S, Hq, k.shape[2], D, float(softmax_scale), _dtype_code(q.dtype), _stream_ptr(q.device),
+        )
+
+
 def _bitfield_attn_backward(
     do: torch.Tensor,
     q: torch.Tensor,
@@ -228,31 +269,10 @@ def _bitfield_attn_backward(
     bf = bitfield_mask if bitfield_mask.stride(1) == 1 else bitfield_mask.contiguous()
     flags = compressed_mask if compressed_mask.stride(-1) == 1 else compressed_mask.contiguous()
     delta = torch.empty_like(lse)
-    code = _dtype_code(q.dtype)
-    stream = _stream_ptr(q.device)
-    with torch.cuda.device(q.device):
-        _bam_hip.call(
-            "bam_bwd_preprocess",
-            ok.data_ptr(), gk.data_ptr(), delta.data_ptr(),
-            ok.stride(0), ok.stride(1), ok.stride(2),
-            gk.stride(0), gk.stride(1), gk.stride(2),
-            batch, seqlen_q, nheads, dp, code, stream,
-        )
-        wq, wk, wv = work
-        _bam_hip.call(
-            "bam_bwd",
-            qk.data_ptr(), kk.data_ptr(), vk.data_ptr(), gk.data_ptr(), lse.data_ptr(), delta.data_ptr(),
-            wq.data_ptr(), wk.data_ptr(), wv.data_ptr(), bf.data_ptr(), flags.data_ptr(),
-            qk.stride(0), qk.stride(1), qk.stride(2),
-            kk.stride(0), kk.stride(1), kk.stride(2),
-            vk.stride(0), vk.stride(1), vk.stride(2),
-            gk.stride(0), gk.stride(1), gk.stride(2),
-            wq.stride(0), wq.stride(1), wq.stride(2),
-            wk.stride(0), wk.stride(1), wk.stride(2),
-            wv.stride(0), wv.stride(1), wv.stride(2),
-            bf.stride(0), flags.stride(0), flags.stride(1),
-            batch, seqlen_q, nheads, nheads_k, dp, float(softmax_scale), code, stream,
-        )
+    wq, wk, wv = work
+    _launch_bwd_preprocess(ok, gk, delta)
+    _launch_bwd_dkdv(qk, kk, vk, gk, lse, delta, wk, wv, bf, flags, softmax_scale)
+    _launch_bwd_dq(qk, kk, vk, gk, lse, delta, wq, bf, flags, softmax_scale)
     # the kernels accumulated into `work`; hand the sums back if those were copies
     for dst, mid, w in zip((dq, dk, dv), acc, work):
         if dp != d:

@@ -98,6 +98,32 @@ int bam_bwd(const void* q, const void* k, const void* v, const void* dout, const
             int64_t dv_stride_h, int64_t bf_stride_b, int64_t flags_stride_b, int64_t flags_stride_m, int B,
             int S, int Hq, int Hkv, int D, float scale, int dtype, void* stream);
 
+/*
+ * The two halves of bam_bwd as separate launches (same reference kernel,
+ * bitfield_attention.py:598-929): bam_bwd_dkdv accumulates dk/dv only, bam_bwd_dq
+ * accumulates dq only.  bam_bwd == bam_bwd_dkdv followed by bam_bwd_dq.  They exist so
+ * that each kernel can be timed on its own and so that a caller that needs only one side
+ * (frozen encoder outputs, for instance) does not pay for the other.
+ */
+int bam_bwd_dkdv(const void* q, const void* k, const void* v, const void* dout, const float* lse,
+                 const float* delta, float* dk, float* dv, const int64_t* bf, const int8_t* flags,
+                 int64_t q_stride_b, int64_t q_stride_s, int64_t q_stride_h, int64_t k_stride_b,
+                 int64_t k_stride_s, int64_t k_stride_h, int64_t v_stride_b, int64_t v_stride_s,
+                 int64_t v_stride_h, int64_t do_stride_b, int64_t do_stride_s, int64_t do_stride_h,
+                 int64_t dk_stride_b, int64_t dk_stride_s, int64_t dk_stride_h, int64_t dv_stride_b,
+                 int64_t dv_stride_s, int64_t dv_stride_h, int64_t bf_stride_b, int64_t flags_stride_b,
+                 int64_t flags_stride_m, int B, int S, int Hq, int Hkv, int D, float scale, int dtype,
+                 void* stream);
+
+int bam_bwd_dq(const void* q, const void* k, const void* v, const void* dout, const float* lse,
+               const float* delta, float* dq, const int64_t* bf, const int8_t* flags, int64_t q_stride_b,
+               int64_t q_stride_s, int64_t q_stride_h, int64_t k_stride_b, int64_t k_stride_s,
+               int64_t k_stride_h, int64_t v_stride_b, int64_t v_stride_s, int64_t v_stride_h,
+               int64_t do_stride_b, int64_t do_stride_s, int64_t do_stride_h, int64_t dq_stride_b,
+               int64_t dq_stride_s, int64_t dq_stride_h, int64_t bf_stride_b, int64_t flags_stride_b,
+               int64_t flags_stride_m, int B, int S, int Hq, int Hkv, int D, float scale, int dtype,
+               void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -227,3 +227,39 @@ def attention_backward(q, k, v, bitfield, do, softmax_scale=None, row_chunk=1024
 def delta(o, do):
     """delta[b,h,i] = sum_d o*do in fp32 (bitfield_attention.py:527-572)."""
     return (o.float() * do.float()).sum(-1).transpose(1, 2).contiguous()
+
+
+def sdpa_forward_backward(q, k, v, bitfield, do=None, softmax_scale=None, row_chunk=2048):
+    """The reference tests' ground truth at scale: bool mask from the bitfields + library
+    SDPA (``enable_gqa``), one block of query rows at a time so that the mask and the score
+    matrix stay bounded.  Returns o, and (dq, dk, dv) of sum(o * do) when ``do`` is given.
+    This is the routine the CPU baseline of the benchmark times."""
+    B, S, Hq, D = q.shape
+    gqa = Hq != k.shape[2]
+    o = torch.empty_like(q)
+    grads = None
+    if do is not None:
+        grads = (torch.zeros_like(q), torch.zeros_like(k), torch.zeros_like(v))
+    for b in range(B):
+        kb = k[b : b + 1].transpose(1, 2)
+        vb = v[b : b + 1].transpose(1, 2)
+        for r0 in range(0, S, row_chunk):
+            r1 = min(r0 + row_chunk, S)
+            allow = allow_rows(bitfield[b], r0, r1)
+            dead = ~allow.any(dim=-1)
+            qc = q[b : b + 1, r0:r1].transpose(1, 2)
+            if do is not None:
+                qc, kc, vc = (t.detach().requires_grad_(True) for t in (qc, kb, vb))
+            else:
+                kc, vc = kb, vb
+            oc = F.scaled_dot_product_attention(
+                qc, kc, vc, attn_mask=allow[None, None], scale=softmax_scale, enable_gqa=gqa
+            )
+            oc = torch.where(dead[None, None, :, None], torch.zeros_like(oc), oc)
+            o[b, r0:r1] = oc.detach().transpose(1, 2)[0]
+            if do is not None:
+                gq, gk, gv = torch.autograd.grad(oc, (qc, kc, vc), do[b : b + 1, r0:r1].transpose(1, 2))
+                grads[0][b, r0:r1] = gq.transpose(1, 2)[0]
+                grads[1][b] += gk.transpose(1, 2)[0]
+                grads[2][b] += gv.transpose(1, 2)[0]
+    return (o, *grads) if grads is not None else o
