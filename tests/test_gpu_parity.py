@@ -1,0 +1,342 @@
+"""Parity of the HIP kernels (through the C ABI) with the oracle, on an MI355X.
+
+Bars: tile flags and materialized mask bit exact; forward output within max-abs 2e-2 of the
+fp32 oracle (1e-2 + 1e-2*|x| elementwise for the reference's own test grid); gradients
+within relative L2 5e-2.  The oracle runs on the CPU for the small cases and, for the
+full-size workloads, as fp32 library math on the GPU (never the HIP kernels).
+"""
+
+import math
+
+import pytest
+import torch
+
+from cornstarch_amd import workloads as W
+from cornstarch_amd.kernel import bitfield_attention as BA
+from cornstarch_amd.kernel import interface
+from oracle import bam_oracle as O
+from oracle import c_oracle as C
+from tests.helpers import random_bitfield, reference_mask_kat, reference_test_bitfield, rel_l2
+
+pytestmark = pytest.mark.gpu
+
+O_MAX_ABS = 2e-2
+GRAD_REL_L2 = 5e-2
+
+
+def dev():
+    return torch.device("cuda:0")
+
+
+def flags_of(bf_gpu):
+    BA.BitfieldUtils.clear_cache()
+    return BA.BitfieldUtils.materialize_compressed_mask_from_bitfield_mask(bf_gpu)
+
+
+def run_hip(q, k, v, bf, do=None, scale=None):
+    """q, k, v, do: CPU tensors in the kernel dtype -> (o, lse[:S], dq, dk, dv) on the CPU."""
+    d = dev()
+    qg, kg, vg = (t.to(d).requires_grad_(do is not None) for t in (q, k, v))
+    bfg = bf.to(d)
+    BA.BitfieldUtils.clear_cache()
+    o = BA.bitfield_attn_func(qg, kg, vg, bfg, softmax_scale=scale)
+    grads = (None, None, None)
+    if do is not None:
+        grads = torch.autograd.grad(o, (qg, kg, vg), do.to(d))
+    _, lse, _ = BA._bitfield_attn_forward(qg.detach(), kg.detach(), vg.detach(), bfg, flags_of(bfg), softmax_scale=scale)
+    torch.cuda.synchronize()
+    S = q.shape[1]
+    return (o.detach().cpu(), lse[:, :, :S].cpu(), *(g.cpu() if g is not None else None for g in grads))
+
+
+def make_inputs(B, S, Hq, Hkv, D, dtype, seed=0, std=0.5):
+    g = torch.Generator().manual_seed(seed)
+    q = (torch.randn(B, S, Hq, D, generator=g) * std).to(dtype)
+    k = (torch.randn(B, S, Hkv, D, generator=g) * std).to(dtype)
+    v = (torch.randn(B, S, Hkv, D, generator=g) * std).to(dtype)
+    do = torch.randn(B, S, Hq, D, generator=g).to(dtype)
+    return q, k, v, do
+
+
+def check_against_oracle(q, k, v, do, bf, scale=None, tight=False):
+    o, lse, dq, dk, dv = run_hip(q, k, v, bf, do, scale)
+    o_ref, lse_ref = O.attention_forward(q, k, v, bf, softmax_scale=scale)
+    gq, gk, gv = O.attention_backward(q, k, v, bf, do, softmax_scale=scale)
+    assert torch.isfinite(o).all()
+    assert (o.float() - o_ref).abs().max().item() <= O_MAX_ABS
+    if tight:  # the reference's own assert_close bar, widened for the bf16 output rounding
+        torch.testing.assert_close(o.float(), o_ref, rtol=1e-2, atol=1e-2)
+    fin = torch.isfinite(lse_ref)
+    assert torch.equal(torch.isfinite(lse), fin)
+    assert (lse[fin] - lse_ref[fin]).abs().max().item() <= 1e-2
+    for got, want in ((dq, gq), (dk, gk), (dv, gv)):
+        assert torch.isfinite(got).all()
+        assert rel_l2(got, want) <= GRAD_REL_L2
+        if tight:
+            torch.testing.assert_close(got.float(), want, rtol=2e-2, atol=2e-2)
+
+
+# ------------------------------------------------------------------ flags and mask
+@pytest.mark.parametrize("size", ["small", "large"])
+def test_mask_kat_of_the_reference(size):
+    bf, expected = reference_mask_kat(size)
+    got = BA.materialize_bitfield_mask(bf.to(dev())).cpu()
+    assert torch.equal(got, expected)
+
+
+@pytest.mark.parametrize("S", [1, 31, 57, 128, 144, 283, 1000])
+@pytest.mark.parametrize("wide", [False, True])
+def test_flags_and_mask_bit_exact_on_irregular_bitfields(S, wide):
+    bf = random_bitfield(3, S, seed=S, pad=min(5, S - 1), wide=wide)
+    bfg = bf.to(dev())
+    assert torch.equal(flags_of(bfg).cpu(), O.tile_flags(bf))
+    assert torch.equal(flags_of(bfg).cpu(), torch.from_numpy(C.tile_flags(bf.numpy())))
+    assert torch.equal(BA.materialize_bitfield_mask(bfg).cpu(), O.materialize_mask(bf))
+
+
+@pytest.mark.parametrize("S", [57, 256, 335, 684, 1024, 2003, 3712])
+def test_flags_rowblock_workloads_of_the_context_parallel_test(S):
+    nn = -(-S // 32)
+    causal = flags_of(torch.full((1, S), (1 << 62) | 1, dtype=torch.int64, device=dev()))[0].cpu()
+    assert [(r > 0).sum().item() for r in causal] == [min(4 * (m + 1), nn) for m in range(causal.shape[0])]
+    dense = flags_of(torch.full((1, S), 1 << 1, dtype=torch.int64, device=dev()))[0].cpu()
+    assert (dense == 2).all()
+
+
+def test_flags_of_a_strided_bitfield_row_view():
+    base = random_bitfield(4, 600, seed=11)
+    big = torch.zeros((4, 1000), dtype=torch.int64)
+    big[:, :600] = base
+    view = big.to(dev())[:, :600]  # row stride 1000
+    assert not view.is_contiguous()
+    assert torch.equal(flags_of(view).cpu(), O.tile_flags(base))
+
+
+@pytest.mark.parametrize("name", ["C1", "C2", "C3", "C4", "C5"])
+def test_flags_bit_exact_on_the_benchmark_workloads(name):
+    bf = W.make_bitfields(name)
+    bfg = bf.to(dev())
+    got = flags_of(bfg)
+    want = O.tile_flags(bfg)  # oracle as torch library ops on the device (4.3e9 cells for C5)
+    assert torch.equal(got, want)
+    if name != "C5":
+        assert torch.equal(got.cpu(), O.tile_flags(bf))
+    if name == "C1":
+        assert [(got == v).sum().item() for v in (0, 1, 2)] == [108, 24, 124]
+
+
+def test_flag_cache_semantics():
+    d = dev()
+    a = random_bitfield(1, 256, 1).to(d)
+    b = random_bitfield(1, 256, 2).to(d)
+    BA.BitfieldUtils.clear_cache()
+    fa = BA.BitfieldUtils.materialize_compressed_mask_from_bitfield_mask(a)
+    assert BA.BitfieldUtils.compressed_mask_cache is fa
+    assert BA.BitfieldUtils.materialize_compressed_mask_from_bitfield_mask(a) is fa  # cached across layers
+    fb = BA.BitfieldUtils.materialize_compressed_mask_from_bitfield_mask(b)  # different mask: never stale
+    assert torch.equal(fb.cpu(), O.tile_flags(b.cpu()))
+    a[0, 5] = 0  # in-place edit bumps the version -> recomputed
+    fa2 = BA.BitfieldUtils.materialize_compressed_mask_from_bitfield_mask(a)
+    assert torch.equal(fa2.cpu(), O.tile_flags(a.cpu()))
+    BA.BitfieldUtils.clear_cache()
+    assert BA.BitfieldUtils.compressed_mask_cache is None
+
+
+# ------------------------------------------------- the reference's fwd/bwd test grids
+@pytest.mark.parametrize("head_dim", [32, 64, 128])
+@pytest.mark.parametrize("seqlen", [57, 128, 144, 256, 283, 512, 1024])
+@pytest.mark.parametrize("batch_size", [1, 4])
+def test_reference_grid_mha_fp16(head_dim, seqlen, batch_size):
+    # tests/test_kernel/test_bitfield_attention.py:113-204 (H = 6, fp16, N(0, 0.5^2))
+    bf, _ = reference_test_bitfield(batch_size, seqlen)
+    q, k, v, do = make_inputs(batch_size, seqlen, 6, 6, head_dim, torch.float16)
+    check_against_oracle(q, k, v, do, bf, tight=True)
+
+
+@pytest.mark.parametrize("head_dim", [32, 64, 128])
+@pytest.mark.parametrize("seqlen", [57, 144, 283, 1024])
+@pytest.mark.parametrize("num_kv_heads", [1, 2, 3])
+def test_reference_grid_gqa_bf16(head_dim, seqlen, num_kv_heads):
+    # tests/test_kernel/test_bitfield_attention.py:207-307 (Hq = 6, bf16)
+    bf, _ = reference_test_bitfield(2, seqlen)
+    q, k, v, do = make_inputs(2, seqlen, 6, num_kv_heads, head_dim, torch.bfloat16)
+    check_against_oracle(q, k, v, do, bf, tight=True)
+
+
+@pytest.mark.parametrize("S,D,Hq,Hkv", [(200, 128, 4, 2), (517, 64, 4, 4), (96, 32, 2, 1)])
+@pytest.mark.parametrize("wide", [False, True])
+def test_irregular_bitfields_with_padding(S, D, Hq, Hkv, wide):
+    bf = random_bitfield(2, S, seed=S + D, pad=9, wide=wide)
+    q, k, v, do = make_inputs(2, S, Hq, Hkv, D, torch.bfloat16, seed=1)
+    o, lse, dq, dk, dv = run_hip(q, k, v, bf, do)
+    # padded rows (bitfield 0): o = 0, lse = -inf, no gradient flows in or out
+    assert (o[:, -9:] == 0).all() and torch.isneginf(lse[:, :, -9:]).all()
+    assert (dq[:, -9:] == 0).all() and (dk[:, -9:] == 0).all() and (dv[:, -9:] == 0).all()
+    check_against_oracle(q, k, v, do, bf)
+
+
+def test_all_text_bitfield_is_causal_attention():
+    # tests/test_shardformer/utils.py:388-391
+    S = 300
+    bf = torch.full((1, S), (1 << 62) | 1, dtype=torch.int64)
+    q, k, v, do = make_inputs(1, S, 4, 4, 64, torch.float16, seed=3)
+    o, *_ = run_hip(q, k, v, bf)
+    want = torch.nn.functional.scaled_dot_product_attention(
+        q.float().transpose(1, 2), k.float().transpose(1, 2), v.float().transpose(1, 2), is_causal=True
+    ).transpose(1, 2)
+    assert (o.float() - want).abs().max().item() <= 5e-3
+
+
+def test_custom_softmax_scale_and_cross_check_with_c_oracle():
+    bf = random_bitfield(1, 150, seed=8)
+    q, k, v, do = make_inputs(1, 150, 2, 1, 32, torch.float16, seed=5)
+    check_against_oracle(q, k, v, do, bf, scale=0.3)
+    o, lse, dq, dk, dv = run_hip(q, k, v, bf, do, scale=0.3)
+    co, clse = C.attn_fwd(q.float().numpy(), k.float().numpy(), v.float().numpy(), bf.numpy(), scale=0.3)
+    assert (o.float() - torch.from_numpy(co)).abs().max().item() <= 5e-3
+    cq, ck, cv = C.attn_bwd(*(x.float().numpy() for x in (q, k, v, do)), clse,
+                            C.delta(co, do.float().numpy()), bf.numpy(), scale=0.3)
+    for got, want in ((dq, cq), (dk, ck), (dv, cv)):
+        assert rel_l2(got, torch.from_numpy(want)) <= 2e-2
+
+
+@pytest.mark.parametrize("D", [16, 40, 80, 96])
+def test_head_dims_between_the_native_ones(D):
+    bf, _ = reference_test_bitfield(1, 144)
+    q, k, v, do = make_inputs(1, 144, 4, 2, D, torch.bfloat16, seed=D)
+    check_against_oracle(q, k, v, do, bf)
+
+
+# ------------------------------------------------------------------------ properties
+def test_gqa_equals_mha_with_repeated_kv_heads_bit_exactly():
+    bf = random_bitfield(2, 400, seed=21)
+    q, k, v, do = make_inputs(2, 400, 8, 2, 128, torch.bfloat16, seed=2)
+    o_g, lse_g, dq_g, dk_g, dv_g = run_hip(q, k, v, bf, do)
+    kr, vr = k.repeat_interleave(4, dim=2), v.repeat_interleave(4, dim=2)
+    o_m, lse_m, dq_m, dk_m, dv_m = run_hip(q, kr, vr, bf, do)
+    assert torch.equal(o_g, o_m) and torch.equal(lse_g, lse_m) and torch.equal(dq_g, dq_m)
+    # dk of a kv head = sum of the dk of its q heads (fp32 sums in another order)
+    assert rel_l2(dk_g, dk_m.float().view(2, 400, 2, 4, 128).sum(3)) <= 1e-2
+    assert rel_l2(dv_g, dv_m.float().view(2, 400, 2, 4, 128).sum(3)) <= 1e-2
+
+
+def test_masked_keys_do_not_influence_anything_bit_exactly():
+    S = 384
+    bf = torch.full((1, S), (1 << 62) | 1 | 2, dtype=torch.int64)
+    bf[0, 100:228] = 4  # a modality the text does not carry: invisible to text, sees only itself
+    q, k, v, do = make_inputs(1, S, 2, 2, 64, torch.bfloat16, seed=4)
+    o1, lse1, dq1, dk1, dv1 = run_hip(q, k, v, bf, do)
+    k2, v2 = k.clone(), v.clone()
+    k2[0, 100:228] = 7.0
+    v2[0, 100:228] = -9.0
+    o2, lse2, dq2, dk2, dv2 = run_hip(q, k2, v2, bf, do)
+    text = torch.ones(S, dtype=torch.bool)
+    text[100:228] = False
+    assert torch.equal(o1[0, text], o2[0, text]) and torch.equal(lse1[0][:, text], lse2[0][:, text])
+    assert torch.equal(dq1[0, text], dq2[0, text])
+    assert torch.equal(dk1[0, text], dk2[0, text]) and torch.equal(dv1[0, text], dv2[0, text])
+
+
+def test_output_is_linear_in_v_and_runs_are_deterministic():
+    bf = random_bitfield(1, 500, seed=31)
+    q, k, v, do = make_inputs(1, 500, 4, 1, 128, torch.bfloat16, seed=6)
+    a = run_hip(q, k, v, bf, do)
+    b = run_hip(q, k, v, bf, do)
+    for x, y in zip(a, b):
+        assert torch.equal(x, y)  # no atomics anywhere: bit-identical reruns
+    o2, lse2, *_ = run_hip(q, k, v * 2, bf)
+    assert torch.equal(o2, a[0] * 2) and torch.equal(lse2, a[1])  # power-of-two scaling is exact
+
+
+def test_strided_views_as_the_hf_adapter_passes_them():
+    class M(torch.nn.Module):
+        pass
+
+    B, H, Hkv, S, D = 2, 4, 2, 200, 64
+    bf = random_bitfield(B, S, seed=41)
+    g = torch.Generator().manual_seed(0)
+    q = (torch.randn(B, H, S, D, generator=g) * 0.5).bfloat16()  # (B, H, S, D) as HF modules hold them
+    k = (torch.randn(B, Hkv, S, D, generator=g) * 0.5).bfloat16()
+    v = (torch.randn(B, Hkv, S, D, generator=g) * 0.5).bfloat16()
+    BA.BitfieldUtils.clear_cache()
+    out, w = interface.bitfield_attention_forward(M(), q.to(dev()), k.to(dev()), v.to(dev()), bf.to(dev()),
+                                                  scaling=123.0)  # ignored, as in the reference
+    assert w is None and out.shape == (B, S, H, D)
+    o_ref, _ = O.attention_forward(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), bf)
+    assert (out.float().cpu() - o_ref).abs().max().item() <= O_MAX_ABS
+
+
+def test_backward_accumulates_into_caller_buffers():
+    # the private backward ADDS into fp32 dq/dk/dv (reference :1248-1250 zeroes them first)
+    d = dev()
+    bf = random_bitfield(1, 256, seed=51)
+    q, k, v, do = (t.to(d) for t in make_inputs(1, 256, 2, 2, 64, torch.bfloat16, seed=7))
+    bfg = bf.to(d)
+    flags = flags_of(bfg)
+    o, lse, sc = BA._bitfield_attn_forward(q, k, v, bfg, flags)
+    assert sc == 1 / math.sqrt(64) and lse.shape == (1, 2, 256) and lse.dtype == torch.float32
+    z = [torch.zeros_like(t, dtype=torch.float32) for t in (q, k, v)]
+    BA._bitfield_attn_backward(do, q, k, v, o, bfg, flags, lse, *z)
+    ones = [torch.ones_like(t, dtype=torch.float32) for t in (q, k, v)]
+    BA._bitfield_attn_backward(do, q, k, v, o, bfg, flags, lse, *ones)
+    for a, b in zip(z, ones):
+        assert torch.allclose(a + 1, b, atol=1e-6)
+    with pytest.raises(NotImplementedError):
+        BA._bitfield_attn_forward(q, k, v, bfg, flags, bias=torch.zeros(1, 2, 1, 256, device=d))
+    with pytest.raises(NotImplementedError):
+        BA._bitfield_attn_forward(q, k, v, bfg, flags, offsets_q=torch.arange(256, device=d))
+
+
+# -------------------------------------------------- the five benchmark configurations
+def _oracle_on_device(q, k, v, do, bf, row_chunk):
+    o, lse = O.attention_forward(q, k, v, bf, row_chunk=row_chunk)
+    grads = O.attention_backward(q, k, v, bf, do, row_chunk=row_chunk) if do is not None else (None,) * 3
+    return (o, lse, *grads)
+
+
+def test_config1_plumbing_fp32_reference_on_cpu():
+    # forward only, fp32 N(0,1) inputs; the oracle runs in fp32 on the CPU, the kernels get the
+    # same values rounded to their 16-bit input types (the oracle consumes the rounded values)
+    q, k, v, _ = W.make_tensors("C1")
+    bf = W.make_bitfields("C1")
+    for dt in (torch.float16, torch.bfloat16):
+        qr, kr, vr = (t.to(dt) for t in (q, k, v))
+        o, lse, *_ = run_hip(qr, kr, vr, bf)
+        o_ref, lse_ref = O.attention_forward(qr, kr, vr, bf)
+        assert (o.float() - o_ref).abs().max().item() <= O_MAX_ABS
+        assert (lse - lse_ref).abs().max().item() <= 1e-2
+        assert (o.float() - O.attention_sdpa(qr.float(), kr.float(), vr.float(), bf)).abs().max().item() <= O_MAX_ABS
+
+
+@pytest.mark.parametrize("name,row_chunk", [("C2", 1024), ("C3", 1024), ("C4", 1024), ("C5", 256)])
+def test_full_size_configs_against_fp32_library_math(name, row_chunk):
+    d = dev()
+    q, k, v, do = (t.to(d) for t in W.make_tensors(name))
+    bf = W.make_bitfields(name).to(d)
+    w = W.WORKLOADS[name]
+    qg, kg, vg = (t.requires_grad_(True) for t in (q, k, v))
+    BA.BitfieldUtils.clear_cache()
+    o = BA.bitfield_attn_func(qg, kg, vg, bf)
+    dq, dk, dv = torch.autograd.grad(o, (qg, kg, vg), do)
+    _, lse, _ = BA._bitfield_attn_forward(q.detach(), k.detach(), v.detach(), bf, flags_of(bf))
+    o = o.detach()
+    # fp32 oracle on the device, one KV group at a time to bound memory
+    G = w.Hq // w.Hkv
+    worst_o, worst_lse = 0.0, 0.0
+    num = {"dq": 0.0, "dk": 0.0, "dv": 0.0}
+    den = {"dq": 0.0, "dk": 0.0, "dv": 0.0}
+    groups = range(w.Hkv) if name != "C5" else (0, w.Hkv - 1)  # C5: two of the eight groups
+    for hk in groups:
+        hs = slice(hk * G, (hk + 1) * G)
+        ks = slice(hk, hk + 1)
+        o_r, lse_r, gq, gk, gv = _oracle_on_device(
+            q.detach()[:, :, hs], k.detach()[:, :, ks], v.detach()[:, :, ks], do[:, :, hs], bf, row_chunk)
+        worst_o = max(worst_o, (o[:, :, hs].float() - o_r).abs().max().item())
+        worst_lse = max(worst_lse, (lse[:, hs, : w.S] - lse_r).abs().max().item())
+        for key, got, want in (("dq", dq[:, :, hs], gq), ("dk", dk[:, :, ks], gk), ("dv", dv[:, :, ks], gv)):
+            num[key] += float((got.double() - want.double()).pow(2).sum())
+            den[key] += float(want.double().pow(2).sum())
+    assert worst_o <= O_MAX_ABS, worst_o
+    assert worst_lse <= 1e-2, worst_lse
+    for key in num:
+        assert math.sqrt(num[key] / den[key]) <= GRAD_REL_L2, (key, math.sqrt(num[key] / den[key]))

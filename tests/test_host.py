@@ -1,0 +1,168 @@
+"""CPU-only checks of the host side: the C-ABI library loads and exports what the header
+declares, host logic mirrors the reference's interface, the product path refuses to run
+without the GPU / the HIP library (no fallback), and the synthetic workloads are the ones
+the baseline document describes."""
+
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+from cornstarch_amd import workloads as W
+from cornstarch_amd.kernel import _bam_hip
+from cornstarch_amd.kernel import attention as sibling
+from cornstarch_amd.kernel import bitfield_attention as BA
+from cornstarch_amd.kernel import interface
+from oracle import bam_oracle as O
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "bam_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(bam_[a-z_0-9]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    if not os.path.exists(_bam_hip.LIB_PATH):
+        from cornstarch_amd import build
+
+        build.build_library(force=True)
+    lib = ctypes.CDLL(_bam_hip.LIB_PATH)
+    names = _declared_symbols()
+    assert {"bam_tile_flags", "bam_fwd", "bam_bwd", "bam_bwd_preprocess", "bam_materialize_mask",
+            "bam_bwd_dkdv", "bam_bwd_dq", "bam_last_error", "bam_abi_version"} <= set(names)
+    for n in names:
+        assert hasattr(lib, n), f"{n} is declared in include/bam_hip.h but not exported"
+    assert _bam_hip.load().bam_abi_version() == _bam_hip.ABI_VERSION
+    # the binding's prototypes cover every compute entry point of the header
+    assert set(_bam_hip.SIGNATURES) == set(names) - {"bam_last_error", "bam_abi_version"}
+
+
+def test_abi_rejects_bad_arguments_without_touching_the_gpu():
+    lib = _bam_hip.load()
+    # null pointers / unsupported head dim are refused before any HIP call
+    rc = lib.bam_tile_flags(None, 0, None, 0, 0, 1, 128, None)
+    assert rc == -1 and b"null" in lib.bam_last_error()
+    args = [ctypes.c_void_p(16)] * 7 + [8] * 15 + [1, 128, 4, 4, 48] + [0.125, 1, None]
+    rc = lib.bam_fwd(*args)
+    assert rc == -2 and b"head dimension 48" in lib.bam_last_error()
+    args = [ctypes.c_void_p(16)] * 7 + [8] * 15 + [1, 128, 6, 4, 64] + [0.125, 1, None]
+    assert lib.bam_fwd(*args) == -1 and b"multiple of Hkv" in lib.bam_last_error()
+    args = [ctypes.c_void_p(8)] + [ctypes.c_void_p(16)] * 6 + [8] * 15 + [1, 128, 4, 4, 64] + [0.125, 1, None]
+    assert lib.bam_fwd(*args) == -1 and b"16-byte aligned" in lib.bam_last_error()
+    args = [ctypes.c_void_p(16)] * 7 + [8] * 15 + [1, 128, 4, 4, 64] + [-1.0, 1, None]
+    assert lib.bam_fwd(*args) == -1 and b"scale" in lib.bam_last_error()
+    with pytest.raises(_bam_hip.BamError):
+        _bam_hip.call("bam_materialize_mask", None, 0, None, 1, 8, None)
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    monkeypatch.setattr(_bam_hip, "_lib", None)
+    monkeypatch.setattr(_bam_hip, "LIB_PATH", "/nonexistent/libbam_hip.so")
+    with pytest.raises(_bam_hip.BamError, match="no fallback"):
+        _bam_hip.load()
+
+
+def test_product_path_has_no_cpu_fallback():
+    q = torch.randn(1, 64, 2, 32, dtype=torch.bfloat16)
+    bf = torch.full((1, 64), (1 << 62) | 1, dtype=torch.int64)
+    with pytest.raises(AssertionError):
+        BA.bitfield_attn_func(q, q, q, bf)
+    with pytest.raises(AssertionError):
+        BA.BitfieldUtils.materialize_compressed_mask_from_bitfield_mask(bf)
+    flags = torch.zeros((1, 1, 2), dtype=torch.int8)
+    with pytest.raises(AssertionError, match="fp16 and bf16"):
+        BA._bitfield_attn_forward(q.float(), q.float(), q.float(), bf, flags)
+    with pytest.raises(AssertionError, match="up to 128"):
+        big = torch.randn(1, 64, 2, 256, dtype=torch.bfloat16)
+        BA._bitfield_attn_forward(big, big, big, bf, flags)
+
+
+def test_module_constants_and_signatures_match_the_reference_interface():
+    import inspect
+
+    assert (BA.BLOCK_M, BA.BLOCK_N, BA.NUM_TOKENS_TO_COMPUTE_PER_BLOCK) == (128, 32, 4096)
+    assert (sibling.BLOCK_M, sibling.BLOCK_N) == (128, 32)
+    assert list(inspect.signature(BA.bitfield_attn_func).parameters) == [
+        "q", "k", "v", "bitfield_mask", "bias", "softmax_scale"]
+    assert list(inspect.signature(BA._bitfield_attn_forward).parameters) == [
+        "q", "k", "v", "bitfield_mask", "compressed_mask", "offsets_q", "offsets_k", "bias", "softmax_scale"]
+    assert list(inspect.signature(BA._bitfield_attn_backward).parameters) == [
+        "do", "q", "k", "v", "o", "bitfield_mask", "compressed_mask", "lse", "dq", "dk", "dv",
+        "offsets_q", "offsets_k", "bias", "softmax_scale"]
+    assert list(inspect.signature(interface.bitfield_attention_forward).parameters) == [
+        "module", "query", "key", "value", "attention_mask", "dropout", "scaling", "sliding_window", "softcap",
+        "kwargs"]
+    assert hasattr(BA.BitfieldUtils, "compressed_mask_cache") and BA.BitfieldUtils.compressed_mask_cache is None
+    BA.BitfieldUtils.clear_cache()
+
+
+def test_create_bitfield_attention_mask_format():
+    ids = torch.tensor([[5, 9, 9, 7, 3, 7, 1]])
+    got = interface.create_bitfield_attention_mask(ids, {"vision": 9, "audio": 7})
+    text = (1 << 62) | 1 | 2 | 4
+    assert got.tolist() == [[text, 2, 2, 4, text, 4, text]] and got.dtype == torch.int64
+    assert interface.create_bitfield_attention_mask(ids).tolist() == [[(1 << 62) | 1] * 7]
+
+
+def test_adapter_requires_int64_mask():
+    class M(torch.nn.Module):
+        pass
+
+    q = torch.randn(1, 2, 8, 32)
+    with pytest.raises(AssertionError, match="int64"):
+        interface.bitfield_attention_forward(M(), q, q, q, torch.ones(1, 8, dtype=torch.bool))
+    # single-token decode of an eval-mode module never reaches the bitfield kernel
+    m = M().eval()
+    q1 = torch.randn(1, 4, 1, 32)
+    kv = torch.randn(1, 2, 9, 32)
+    out, w = interface.bitfield_attention_forward(m, q1, kv, kv, None)
+    assert out.shape == (1, 1, 4, 32) and w is None
+    want = torch.softmax(
+        (q1 @ kv.repeat_interleave(2, 1).transpose(-1, -2)) / 32**0.5, -1) @ kv.repeat_interleave(2, 1)
+    assert torch.allclose(out, want.transpose(1, 2), atol=1e-5)
+
+
+# histogram / pair counts of the synthetic workloads quoted by the baseline document
+EXPECTED = {
+    "C1": (557440, [108, 24, 124]),
+    "C2": (24536064, [9685, 1334, 5365]),
+    "C3": (91592220, [41456, 2998, 21082]),
+    "C4": (38492218, [20466, 5287, 7015]),
+}
+
+
+@pytest.mark.parametrize("name", sorted(EXPECTED))
+def test_workload_generator_statistics(name):
+    bf = W.make_bitfields(name)
+    w = W.WORKLOADS[name]
+    assert bf.shape == (w.B, w.S) and bf.dtype == torch.int64
+    pairs, hist = EXPECTED[name]
+    assert O.unmasked_pairs(bf) == pairs
+    flags = O.tile_flags(bf)
+    assert [(flags == v).sum().item() for v in (0, 1, 2)] == hist
+    assert W.flops(name, pairs) == (4 * w.D * w.Hq * pairs, 10 * w.D * w.Hq * pairs)
+
+
+def test_workload_tensors_are_seeded_and_sliceable():
+    q, k, v, do = W.make_tensors("C1")
+    q2, *_ = W.make_tensors("C1")
+    assert q.dtype == torch.float32 and torch.equal(q, q2) and q.shape == (1, 1024, 8, 64)
+    qa, ka, va, doa = W.make_tensors("C4", heads=(2, 4))
+    qf, kf, vf, dof = W.make_tensors("C4")
+    assert torch.equal(qa, qf[:, :, 2:4]) and torch.equal(ka, kf[:, :, 2:4]) and torch.equal(doa, dof[:, :, 2:4])
+    assert qf.dtype == torch.bfloat16
+
+
+def test_c5_layout_shape():
+    bf = W.make_bitfields("C5")
+    assert bf.shape == (1, 65536)
+    text = W.text_bits(range(1, 17))
+    seg = bf[0] != text
+    # 200 segments of 16..512 tokens
+    assert 200 * 16 <= int(seg.sum()) <= 200 * 512
+    assert set(bf[0][seg].tolist()) <= {1 << b for b in range(1, 17)}
