@@ -27,6 +27,8 @@ int check_half_tensor(const char* name, const void* ptr, int64_t sb, int64_t ss,
     if ((sb % 8) || (ss % 8) || (sh % 8))
         return fail(BAM_ERR_INVALID_ARGUMENT, "%s: strides (%lld, %lld, %lld) must be multiples of 8 elements", name,
                     (long long)sb, (long long)ss, (long long)sh);
+    if (ss < 0 || ss >= (1ll << 24))
+        return fail(BAM_ERR_UNSUPPORTED, "%s: sequence stride %lld is outside [0, 2^24) elements", name, (long long)ss);
     return BAM_OK;
 }
 

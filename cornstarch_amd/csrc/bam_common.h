@@ -28,28 +28,37 @@ __device__ __forceinline__ bool allow_rule(int64_t qf, int64_t kf, int64_t i, in
     return text ? (i >= j && (qb & kb) != 0) : (qb == kb && qb != 0);
 }
 
-// Per-query constants of the rule, split in 32-bit halves so that the per-pair test is
-// three 32-bit logic ops, two compares and a select:
-//   text query     : allow = ((q & k) != 0) && kpos <= qpos
-//   modality query : allow = ((q ^ k) == 0) && q != 0
+// Per-query constants of the rule, split in 32-bit halves and arranged so that the
+// per-pair test is branch free and identical for text and modality queries:
+//   v = ((k & a) ^ x)  over both halves
+//   text query     : a = q,  x = 0  -> v = q & k ; allowed iff v != 0 and kpos <= qpos
+//   modality query : a = ~0, x = q  -> v = q ^ k ; allowed iff v == 0 and q != 0
+// `lim` folds the position test and the q != 0 test into one compare (kpos <= lim).
 struct QueryBits {
-    unsigned lo, hi;  // modality bits (bit 62/63 stripped)
-    int lim;          // kpos <= lim must hold: qpos for text, INT_MAX / -1 for modality rows
+    unsigned a_lo, a_hi, x_lo, x_hi;
+    int lim;    // qpos for text rows, INT_MAX for live modality rows, -1 for rows that see nothing
     bool text;
 };
 
 __device__ __forceinline__ QueryBits make_query_bits(int64_t qf, int qpos) {
+    const unsigned lo = (unsigned)(qf & 0xFFFFFFFFll);
+    const unsigned hi = ((unsigned)((uint64_t)qf >> 32)) & HI_MODALITY_MASK;
     QueryBits q;
-    q.lo = (unsigned)(qf & 0xFFFFFFFFll);
-    q.hi = ((unsigned)((uint64_t)qf >> 32)) & HI_MODALITY_MASK;
-    q.text = (q.lo & 1u) != 0;
-    q.lim = q.text ? qpos : (((q.lo | q.hi) != 0) ? 0x7FFFFFFF : -1);
+    q.text = (lo & 1u) != 0;
+    q.a_lo = q.text ? lo : 0xFFFFFFFFu;
+    q.a_hi = q.text ? hi : 0xFFFFFFFFu;
+    q.x_lo = q.text ? 0u : lo;
+    q.x_hi = q.text ? 0u : hi;
+    q.lim = q.text ? qpos : (((lo | hi) != 0) ? 0x7FFFFFFF : -1);
     return q;
 }
 
+// klo/khi: modality bits of the key (bits 62/63 stripped), kpos: its position.
 __device__ __forceinline__ bool allow_pair(const QueryBits& q, unsigned klo, unsigned khi, int kpos) {
-    const unsigned r = q.text ? ((q.lo & klo) | (q.hi & khi)) : ((q.lo ^ klo) | (q.hi ^ khi));
-    return ((r != 0) == q.text) && (kpos <= q.lim);
+    const unsigned v = ((klo & q.a_lo) ^ q.x_lo) | ((khi & q.a_hi) ^ q.x_hi);
+    const bool nz = v != 0u;
+    const bool pos_ok = kpos <= q.lim;
+    return (nz == q.text) & pos_ok;
 }
 
 // ---------------------------------------------------------------------------------
@@ -175,6 +184,22 @@ __device__ __forceinline__ float half_swap_sum(float x) {
     float a, b;
     half_swap(x, a, b);
     return a + b;
+}
+
+// Scheduling hint: interleave `n` MFMAs with the LDS reads that feed them so that reads run
+// `ahead` operands in front of their MFMA (reads_per_op LDS instructions per operand).  Must
+// follow, in the same basic block, the n operand reads and the n MFMAs it orders.
+template <int N, int AHEAD, int READS_PER_OP>
+__device__ __forceinline__ void sched_pipeline_mfma_lds() {
+#pragma unroll
+    for (int i = 0; i < AHEAD; ++i) __builtin_amdgcn_sched_group_barrier(0x100, READS_PER_OP, 0);
+#pragma unroll
+    for (int i = 0; i < N - AHEAD; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, READS_PER_OP, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < AHEAD; ++i) __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
 }
 
 // Workgroups are dealt round-robin to the 8 XCDs.  Map a linear block id onto

@@ -6,37 +6,55 @@
 
 namespace bam {
 
-// ROWS x D tile of 2-byte elements moved by THREADS threads, 16 bytes per access.  `load`
-// only issues the global reads (rows past `S` read zeros); `store` writes the registers
-// into the swizzled LDS tile, so the two can be separated by a whole tile of MFMA work.
+// ROWS x D tile of 2-byte elements copied global -> LDS by THREADS threads, 16 bytes per lane.
+// Full tiles use the direct global-to-LDS load (no staging registers, no LDS write
+// instructions): a wave's 64 lanes fill 64 consecutive chunk slots of the LDS tile, so the
+// XOR swizzle is applied on the SOURCE side -- lane `id` fetches the chunk that belongs in
+// slot `id`.  `setup` fixes those source offsets once per kernel.  The copy is asynchronous:
+// the caller waits with wait_async() and a workgroup barrier before anyone reads the tile.
+// The last, ragged tile of a sequence takes the synchronous path, which zero-fills the rows
+// past the end.  Row strides are limited to 2^24 elements by the host checks, so the
+// offsets fit 32 bits.
 template <int D, int ROWS, int THREADS>
 struct TileStage {
     static constexpr int NCH = D / 8;
     static constexpr int CHUNKS = ROWS * NCH;
     static constexpr int CPT = (CHUNKS + THREADS - 1) / THREADS;
-    u32x4 r[CPT];
+    static constexpr bool EXACT = (CHUNKS % THREADS) == 0;
+    unsigned goff[CPT];
 
-    __device__ __forceinline__ void load(const char* base, int64_t row_stride_bytes, int row0, int S, int tid) {
+    __device__ __forceinline__ void setup(int64_t row_stride_bytes, int tid) {
 #pragma unroll
         for (int i = 0; i < CPT; ++i) {
             const int id = tid + THREADS * i;
-            const int row = id / NCH, c = id % NCH;
-            const int grow = row0 + row;
-            u32x4 z = {0u, 0u, 0u, 0u};
-            if ((CHUNKS % THREADS == 0 || id < CHUNKS) && grow < S)
-                z = *(const u32x4*)(base + (int64_t)grow * row_stride_bytes + c * 16);
-            r[i] = z;
+            const int row = id / NCH, pc = id % NCH;
+            goff[i] = (unsigned)(row * row_stride_bytes + (pc ^ swz<D>(row)) * 16);
         }
     }
-    __device__ __forceinline__ void store(u32x4* tile, int tid) const {
+    // tile_base: first row of the tile in global memory; rows_valid: rows of it inside the sequence
+    __device__ __forceinline__ void load(const char* tile_base, u32x4* tile, int rows_valid, int tid) const {
+        typedef __attribute__((address_space(1))) const void* gptr;
+        typedef __attribute__((address_space(3))) void* lptr;
+        if (rows_valid >= ROWS) {
 #pragma unroll
-        for (int i = 0; i < CPT; ++i) {
-            const int id = tid + THREADS * i;
-            const int row = id / NCH, c = id % NCH;
-            if (CHUNKS % THREADS == 0 || id < CHUNKS) tile[chunk_slot<D>(row, c)] = r[i];
+            for (int i = 0; i < CPT; ++i)
+                if (EXACT || (tid & ~63) + THREADS * i < CHUNKS)  // wave-uniform
+                    __builtin_amdgcn_global_load_lds((gptr)(tile_base + goff[i]),
+                                                     (lptr)(tile + THREADS * i + (tid & ~63)), 16, 0, 0);
+        } else {
+#pragma unroll
+            for (int i = 0; i < CPT; ++i) {
+                const int id = tid + THREADS * i;
+                u32x4 z = {0u, 0u, 0u, 0u};
+                if ((EXACT || id < CHUNKS) && id / NCH < rows_valid) z = *(const u32x4*)(tile_base + goff[i]);
+                if (EXACT || id < CHUNKS) tile[id] = z;
+            }
         }
     }
 };
+
+// All direct global-to-LDS copies this wave has issued have landed (pair with a barrier).
+__device__ __forceinline__ void wait_async() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
 // List, in ascending order, the 64-key tiles a 128-row query block has to visit.
 // entry = (tile << 2) | cls ; cls 1: evaluate the mask, cls 2: every pair allowed.

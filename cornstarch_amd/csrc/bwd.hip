@@ -46,29 +46,39 @@ __global__ __launch_bounds__(256) void bwd_preprocess_kernel(const AttnParams p)
 }
 
 // ---------------------------------------------------------------------------------------
-// dK, dV.  Wave w owns keys [32w, 32w+32) of the 128-key tile: K and V of those keys stay in
-// registers as MFMA B operands for the whole kernel, dK^T and dV^T (d x keys) stay in
-// accumulators.  Query rows arrive in 32-row tiles of Q and dO through LDS (double buffered).
+// dK, dV.  One workgroup = one 128-key tile of one (batch, kv head), 8 waves: wave w owns keys
+// [32 (w & 3), +32) and works on query rows [32 (w >> 2), +32) of every 64-row tile of Q / dO
+// that streams through LDS (double buffered), so each SIMD holds two waves whose MFMA and
+// softmax phases interleave.  K and V of the tile sit in LDS for the whole kernel and are
+// read as MFMA B operands; dK^T and dV^T (d x keys) stay in accumulators.
 // With S = Q K^T computed as queries x keys, a lane of the C fragment owns ONE key and 16
 // query rows, so P and dS feed dV^T = dO^T P and dK^T = Q^T dS as B operands from registers;
 // Q^T and dO^T come from the transposing LDS read of the same row-major tiles.
-constexpr int DKDV_QT = 32;
-constexpr int DKDV_THREADS = 256;
+// The two waves that share a key group hold partial sums; they add them to the caller's
+// buffers one after the other (workgroup barrier in between), so the result stays
+// deterministic and atomic free.
+constexpr int DKDV_QT = 64;
+constexpr int DKDV_THREADS = 512;
 
 template <typename T, int D>
-__global__ __launch_bounds__(DKDV_THREADS, 1) void bwd_dkdv_kernel(const AttnParams p) {
+__global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnParams p) {
     constexpr int NCH = D / 8, KK = D / 16, DB = D / 32;
+    __shared__ u32x4 sK[128 * NCH];
+    __shared__ u32x4 sV[128 * NCH];
     __shared__ u32x4 sQ[2][DKDV_QT * NCH];
     __shared__ u32x4 sDO[2][DKDV_QT * NCH];
     __shared__ __attribute__((aligned(16))) float sLse[2][DKDV_QT];
     __shared__ __attribute__((aligned(16))) float sDelta[2][DKDV_QT];
-    __shared__ __attribute__((aligned(16))) unsigned sQlo[2][DKDV_QT];
-    __shared__ __attribute__((aligned(16))) unsigned sQhi[2][DKDV_QT];
+    __shared__ __attribute__((aligned(16))) unsigned sQalo[2][DKDV_QT];
+    __shared__ __attribute__((aligned(16))) unsigned sQahi[2][DKDV_QT];
+    __shared__ __attribute__((aligned(16))) unsigned sQxlo[2][DKDV_QT];
+    __shared__ __attribute__((aligned(16))) unsigned sQxhi[2][DKDV_QT];
     __shared__ __attribute__((aligned(16))) int sQlim[2][DKDV_QT];
-    __shared__ int sList[MAX_LIST];
+    __shared__ int sList[MAX_LIST / 2];
     __shared__ int sCount;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int kg = wave & 3, st = wave >> 2;
     const int hi = lane >> 5, l32 = lane & 31, half16 = (lane >> 4) & 1;
     const int S = p.S;
     const int G = p.Hq / p.Hkv;
@@ -83,24 +93,18 @@ __global__ __launch_bounds__(DKDV_THREADS, 1) void bwd_dkdv_kernel(const AttnPar
         build_query_block_list(p.flags + (int64_t)b * p.flags_sb, p.flags_sm, p.num_m, p.num_n, nt, lane, sList,
                                &sCount);
 
-    // ---- per-lane key state ---------------------------------------------------------------
-    const int key = nt * 128 + wave * 32 + l32;
-    const bool kvalid = key < S;
-    u32x4 kreg[KK], vreg[KK];
+    // ---- K, V of the tile -> LDS (once) ---------------------------------------------------
     {
-        const char* kp = (const char*)p.k.ptr + 2 * ((int64_t)b * p.k.sb + (int64_t)key * p.k.ss + (int64_t)hk * p.k.sh);
-        const char* vp = (const char*)p.v.ptr + 2 * ((int64_t)b * p.v.sb + (int64_t)key * p.v.ss + (int64_t)hk * p.v.sh);
-#pragma unroll
-        for (int kk = 0; kk < KK; ++kk) {
-            u32x4 zk = {0u, 0u, 0u, 0u}, zv = {0u, 0u, 0u, 0u};
-            if (kvalid) {
-                zk = *(const u32x4*)(kp + (16 * kk + 8 * hi) * 2);
-                zv = *(const u32x4*)(vp + (16 * kk + 8 * hi) * 2);
-            }
-            kreg[kk] = zk;
-            vreg[kk] = zv;
-        }
+        TileStage<D, 128, DKDV_THREADS> stK, stV;
+        stK.setup(2 * p.k.ss, tid);
+        stV.setup(2 * p.v.ss, tid);
+        const char* kb = (const char*)p.k.ptr + 2 * ((int64_t)b * p.k.sb + (int64_t)hk * p.k.sh + (int64_t)nt * 128 * p.k.ss);
+        const char* vb = (const char*)p.v.ptr + 2 * ((int64_t)b * p.v.sb + (int64_t)hk * p.v.sh + (int64_t)nt * 128 * p.v.ss);
+        stK.load(kb, sK, S - nt * 128, tid);
+        stV.load(vb, sV, S - nt * 128, tid);
     }
+    const int key = nt * 128 + kg * 32 + l32;
+    const bool kvalid = key < S;
     const int64_t kf = kvalid ? p.bf[(int64_t)b * p.bf_sb + key] : 0;
     const unsigned klo = (unsigned)(kf & 0xFFFFFFFFll);
     const unsigned khi = ((unsigned)((uint64_t)kf >> 32)) & HI_MODALITY_MASK;
@@ -113,24 +117,28 @@ __global__ __launch_bounds__(DKDV_THREADS, 1) void bwd_dkdv_kernel(const AttnPar
             dk[db][i] = 0.f;
             dv[db][i] = 0.f;
         }
+    f32x16 zero16;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) zero16[i] = 0.f;
     const float c2 = p.scale * LOG2E;
     const int64_t* bfrow = p.bf + (int64_t)b * p.bf_sb;
 
     TileStage<D, DKDV_QT, DKDV_THREADS> stQ, stDO;
+    stQ.setup(2 * p.q.ss, tid);
+    stDO.setup(2 * p.dout.ss, tid);
     float lse_stage = 0.f, delta_stage = 0.f;
     int64_t qf_stage = 0;
 
-    // iteration `it` -> (q head of the group, list entry, 32-row sub block)
-    auto stage_load = [&](int it, int n) {
-        const int g = it / (4 * n);
-        const int rem = it - g * 4 * n;
-        const int entry = sList[rem >> 2];
-        const int row0 = (entry >> 8) * BLOCK_M + (rem & 3) * DKDV_QT;
+    // iteration `it` -> (q head of the group, list entry, 64-row half of the 128-row block)
+    auto tile_row0 = [&](int rem) { return (sList[rem >> 1] >> 8) * BLOCK_M + (rem & 1) * DKDV_QT; };
+    auto stage_load = [&](int it, int n, int buf) {
+        const int g = it / (2 * n);
+        const int row0 = tile_row0(it - g * 2 * n);
         const int h = hk * G + g;
         const char* qbase = (const char*)p.q.ptr + 2 * ((int64_t)b * p.q.sb + (int64_t)h * p.q.sh);
         const char* gbase = (const char*)p.dout.ptr + 2 * ((int64_t)b * p.dout.sb + (int64_t)h * p.dout.sh);
-        stQ.load(qbase, 2 * p.q.ss, row0, S, tid);
-        stDO.load(gbase, 2 * p.dout.ss, row0, S, tid);
+        stQ.load(qbase + (int64_t)row0 * 2 * p.q.ss, sQ[buf], S - row0, tid);
+        stDO.load(gbase + (int64_t)row0 * 2 * p.dout.ss, sDO[buf], S - row0, tid);
         if (tid < DKDV_QT) {
             const int r = row0 + tid;
             const bool ok = r < S;
@@ -138,85 +146,92 @@ __global__ __launch_bounds__(DKDV_THREADS, 1) void bwd_dkdv_kernel(const AttnPar
             const float l = ok ? p.lse[off] : -INFINITY;
             // rows past the end, and rows that allow no key (lse = -inf), must give P = 0
             lse_stage = (l == -INFINITY) ? INFINITY : l * LOG2E;
-            delta_stage = ok ? p.delta[off] : 0.f;
+            delta_stage = ok ? p.delta[off] * p.scale : 0.f;  // pre-scaled: dS = P (dP*scale - delta*scale)
             qf_stage = ok ? bfrow[r] : 0;
         }
     };
     auto stage_store = [&](int it, int n, int buf) {
-        stQ.store(sQ[buf], tid);
-        stDO.store(sDO[buf], tid);
         if (tid < DKDV_QT) {
-            const int rem = it % (4 * n);
-            const int row0 = (sList[rem >> 2] >> 8) * BLOCK_M + (rem & 3) * DKDV_QT;
-            const QueryBits qb = make_query_bits(qf_stage, row0 + tid);
+            const QueryBits qb = make_query_bits(qf_stage, tile_row0(it % (2 * n)) + tid);
             sLse[buf][tid] = lse_stage;
             sDelta[buf][tid] = delta_stage;
-            sQlo[buf][tid] = qb.lo;
-            sQhi[buf][tid] = qb.hi;
+            sQalo[buf][tid] = qb.a_lo;
+            sQahi[buf][tid] = qb.a_hi;
+            sQxlo[buf][tid] = qb.x_lo;
+            sQxhi[buf][tid] = qb.x_hi;
             sQlim[buf][tid] = qb.lim;
         }
     };
 
     __syncthreads();
     const int n = sCount;
-    const int total = n * 4 * G;
+    const int total = n * 2 * G;
     if (total > 0) {
-        stage_load(0, n);
+        stage_load(0, n, 0);
         stage_store(0, n, 0);
+        wait_async();
         __syncthreads();
+        const int qr = 32 * st;  // this wave's rows inside the 64-row tile
         for (int it = 0; it < total; ++it) {
             const int cur = it & 1;
             const bool more = it + 1 < total;
-            if (more) stage_load(it + 1, n);
+            if (more) stage_load(it + 1, n, cur ^ 1);
 
-            const int rem = it % (4 * n);
-            const int entry = sList[rem >> 2];
-            const int cls = (entry >> (2 * wave)) & 3;  // this wave's own 128x32 flag
+            const int entry = sList[(it % (2 * n)) >> 1];
+            const int cls = (entry >> (2 * kg)) & 3;  // this wave's own 128x32 flag
             if (cls != 0) {
-                // ---- S = Q K^T and dP = dO V^T : 32 queries x 32 keys ---------------------
+                // ---- S = Q K^T and dP = dO V^T : 32 queries x 32 keys; both operands of every MFMA
+                // come from LDS and are requested a few MFMAs ahead of their use
                 f32x16 s, dp;
+                {
+                    u32x4 aq[KK], ag[KK], bk[KK], bv[KK];
 #pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    s[i] = 0.f;
-                    dp[i] = 0.f;
-                }
+                    for (int kk = 0; kk < KK; ++kk) {
+                        aq[kk] = lds_read_chunk<D>(sQ[cur], qr + l32, 2 * kk + hi);
+                        bk[kk] = lds_read_chunk<D>(sK, 32 * kg + l32, 2 * kk + hi);
+                        ag[kk] = lds_read_chunk<D>(sDO[cur], qr + l32, 2 * kk + hi);
+                        bv[kk] = lds_read_chunk<D>(sV, 32 * kg + l32, 2 * kk + hi);
+                    }
+                    s = T::mfma(aq[0], bk[0], zero16);
+                    dp = T::mfma(ag[0], bv[0], zero16);
 #pragma unroll
-                for (int kk = 0; kk < KK; ++kk) {
-                    const u32x4 a = lds_read_chunk<D>(sQ[cur], l32, 2 * kk + hi);
-                    s = T::mfma(a, kreg[kk], s);
-                }
-#pragma unroll
-                for (int kk = 0; kk < KK; ++kk) {
-                    const u32x4 a = lds_read_chunk<D>(sDO[cur], l32, 2 * kk + hi);
-                    dp = T::mfma(a, vreg[kk], dp);
+                    for (int kk = 1; kk < KK; ++kk) {
+                        s = T::mfma(aq[kk], bk[kk], s);
+                        dp = T::mfma(ag[kk], bv[kk], dp);
+                    }
+                    sched_pipeline_mfma_lds<2 * KK, 2, 2>();
                 }
                 // ---- P, dS (C fragment: register i <-> query row 8*(i/4) + 4*hi + i%4) --------
 #pragma unroll
                 for (int grp = 0; grp < 4; ++grp) {
-                    const int roff = 8 * grp + 4 * hi;
+                    const int roff = qr + 8 * grp + 4 * hi;
                     const f32x4 l4 = *(const f32x4*)&sLse[cur][roff];
                     const f32x4 d4 = *(const f32x4*)&sDelta[cur][roff];
 #pragma unroll
                     for (int x = 0; x < 4; ++x) {
                         const float e = __builtin_amdgcn_exp2f(fmaf(s[4 * grp + x], c2, -l4[x]));
                         s[4 * grp + x] = e;
-                        dp[4 * grp + x] = e * (dp[4 * grp + x] - d4[x]) * p.scale;
+                        dp[4 * grp + x] = e * fmaf(dp[4 * grp + x], p.scale, -d4[x]);
                     }
                 }
                 if (cls == 1) {
 #pragma unroll
                     for (int grp = 0; grp < 4; ++grp) {
-                        const int roff = 8 * grp + 4 * hi;
-                        const u32x4 qlo = *(const u32x4*)&sQlo[cur][roff];
-                        const u32x4 qhi = *(const u32x4*)&sQhi[cur][roff];
+                        const int roff = qr + 8 * grp + 4 * hi;
+                        const u32x4 qalo = *(const u32x4*)&sQalo[cur][roff];
+                        const u32x4 qahi = *(const u32x4*)&sQahi[cur][roff];
+                        const u32x4 qxlo = *(const u32x4*)&sQxlo[cur][roff];
+                        const u32x4 qxhi = *(const u32x4*)&sQxhi[cur][roff];
                         const u32x4 qlim = *(const u32x4*)&sQlim[cur][roff];
 #pragma unroll
                         for (int x = 0; x < 4; ++x) {
                             QueryBits qb;
-                            qb.lo = qlo[x];
-                            qb.hi = qhi[x];
+                            qb.a_lo = qalo[x];
+                            qb.a_hi = qahi[x];
+                            qb.x_lo = qxlo[x];
+                            qb.x_hi = qxhi[x];
                             qb.lim = (int)qlim[x];
-                            qb.text = (qlo[x] & 1u) != 0;
+                            qb.text = (int)qahi[x] >= 0;  // modality rows carry a_hi = ~0
                             const bool a = allow_pair(qb, klo, khi, key);
                             s[4 * grp + x] = a ? s[4 * grp + x] : 0.f;
                             dp[4 * grp + x] = a ? dp[4 * grp + x] : 0.f;
@@ -230,44 +245,55 @@ __global__ __launch_bounds__(DKDV_THREADS, 1) void bwd_dkdv_kernel(const AttnPar
                     dsb[t] = pack8<T>(dp, 8 * t);
                 }
                 // ---- dV^T += dO^T P ; dK^T += Q^T dS -------------------------------------------
+                {
+                    u32x4 tg[2][DB], tq[2][DB];
 #pragma unroll
-                for (int db = 0; db < DB; ++db)
+                    for (int t = 0; t < 2; ++t)
 #pragma unroll
-                    for (int t = 0; t < 2; ++t) {
-                        const u32x4 a = lds_read_transposed<D>(sDO[cur], lane, 16 * t + 4 * hi, 32 * db + 16 * half16);
-                        dv[db] = T::mfma(a, pb[t], dv[db]);
-                    }
+                        for (int db = 0; db < DB; ++db) {
+                            tg[t][db] = lds_read_transposed<D>(sDO[cur], lane, qr + 16 * t + 4 * hi, 32 * db + 16 * half16);
+                            tq[t][db] = lds_read_transposed<D>(sQ[cur], lane, qr + 16 * t + 4 * hi, 32 * db + 16 * half16);
+                        }
 #pragma unroll
-                for (int db = 0; db < DB; ++db)
+                    for (int t = 0; t < 2; ++t)
 #pragma unroll
-                    for (int t = 0; t < 2; ++t) {
-                        const u32x4 a = lds_read_transposed<D>(sQ[cur], lane, 16 * t + 4 * hi, 32 * db + 16 * half16);
-                        dk[db] = T::mfma(a, dsb[t], dk[db]);
-                    }
+                        for (int db = 0; db < DB; ++db) {
+                            dv[db] = T::mfma(tg[t][db], pb[t], dv[db]);
+                            dk[db] = T::mfma(tq[t][db], dsb[t], dk[db]);
+                        }
+                    sched_pipeline_mfma_lds<4 * DB, 3, 2>();
+                }
             }
             if (more) stage_store(it + 1, n, cur ^ 1);
+            wait_async();
             __syncthreads();
         }
     }
 
-    // ---- epilogue: accumulate into the caller's fp32 buffers (sole owner of these rows) -----
-    if (kvalid) {
-        float* dkp = (float*)p.dk.ptr + ((int64_t)b * p.dk.sb + (int64_t)key * p.dk.ss + (int64_t)hk * p.dk.sh);
-        float* dvp = (float*)p.dv.ptr + ((int64_t)b * p.dv.sb + (int64_t)key * p.dv.ss + (int64_t)hk * p.dv.sh);
+    // ---- epilogue: the two waves of a key group add their partial sums to the caller's fp32
+    // buffers in turn (this workgroup is the sole owner of these rows)
+    float* dkp = (float*)p.dk.ptr + ((int64_t)b * p.dk.sb + (int64_t)key * p.dk.ss + (int64_t)hk * p.dk.sh);
+    float* dvp = (float*)p.dv.ptr + ((int64_t)b * p.dv.sb + (int64_t)key * p.dv.ss + (int64_t)hk * p.dv.sh);
 #pragma unroll
-        for (int db = 0; db < DB; ++db)
+    for (int turn = 0; turn < 2; ++turn) {
+        if (st == turn && kvalid) {
 #pragma unroll
-            for (int grp = 0; grp < 4; ++grp) {
-                const int d0 = 32 * db + 8 * grp + 4 * hi;
-                f32x4 a = *(f32x4*)(dkp + d0), c = *(f32x4*)(dvp + d0);
+            for (int db = 0; db < DB; ++db)
 #pragma unroll
-                for (int x = 0; x < 4; ++x) {
-                    a[x] += dk[db][4 * grp + x];
-                    c[x] += dv[db][4 * grp + x];
+                for (int grp = 0; grp < 4; ++grp) {
+                    const int d0 = 32 * db + 8 * grp + 4 * hi;
+                    f32x4 a = *(f32x4*)(dkp + d0), c = *(f32x4*)(dvp + d0);
+#pragma unroll
+                    for (int x = 0; x < 4; ++x) {
+                        a[x] += dk[db][4 * grp + x];
+                        c[x] += dv[db][4 * grp + x];
+                    }
+                    *(f32x4*)(dkp + d0) = a;
+                    *(f32x4*)(dvp + d0) = c;
                 }
-                *(f32x4*)(dkp + d0) = a;
-                *(f32x4*)(dvp + d0) = c;
-            }
+        }
+        __threadfence_block();
+        __syncthreads();
     }
 }
 
@@ -341,10 +367,12 @@ __global__ __launch_bounds__(DQ_THREADS, 2) void bwd_dq_kernel(const AttnParams 
 
     const char* kbase = (const char*)p.k.ptr + 2 * ((int64_t)b * p.k.sb + (int64_t)hk * p.k.sh);
     const char* vbase = (const char*)p.v.ptr + 2 * ((int64_t)b * p.v.sb + (int64_t)hk * p.v.sh);
-    const int64_t k_rs = 2 * p.k.ss, v_rs = 2 * p.v.ss;
+    const int64_t k_ts = 2 * p.k.ss * DQ_KT, v_ts = 2 * p.v.ss * DQ_KT;  // bytes per tile
     const int64_t* bfrow = p.bf + (int64_t)b * p.bf_sb;
 
     TileStage<D, DQ_KT, DQ_THREADS> stK, stV;
+    stK.setup(2 * p.k.ss, tid);
+    stV.setup(2 * p.v.ss, tid);
     int64_t kf_stage = 0;
 
     __syncthreads();
@@ -352,16 +380,15 @@ __global__ __launch_bounds__(DQ_THREADS, 2) void bwd_dq_kernel(const AttnParams 
     if (n > 0) {
         {
             const int kt = sList[0] >> 2;
-            stK.load(kbase, k_rs, kt * DQ_KT, S, tid);
-            stV.load(vbase, v_rs, kt * DQ_KT, S, tid);
+            stK.load(kbase + kt * k_ts, sK[0], S - kt * DQ_KT, tid);
+            stV.load(vbase + kt * v_ts, sV[0], S - kt * DQ_KT, tid);
             if (tid < DQ_KT) kf_stage = (kt * DQ_KT + tid < S) ? bfrow[kt * DQ_KT + tid] : 0;
-            stK.store(sK[0], tid);
-            stV.store(sV[0], tid);
             if (tid < DQ_KT) {
                 sKlo[0][tid] = (unsigned)(kf_stage & 0xFFFFFFFFll);
                 sKhi[0][tid] = ((unsigned)((uint64_t)kf_stage >> 32)) & HI_MODALITY_MASK;
             }
         }
+        wait_async();
         __syncthreads();
         for (int it = 0; it < n; ++it) {
             const int cur = it & 1;
@@ -370,8 +397,8 @@ __global__ __launch_bounds__(DQ_THREADS, 2) void bwd_dq_kernel(const AttnParams 
             const bool more = it + 1 < n;
             if (more) {
                 const int kt1 = sList[it + 1] >> 2;
-                stK.load(kbase, k_rs, kt1 * DQ_KT, S, tid);
-                stV.load(vbase, v_rs, kt1 * DQ_KT, S, tid);
+                stK.load(kbase + kt1 * k_ts, sK[cur ^ 1], S - kt1 * DQ_KT, tid);
+                stV.load(vbase + kt1 * v_ts, sV[cur ^ 1], S - kt1 * DQ_KT, tid);
                 if (tid < DQ_KT) kf_stage = (kt1 * DQ_KT + tid < S) ? bfrow[kt1 * DQ_KT + tid] : 0;
             }
 #pragma unroll
@@ -382,15 +409,19 @@ __global__ __launch_bounds__(DQ_THREADS, 2) void bwd_dq_kernel(const AttnParams 
                     s[i] = 0.f;
                     dp[i] = 0.f;
                 }
+                {
+                    u32x4 ka[KK], va[KK];
 #pragma unroll
-                for (int kk = 0; kk < KK; ++kk) {
-                    const u32x4 a = lds_read_chunk<D>(sK[cur], 32 * kb + l32, 2 * kk + hi);
-                    s = T::mfma(a, qreg[kk], s);
-                }
+                    for (int kk = 0; kk < KK; ++kk) {
+                        ka[kk] = lds_read_chunk<D>(sK[cur], 32 * kb + l32, 2 * kk + hi);
+                        va[kk] = lds_read_chunk<D>(sV[cur], 32 * kb + l32, 2 * kk + hi);
+                    }
 #pragma unroll
-                for (int kk = 0; kk < KK; ++kk) {
-                    const u32x4 a = lds_read_chunk<D>(sV[cur], 32 * kb + l32, 2 * kk + hi);
-                    dp = T::mfma(a, greg[kk], dp);
+                    for (int kk = 0; kk < KK; ++kk) {
+                        s = T::mfma(ka[kk], qreg[kk], s);
+                        dp = T::mfma(va[kk], greg[kk], dp);
+                    }
+                    sched_pipeline_mfma_lds<2 * KK, 4, 1>();
                 }
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
@@ -412,23 +443,26 @@ __global__ __launch_bounds__(DQ_THREADS, 2) void bwd_dq_kernel(const AttnParams 
                 u32x4 dsb[2];
 #pragma unroll
                 for (int t = 0; t < 2; ++t) dsb[t] = pack8<T>(dp, 8 * t);
+                {
+                    u32x4 ta[2][DB];
 #pragma unroll
-                for (int db = 0; db < DB; ++db)
+                    for (int t = 0; t < 2; ++t)
 #pragma unroll
-                    for (int t = 0; t < 2; ++t) {
-                        const u32x4 a =
-                            lds_read_transposed<D>(sK[cur], lane, 32 * kb + 16 * t + 4 * hi, 32 * db + 16 * half16);
-                        dq[db] = T::mfma(a, dsb[t], dq[db]);
-                    }
-            }
-            if (more) {
-                stK.store(sK[cur ^ 1], tid);
-                stV.store(sV[cur ^ 1], tid);
-                if (tid < DQ_KT) {
-                    sKlo[cur ^ 1][tid] = (unsigned)(kf_stage & 0xFFFFFFFFll);
-                    sKhi[cur ^ 1][tid] = ((unsigned)((uint64_t)kf_stage >> 32)) & HI_MODALITY_MASK;
+                        for (int db = 0; db < DB; ++db)
+                            ta[t][db] = lds_read_transposed<D>(sK[cur], lane, 32 * kb + 16 * t + 4 * hi,
+                                                               32 * db + 16 * half16);
+#pragma unroll
+                    for (int t = 0; t < 2; ++t)
+#pragma unroll
+                        for (int db = 0; db < DB; ++db) dq[db] = T::mfma(ta[t][db], dsb[t], dq[db]);
+                    sched_pipeline_mfma_lds<2 * DB, 2, 2>();
                 }
             }
+            if (more && tid < DQ_KT) {
+                sKlo[cur ^ 1][tid] = (unsigned)(kf_stage & 0xFFFFFFFFll);
+                sKhi[cur ^ 1][tid] = ((unsigned)((uint64_t)kf_stage >> 32)) & HI_MODALITY_MASK;
+            }
+            wait_async();
             __syncthreads();
         }
     }

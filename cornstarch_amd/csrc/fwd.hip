@@ -7,7 +7,8 @@
 //   key loop   = 64-key tiles taken from the flag row of this query block: empty tiles are
 //                never touched, "full" tiles skip the mask, "partial" tiles evaluate the
 //                bitfield rule in registers.
-//   K/V tiles  = double buffered in LDS (global -> registers is issued one tile ahead).
+//   K/V tiles  = double buffered in LDS; the next tile is copied global -> LDS directly while
+//                the current one is consumed.
 // Math layout
 //   S^T = K Q^T on v_mfma_f32_32x32x16 with K rows as the A operand (LDS) and Q as the B
 //   operand (registers).  In the C fragment a lane owns ONE query (lane & 31) and 16 of the
@@ -72,15 +73,27 @@ __global__ __launch_bounds__(FWD_THREADS, 2) void fwd_kernel(const AttnParams p)
     for (int db = 0; db < DB; ++db)
 #pragma unroll
         for (int i = 0; i < 16; ++i) o[db][i] = 0.f;
-    float m_i = -INFINITY, l_i = 0.f;
+    // Online softmax state.  m_i is the reference maximum the exponentials are taken against;
+    // it is only moved (and O, l rescaled) when a tile raises a row's maximum by more than
+    // RESCALE_LOG2 in the exponent, so most tiles skip the rescale entirely.  Until then the
+    // probabilities are at most 2^RESCALE_LOG2, harmless in fp32 / bf16 and cancelled by the
+    // final division by l.
+    constexpr float RESCALE_LOG2 = 8.f;
+    float m_i = -INFINITY, l_i = 0.f, nb = 0.f;  // nb = -m_i * c2 (0 while m_i is -inf)
     const float c2 = p.scale * LOG2E;
+    const float rescale_thr = RESCALE_LOG2 / c2;
+    f32x16 zero16;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) zero16[i] = 0.f;
 
     const char* kbase = (const char*)p.k.ptr + 2 * ((int64_t)b * p.k.sb + (int64_t)hk * p.k.sh);
     const char* vbase = (const char*)p.v.ptr + 2 * ((int64_t)b * p.v.sb + (int64_t)hk * p.v.sh);
-    const int64_t k_rs = 2 * p.k.ss, v_rs = 2 * p.v.ss;
+    const int64_t k_ts = 2 * p.k.ss * FWD_KT, v_ts = 2 * p.v.ss * FWD_KT;  // bytes per tile
     const int64_t* bfrow = p.bf + (int64_t)b * p.bf_sb;
 
     TileStage<D, FWD_KT, FWD_THREADS> stK, stV;
+    stK.setup(2 * p.k.ss, tid);
+    stV.setup(2 * p.v.ss, tid);
     int64_t kf_stage = 0;
 
     __syncthreads();
@@ -88,16 +101,15 @@ __global__ __launch_bounds__(FWD_THREADS, 2) void fwd_kernel(const AttnParams p)
     if (n > 0) {
         {
             const int kt = sList[0] >> 2;
-            stK.load(kbase, k_rs, kt * FWD_KT, S, tid);
-            stV.load(vbase, v_rs, kt * FWD_KT, S, tid);
+            stK.load(kbase + kt * k_ts, sK[0], S - kt * FWD_KT, tid);
+            stV.load(vbase + kt * v_ts, sV[0], S - kt * FWD_KT, tid);
             if (tid < FWD_KT) kf_stage = (kt * FWD_KT + tid < S) ? bfrow[kt * FWD_KT + tid] : 0;
-            stK.store(sK[0], tid);
-            stV.store(sV[0], tid);
             if (tid < FWD_KT) {
                 sKlo[0][tid] = (unsigned)(kf_stage & 0xFFFFFFFFll);
                 sKhi[0][tid] = ((unsigned)((uint64_t)kf_stage >> 32)) & HI_MODALITY_MASK;
             }
         }
+        wait_async();
         __syncthreads();
         for (int it = 0; it < n; ++it) {
             const int cur = it & 1;
@@ -106,22 +118,28 @@ __global__ __launch_bounds__(FWD_THREADS, 2) void fwd_kernel(const AttnParams p)
             const bool more = it + 1 < n;
             if (more) {
                 const int kt1 = sList[it + 1] >> 2;
-                stK.load(kbase, k_rs, kt1 * FWD_KT, S, tid);
-                stV.load(vbase, v_rs, kt1 * FWD_KT, S, tid);
+                stK.load(kbase + kt1 * k_ts, sK[cur ^ 1], S - kt1 * FWD_KT, tid);
+                stV.load(vbase + kt1 * v_ts, sV[cur ^ 1], S - kt1 * FWD_KT, tid);
                 if (tid < FWD_KT) kf_stage = (kt1 * FWD_KT + tid < S) ? bfrow[kt1 * FWD_KT + tid] : 0;
             }
 
             // ---- S^T = K Q^T : 64 keys x 32 queries per wave ----------------------------
+            // two independent accumulator chains (key blocks 0 and 1) alternate; operand reads
+            // run a few MFMAs ahead of their use; the first MFMA of a chain takes C = 0
             f32x16 s[2];
+            {
+                u32x4 ka[KK][2];
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb) {
+                for (int kk = 0; kk < KK; ++kk)
 #pragma unroll
-                for (int i = 0; i < 16; ++i) s[kb][i] = 0.f;
+                    for (int kb = 0; kb < 2; ++kb) ka[kk][kb] = lds_read_chunk<D>(sK[cur], 32 * kb + l32, 2 * kk + hi);
 #pragma unroll
-                for (int kk = 0; kk < KK; ++kk) {
-                    const u32x4 a = lds_read_chunk<D>(sK[cur], 32 * kb + l32, 2 * kk + hi);
-                    s[kb] = T::mfma(a, qreg[kk], s[kb]);
-                }
+                for (int kb = 0; kb < 2; ++kb) s[kb] = T::mfma(ka[0][kb], qreg[0], zero16);
+#pragma unroll
+                for (int kk = 1; kk < KK; ++kk)
+#pragma unroll
+                    for (int kb = 0; kb < 2; ++kb) s[kb] = T::mfma(ka[kk][kb], qreg[kk], s[kb]);
+                sched_pipeline_mfma_lds<2 * KK, 4, 1>();
             }
 
             // ---- bitfield rule in registers (partial tiles only) ------------------------
@@ -143,31 +161,33 @@ __global__ __launch_bounds__(FWD_THREADS, 2) void fwd_kernel(const AttnParams p)
             }
 
             // ---- online softmax (per-lane scalars) ----------------------------------------
-            float mloc = s[0][0];
+            float mloc = fmaxf(s[0][0], s[1][0]);
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-                for (int i = 0; i < 16; ++i) mloc = fmaxf(mloc, s[kb][i]);
+            for (int i = 1; i < 16; ++i) mloc = fmaxf(mloc, fmaxf(s[0][i], s[1][i]));
             mloc = half_swap_max(mloc);
-            const float mnew = fmaxf(m_i, mloc);
-            const float muse = (mnew == -INFINITY) ? 0.f : mnew;
-            const float alpha = __builtin_amdgcn_exp2f((m_i - muse) * c2);
-            m_i = mnew;
-            const float nb = -muse * c2;
-            float psum = 0.f;
+            if (__any(mloc > m_i + rescale_thr)) {  // wave-uniform; rare after the first tiles
+                const float mnew = fmaxf(m_i, mloc);
+                const float muse = (mnew == -INFINITY) ? 0.f : mnew;
+                const float alpha = __builtin_amdgcn_exp2f((m_i - muse) * c2);  // 0 when m_i = -inf
+                m_i = mnew;
+                nb = -muse * c2;
+                l_i *= alpha;
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
+                for (int db = 0; db < DB; ++db)
 #pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    const float e = __builtin_amdgcn_exp2f(fmaf(s[kb][i], c2, nb));
-                    s[kb][i] = e;
-                    psum += e;
-                }
-            l_i = l_i * alpha + psum;
+                    for (int i = 0; i < 16; ++i) o[db][i] *= alpha;
+            }
+            float psum0 = 0.f, psum1 = 0.f;
 #pragma unroll
-            for (int db = 0; db < DB; ++db)
-#pragma unroll
-                for (int i = 0; i < 16; ++i) o[db][i] *= alpha;
+            for (int i = 0; i < 16; ++i) {
+                const float e0 = __builtin_amdgcn_exp2f(fmaf(s[0][i], c2, nb));
+                const float e1 = __builtin_amdgcn_exp2f(fmaf(s[1][i], c2, nb));
+                s[0][i] = e0;
+                s[1][i] = e1;
+                psum0 += e0;
+                psum1 += e1;
+            }
+            l_i += psum0 + psum1;
 
             u32x4 pb[2][2];
 #pragma unroll
@@ -176,25 +196,30 @@ __global__ __launch_bounds__(FWD_THREADS, 2) void fwd_kernel(const AttnParams p)
                 for (int t = 0; t < 2; ++t) pb[kb][t] = pack8<T>(s[kb], 8 * t);
 
             // ---- O^T += V^T P^T ---------------------------------------------------------------
-#pragma unroll
-            for (int db = 0; db < DB; ++db)
+            {
+                u32x4 va[2][2][DB];
 #pragma unroll
                 for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-                    for (int t = 0; t < 2; ++t) {
-                        const u32x4 a =
-                            lds_read_transposed<D>(sV[cur], lane, 32 * kb + 16 * t + 4 * hi, 32 * db + 16 * half16);
-                        o[db] = T::mfma(a, pb[kb][t], o[db]);
-                    }
-
-            if (more) {
-                stK.store(sK[cur ^ 1], tid);
-                stV.store(sV[cur ^ 1], tid);
-                if (tid < FWD_KT) {
-                    sKlo[cur ^ 1][tid] = (unsigned)(kf_stage & 0xFFFFFFFFll);
-                    sKhi[cur ^ 1][tid] = ((unsigned)((uint64_t)kf_stage >> 32)) & HI_MODALITY_MASK;
-                }
+                    for (int t = 0; t < 2; ++t)
+#pragma unroll
+                        for (int db = 0; db < DB; ++db)
+                            va[kb][t][db] = lds_read_transposed<D>(sV[cur], lane, 32 * kb + 16 * t + 4 * hi,
+                                                                   32 * db + 16 * half16);
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                    for (int t = 0; t < 2; ++t)
+#pragma unroll
+                        for (int db = 0; db < DB; ++db) o[db] = T::mfma(va[kb][t][db], pb[kb][t], o[db]);
+                sched_pipeline_mfma_lds<4 * DB, (DB >= 2 ? 3 : 2), 2>();
             }
+
+            if (more && tid < FWD_KT) {
+                sKlo[cur ^ 1][tid] = (unsigned)(kf_stage & 0xFFFFFFFFll);
+                sKhi[cur ^ 1][tid] = ((unsigned)((uint64_t)kf_stage >> 32)) & HI_MODALITY_MASK;
+            }
+            wait_async();
             __syncthreads();
         }
     }
