@@ -32,8 +32,10 @@ __device__ __forceinline__ bool allow_rule(int64_t qf, int64_t kf, int64_t i, in
 // per-pair test is branch free and identical for text and modality queries:
 //   v = ((k & a) ^ x)  over both halves
 //   text query     : a = q,  x = 0  -> v = q & k ; allowed iff v != 0 and kpos <= qpos
-//   modality query : a = ~0, x = q  -> v = q ^ k ; allowed iff v == 0 and q != 0
-// `lim` folds the position test and the q != 0 test into one compare (kpos <= lim).
+//   modality query : a = M,  x = q  -> v = q ^ k ; allowed iff v == 0 and q != 0
+// where M keeps the modality bits (everything but bits 62 and 63), so the key words can be
+// the raw halves of the int64 bitfield.  `lim` folds the position test and the q != 0 test
+// into one compare (kpos <= lim).
 struct QueryBits {
     unsigned a_lo, a_hi, x_lo, x_hi;
     int lim;    // qpos for text rows, INT_MAX for live modality rows, -1 for rows that see nothing
@@ -46,14 +48,14 @@ __device__ __forceinline__ QueryBits make_query_bits(int64_t qf, int qpos) {
     QueryBits q;
     q.text = (lo & 1u) != 0;
     q.a_lo = q.text ? lo : 0xFFFFFFFFu;
-    q.a_hi = q.text ? hi : 0xFFFFFFFFu;
+    q.a_hi = q.text ? hi : HI_MODALITY_MASK;
     q.x_lo = q.text ? 0u : lo;
     q.x_hi = q.text ? 0u : hi;
     q.lim = q.text ? qpos : (((lo | hi) != 0) ? 0x7FFFFFFF : -1);
     return q;
 }
 
-// klo/khi: modality bits of the key (bits 62/63 stripped), kpos: its position.
+// klo/khi: the two halves of the key's int64 bitfield (bits 62/63 may be set), kpos: its position.
 __device__ __forceinline__ bool allow_pair(const QueryBits& q, unsigned klo, unsigned khi, int kpos) {
     const unsigned v = ((klo & q.a_lo) ^ q.x_lo) | ((khi & q.a_hi) ^ q.x_hi);
     const bool nz = v != 0u;

@@ -53,6 +53,17 @@ struct TileStage {
     }
 };
 
+// One wave copies `DWORDS` consecutive dwords (a multiple of 64) global -> LDS asynchronously.
+template <int DWORDS>
+__device__ __forceinline__ void copy_dwords_async(const void* src, void* dst_lds, int lane) {
+    typedef __attribute__((address_space(1))) const void* gptr;
+    typedef __attribute__((address_space(3))) void* lptr;
+#pragma unroll
+    for (int i = 0; i < DWORDS / 64; ++i)
+        __builtin_amdgcn_global_load_lds((gptr)((const unsigned*)src + 64 * i + lane),
+                                         (lptr)((unsigned*)dst_lds + 64 * i), 4, 0, 0);
+}
+
 // All direct global-to-LDS copies this wave has issued have landed (pair with a barrier).
 __device__ __forceinline__ void wait_async() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 

@@ -67,13 +67,10 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
     __shared__ u32x4 sV[128 * NCH];
     __shared__ u32x4 sQ[2][DKDV_QT * NCH];
     __shared__ u32x4 sDO[2][DKDV_QT * NCH];
-    __shared__ __attribute__((aligned(16))) float sLse[2][DKDV_QT];
+    __shared__ __attribute__((aligned(16))) float sLse[2][DKDV_QT];      // natural-log lse of the rows
     __shared__ __attribute__((aligned(16))) float sDelta[2][DKDV_QT];
-    __shared__ __attribute__((aligned(16))) unsigned sQalo[2][DKDV_QT];
-    __shared__ __attribute__((aligned(16))) unsigned sQahi[2][DKDV_QT];
-    __shared__ __attribute__((aligned(16))) unsigned sQxlo[2][DKDV_QT];
-    __shared__ __attribute__((aligned(16))) unsigned sQxhi[2][DKDV_QT];
-    __shared__ __attribute__((aligned(16))) int sQlim[2][DKDV_QT];
+    __shared__ __attribute__((aligned(16))) int64_t sQbf[2][DKDV_QT];    // raw bitfields of the rows
+    __shared__ __attribute__((aligned(16))) unsigned sWq[DKDV_THREADS / 64][5][32];  // per-wave rule constants
     __shared__ int sList[MAX_LIST / 2];
     __shared__ int sCount;
 
@@ -105,9 +102,10 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
     }
     const int key = nt * 128 + kg * 32 + l32;
     const bool kvalid = key < S;
-    const int64_t kf = kvalid ? p.bf[(int64_t)b * p.bf_sb + key] : 0;
+    const int64_t* bfrow = p.bf + (int64_t)b * p.bf_sb;
+    const int64_t kf = kvalid ? bfrow[key] : 0;
     const unsigned klo = (unsigned)(kf & 0xFFFFFFFFll);
-    const unsigned khi = ((unsigned)((uint64_t)kf >> 32)) & HI_MODALITY_MASK;
+    const unsigned khi = (unsigned)((uint64_t)kf >> 32);
 
     f32x16 dk[DB], dv[DB];
 #pragma unroll
@@ -121,45 +119,38 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
 #pragma unroll
     for (int i = 0; i < 16; ++i) zero16[i] = 0.f;
     const float c2 = p.scale * LOG2E;
-    const int64_t* bfrow = p.bf + (int64_t)b * p.bf_sb;
 
     TileStage<D, DKDV_QT, DKDV_THREADS> stQ, stDO;
     stQ.setup(2 * p.q.ss, tid);
     stDO.setup(2 * p.dout.ss, tid);
-    float lse_stage = 0.f, delta_stage = 0.f;
-    int64_t qf_stage = 0;
 
-    // iteration `it` -> (q head of the group, list entry, 64-row half of the 128-row block)
-    auto tile_row0 = [&](int rem) { return (sList[rem >> 1] >> 8) * BLOCK_M + (rem & 1) * DKDV_QT; };
-    auto stage_load = [&](int it, int n, int buf) {
+    // iteration `it` -> (q head of the group, list entry, 64-row half of the 128-row block).
+    // Query blocks are visited from the LAST one down: the workgroups of one kv head that are
+    // resident together then read the same Q / dO tile at about the same time, and all but the
+    // first of them find it in L2.
+    auto list_at = [&](int rem, int n) { return sList[n - 1 - (rem >> 1)]; };
+    auto tile_row0 = [&](int rem, int n) { return (list_at(rem, n) >> 8) * BLOCK_M + (1 - (rem & 1)) * DKDV_QT; };
+    // Everything a tile needs (Q, dO rows, their lse, delta and bitfields) is copied global -> LDS
+    // without passing through registers; only the ragged last tile of a sequence is staged
+    // synchronously, with neutral values for the rows past the end (lse = +inf gives P = 0).
+    auto stage = [&](int it, int n, int buf) {
         const int g = it / (2 * n);
-        const int row0 = tile_row0(it - g * 2 * n);
+        const int row0 = tile_row0(it - g * 2 * n, n);
         const int h = hk * G + g;
         const char* qbase = (const char*)p.q.ptr + 2 * ((int64_t)b * p.q.sb + (int64_t)h * p.q.sh);
         const char* gbase = (const char*)p.dout.ptr + 2 * ((int64_t)b * p.dout.sb + (int64_t)h * p.dout.sh);
         stQ.load(qbase + (int64_t)row0 * 2 * p.q.ss, sQ[buf], S - row0, tid);
         stDO.load(gbase + (int64_t)row0 * 2 * p.dout.ss, sDO[buf], S - row0, tid);
-        if (tid < DKDV_QT) {
-            const int r = row0 + tid;
-            const bool ok = r < S;
-            const int64_t off = ((int64_t)b * p.Hq + h) * p.S_rounded + r;
-            const float l = ok ? p.lse[off] : -INFINITY;
-            // rows past the end, and rows that allow no key (lse = -inf), must give P = 0
-            lse_stage = (l == -INFINITY) ? INFINITY : l * LOG2E;
-            delta_stage = ok ? p.delta[off] * p.scale : 0.f;  // pre-scaled: dS = P (dP*scale - delta*scale)
-            qf_stage = ok ? bfrow[r] : 0;
-        }
-    };
-    auto stage_store = [&](int it, int n, int buf) {
-        if (tid < DKDV_QT) {
-            const QueryBits qb = make_query_bits(qf_stage, tile_row0(it % (2 * n)) + tid);
-            sLse[buf][tid] = lse_stage;
-            sDelta[buf][tid] = delta_stage;
-            sQalo[buf][tid] = qb.a_lo;
-            sQahi[buf][tid] = qb.a_hi;
-            sQxlo[buf][tid] = qb.x_lo;
-            sQxhi[buf][tid] = qb.x_hi;
-            sQlim[buf][tid] = qb.lim;
+        const int64_t off = ((int64_t)b * p.Hq + h) * p.S_rounded + row0;
+        if (S - row0 >= DKDV_QT) {
+            if (wave == 1) copy_dwords_async<DKDV_QT>(p.lse + off, sLse[buf], lane);
+            if (wave == 2) copy_dwords_async<DKDV_QT>(p.delta + off, sDelta[buf], lane);
+            if (wave == 3) copy_dwords_async<2 * DKDV_QT>(bfrow + row0, sQbf[buf], lane);
+        } else if (tid < DKDV_QT) {
+            const bool ok = row0 + tid < S;
+            sLse[buf][tid] = ok ? p.lse[off + tid] : INFINITY;
+            sDelta[buf][tid] = ok ? p.delta[off + tid] : 0.f;
+            sQbf[buf][tid] = ok ? bfrow[row0 + tid] : 0;
         }
     };
 
@@ -167,17 +158,16 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
     const int n = sCount;
     const int total = n * 2 * G;
     if (total > 0) {
-        stage_load(0, n, 0);
-        stage_store(0, n, 0);
+        stage(0, n, 0);
         wait_async();
         __syncthreads();
         const int qr = 32 * st;  // this wave's rows inside the 64-row tile
         for (int it = 0; it < total; ++it) {
             const int cur = it & 1;
-            const bool more = it + 1 < total;
-            if (more) stage_load(it + 1, n, cur ^ 1);
+            if (it + 1 < total) stage(it + 1, n, cur ^ 1);
 
-            const int entry = sList[(it % (2 * n)) >> 1];
+            const int rem = it % (2 * n);
+            const int entry = list_at(rem, n);
             const int cls = (entry >> (2 * kg)) & 3;  // this wave's own 128x32 flag
             if (cls != 0) {
                 // ---- S = Q K^T and dP = dO V^T : 32 queries x 32 keys; both operands of every MFMA
@@ -201,7 +191,9 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
                     }
                     sched_pipeline_mfma_lds<2 * KK, 2, 2>();
                 }
-                // ---- P, dS (C fragment: register i <-> query row 8*(i/4) + 4*hi + i%4) --------
+                // ---- P = exp(scale s - lse), dS/scale = P (dP - delta)   (the factor `scale` of dS
+                // is applied once to dK in the epilogue).  C fragment: register i <-> query row
+                // 8*(i/4) + 4*hi + i%4 of this wave's 32 rows.
 #pragma unroll
                 for (int grp = 0; grp < 4; ++grp) {
                     const int roff = qr + 8 * grp + 4 * hi;
@@ -209,20 +201,33 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
                     const f32x4 d4 = *(const f32x4*)&sDelta[cur][roff];
 #pragma unroll
                     for (int x = 0; x < 4; ++x) {
-                        const float e = __builtin_amdgcn_exp2f(fmaf(s[4 * grp + x], c2, -l4[x]));
+                        const float e = __builtin_amdgcn_exp2f(fmaf(s[4 * grp + x], c2, l4[x] * -LOG2E));
                         s[4 * grp + x] = e;
-                        dp[4 * grp + x] = e * fmaf(dp[4 * grp + x], p.scale, -d4[x]);
+                        dp[4 * grp + x] = e * (dp[4 * grp + x] - d4[x]);
                     }
                 }
                 if (cls == 1) {
+                    // rule constants of this wave's 32 rows, derived once per row (lane r < 32 takes
+                    // row r) and handed to all lanes through a wave-private LDS scratch
+                    {
+                        const int row0 = tile_row0(rem, n);
+                        const QueryBits qb = make_query_bits(sQbf[cur][qr + l32], row0 + qr + l32);
+                        if (hi == 0) {
+                            sWq[wave][0][l32] = qb.a_lo;
+                            sWq[wave][1][l32] = qb.a_hi;
+                            sWq[wave][2][l32] = qb.x_lo;
+                            sWq[wave][3][l32] = qb.x_hi;
+                            sWq[wave][4][l32] = (unsigned)qb.lim;
+                        }
+                    }
 #pragma unroll
                     for (int grp = 0; grp < 4; ++grp) {
-                        const int roff = qr + 8 * grp + 4 * hi;
-                        const u32x4 qalo = *(const u32x4*)&sQalo[cur][roff];
-                        const u32x4 qahi = *(const u32x4*)&sQahi[cur][roff];
-                        const u32x4 qxlo = *(const u32x4*)&sQxlo[cur][roff];
-                        const u32x4 qxhi = *(const u32x4*)&sQxhi[cur][roff];
-                        const u32x4 qlim = *(const u32x4*)&sQlim[cur][roff];
+                        const int roff = 8 * grp + 4 * hi;
+                        const u32x4 qalo = *(const u32x4*)&sWq[wave][0][roff];
+                        const u32x4 qahi = *(const u32x4*)&sWq[wave][1][roff];
+                        const u32x4 qxlo = *(const u32x4*)&sWq[wave][2][roff];
+                        const u32x4 qxhi = *(const u32x4*)&sWq[wave][3][roff];
+                        const u32x4 qlim = *(const u32x4*)&sWq[wave][4][roff];
 #pragma unroll
                         for (int x = 0; x < 4; ++x) {
                             QueryBits qb;
@@ -231,7 +236,7 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
                             qb.x_lo = qxlo[x];
                             qb.x_hi = qxhi[x];
                             qb.lim = (int)qlim[x];
-                            qb.text = (int)qahi[x] >= 0;  // modality rows carry a_hi = ~0
+                            qb.text = qlim[x] < 0x7FFFFFFFu;  // text rows carry their position, modality rows INT_MAX or -1
                             const bool a = allow_pair(qb, klo, khi, key);
                             s[4 * grp + x] = a ? s[4 * grp + x] : 0.f;
                             dp[4 * grp + x] = a ? dp[4 * grp + x] : 0.f;
@@ -264,7 +269,6 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
                     sched_pipeline_mfma_lds<4 * DB, 3, 2>();
                 }
             }
-            if (more) stage_store(it + 1, n, cur ^ 1);
             wait_async();
             __syncthreads();
         }
@@ -285,7 +289,7 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
                     f32x4 a = *(f32x4*)(dkp + d0), c = *(f32x4*)(dvp + d0);
 #pragma unroll
                     for (int x = 0; x < 4; ++x) {
-                        a[x] += dk[db][4 * grp + x];
+                        a[x] = fmaf(dk[db][4 * grp + x], p.scale, a[x]);
                         c[x] += dv[db][4 * grp + x];
                     }
                     *(f32x4*)(dkp + d0) = a;
@@ -309,8 +313,7 @@ __global__ __launch_bounds__(DQ_THREADS, 2) void bwd_dq_kernel(const AttnParams 
     constexpr int NCH = D / 8, KK = D / 16, DB = D / 32;
     __shared__ u32x4 sK[2][DQ_KT * NCH];
     __shared__ u32x4 sV[2][DQ_KT * NCH];
-    __shared__ __attribute__((aligned(16))) unsigned sKlo[2][DQ_KT];
-    __shared__ __attribute__((aligned(16))) unsigned sKhi[2][DQ_KT];
+    __shared__ __attribute__((aligned(16))) int64_t sKbf[2][DQ_KT];  // raw bitfields of the tile's keys
     __shared__ int sList[MAX_LIST];
     __shared__ int sCount;
 
@@ -373,7 +376,15 @@ __global__ __launch_bounds__(DQ_THREADS, 2) void bwd_dq_kernel(const AttnParams 
     TileStage<D, DQ_KT, DQ_THREADS> stK, stV;
     stK.setup(2 * p.k.ss, tid);
     stV.setup(2 * p.v.ss, tid);
-    int64_t kf_stage = 0;
+    // bitfields of a tile's keys: direct global -> LDS copy by wave 1; the ragged last tile is
+    // staged synchronously with 0 (never allowed) for the keys past the end
+    auto stage_key_bits = [&](int kt, int buf) {
+        if (S - kt * DQ_KT >= DQ_KT) {
+            if (wave == 1) copy_dwords_async<2 * DQ_KT>(bfrow + kt * DQ_KT, sKbf[buf], lane);
+        } else if (tid < DQ_KT) {
+            sKbf[buf][tid] = (kt * DQ_KT + tid < S) ? bfrow[kt * DQ_KT + tid] : 0;
+        }
+    };
 
     __syncthreads();
     const int n = sCount;
@@ -382,11 +393,7 @@ __global__ __launch_bounds__(DQ_THREADS, 2) void bwd_dq_kernel(const AttnParams 
             const int kt = sList[0] >> 2;
             stK.load(kbase + kt * k_ts, sK[0], S - kt * DQ_KT, tid);
             stV.load(vbase + kt * v_ts, sV[0], S - kt * DQ_KT, tid);
-            if (tid < DQ_KT) kf_stage = (kt * DQ_KT + tid < S) ? bfrow[kt * DQ_KT + tid] : 0;
-            if (tid < DQ_KT) {
-                sKlo[0][tid] = (unsigned)(kf_stage & 0xFFFFFFFFll);
-                sKhi[0][tid] = ((unsigned)((uint64_t)kf_stage >> 32)) & HI_MODALITY_MASK;
-            }
+            stage_key_bits(kt, 0);
         }
         wait_async();
         __syncthreads();
@@ -399,7 +406,7 @@ __global__ __launch_bounds__(DQ_THREADS, 2) void bwd_dq_kernel(const AttnParams 
                 const int kt1 = sList[it + 1] >> 2;
                 stK.load(kbase + kt1 * k_ts, sK[cur ^ 1], S - kt1 * DQ_KT, tid);
                 stV.load(vbase + kt1 * v_ts, sV[cur ^ 1], S - kt1 * DQ_KT, tid);
-                if (tid < DQ_KT) kf_stage = (kt1 * DQ_KT + tid < S) ? bfrow[kt1 * DQ_KT + tid] : 0;
+                stage_key_bits(kt1, cur ^ 1);
             }
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb) {
@@ -426,15 +433,17 @@ __global__ __launch_bounds__(DQ_THREADS, 2) void bwd_dq_kernel(const AttnParams 
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
                     const float e = __builtin_amdgcn_exp2f(fmaf(s[i], c2, -lse2));
-                    dp[i] = e * (dp[i] - dlt) * p.scale;
+                    dp[i] = e * (dp[i] - dlt);  // the factor `scale` of dS is applied to dQ in the epilogue
                 }
                 if (cls == 1) {
                     const int kt0 = kt * DQ_KT;
 #pragma unroll
                     for (int grp = 0; grp < 4; ++grp) {
                         const int koff = 32 * kb + 8 * grp + 4 * hi;
-                        const u32x4 klo = *(const u32x4*)&sKlo[cur][koff];
-                        const u32x4 khi = *(const u32x4*)&sKhi[cur][koff];
+                        const u32x4 k01 = *(const u32x4*)&sKbf[cur][koff];      // lo0 hi0 lo1 hi1
+                        const u32x4 k23 = *(const u32x4*)&sKbf[cur][koff + 2];  // lo2 hi2 lo3 hi3
+                        const unsigned klo[4] = {k01[0], k01[2], k23[0], k23[2]};
+                        const unsigned khi[4] = {k01[1], k01[3], k23[1], k23[3]};
 #pragma unroll
                         for (int x = 0; x < 4; ++x)
                             dp[4 * grp + x] = allow_pair(qb, klo[x], khi[x], kt0 + koff + x) ? dp[4 * grp + x] : 0.f;
@@ -458,10 +467,6 @@ __global__ __launch_bounds__(DQ_THREADS, 2) void bwd_dq_kernel(const AttnParams 
                     sched_pipeline_mfma_lds<2 * DB, 2, 2>();
                 }
             }
-            if (more && tid < DQ_KT) {
-                sKlo[cur ^ 1][tid] = (unsigned)(kf_stage & 0xFFFFFFFFll);
-                sKhi[cur ^ 1][tid] = ((unsigned)((uint64_t)kf_stage >> 32)) & HI_MODALITY_MASK;
-            }
             wait_async();
             __syncthreads();
         }
@@ -476,7 +481,7 @@ __global__ __launch_bounds__(DQ_THREADS, 2) void bwd_dq_kernel(const AttnParams 
                 const int d0 = 32 * db + 8 * grp + 4 * hi;
                 f32x4 a = *(f32x4*)(dqp + d0);
 #pragma unroll
-                for (int x = 0; x < 4; ++x) a[x] += dq[db][4 * grp + x];
+                for (int x = 0; x < 4; ++x) a[x] = fmaf(dq[db][4 * grp + x], p.scale, a[x]);
                 *(f32x4*)(dqp + d0) = a;
             }
     }

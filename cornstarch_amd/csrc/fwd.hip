@@ -30,8 +30,7 @@ __global__ __launch_bounds__(FWD_THREADS, 2) void fwd_kernel(const AttnParams p)
     constexpr int NCH = D / 8, KK = D / 16, DB = D / 32;
     __shared__ u32x4 sK[2][FWD_KT * NCH];
     __shared__ u32x4 sV[2][FWD_KT * NCH];
-    __shared__ __attribute__((aligned(16))) unsigned sKlo[2][FWD_KT];
-    __shared__ __attribute__((aligned(16))) unsigned sKhi[2][FWD_KT];
+    __shared__ __attribute__((aligned(16))) int64_t sKbf[2][FWD_KT];  // raw bitfields of the tile's keys
     __shared__ int sList[MAX_LIST];
     __shared__ int sCount;
 
@@ -94,7 +93,15 @@ __global__ __launch_bounds__(FWD_THREADS, 2) void fwd_kernel(const AttnParams p)
     TileStage<D, FWD_KT, FWD_THREADS> stK, stV;
     stK.setup(2 * p.k.ss, tid);
     stV.setup(2 * p.v.ss, tid);
-    int64_t kf_stage = 0;
+    // bitfields of a tile's keys: direct global -> LDS copy by wave 1; the ragged last tile is
+    // staged synchronously with 0 (never allowed) for the keys past the end
+    auto stage_key_bits = [&](int kt, int buf) {
+        if (S - kt * FWD_KT >= FWD_KT) {
+            if (wave == 1) copy_dwords_async<2 * FWD_KT>(bfrow + kt * FWD_KT, sKbf[buf], lane);
+        } else if (tid < FWD_KT) {
+            sKbf[buf][tid] = (kt * FWD_KT + tid < S) ? bfrow[kt * FWD_KT + tid] : 0;
+        }
+    };
 
     __syncthreads();
     const int n = sCount;
@@ -103,11 +110,7 @@ __global__ __launch_bounds__(FWD_THREADS, 2) void fwd_kernel(const AttnParams p)
             const int kt = sList[0] >> 2;
             stK.load(kbase + kt * k_ts, sK[0], S - kt * FWD_KT, tid);
             stV.load(vbase + kt * v_ts, sV[0], S - kt * FWD_KT, tid);
-            if (tid < FWD_KT) kf_stage = (kt * FWD_KT + tid < S) ? bfrow[kt * FWD_KT + tid] : 0;
-            if (tid < FWD_KT) {
-                sKlo[0][tid] = (unsigned)(kf_stage & 0xFFFFFFFFll);
-                sKhi[0][tid] = ((unsigned)((uint64_t)kf_stage >> 32)) & HI_MODALITY_MASK;
-            }
+            stage_key_bits(kt, 0);
         }
         wait_async();
         __syncthreads();
@@ -120,7 +123,7 @@ __global__ __launch_bounds__(FWD_THREADS, 2) void fwd_kernel(const AttnParams p)
                 const int kt1 = sList[it + 1] >> 2;
                 stK.load(kbase + kt1 * k_ts, sK[cur ^ 1], S - kt1 * FWD_KT, tid);
                 stV.load(vbase + kt1 * v_ts, sV[cur ^ 1], S - kt1 * FWD_KT, tid);
-                if (tid < FWD_KT) kf_stage = (kt1 * FWD_KT + tid < S) ? bfrow[kt1 * FWD_KT + tid] : 0;
+                stage_key_bits(kt1, cur ^ 1);
             }
 
             // ---- S^T = K Q^T : 64 keys x 32 queries per wave ----------------------------
@@ -150,8 +153,10 @@ __global__ __launch_bounds__(FWD_THREADS, 2) void fwd_kernel(const AttnParams p)
 #pragma unroll
                     for (int grp = 0; grp < 4; ++grp) {
                         const int koff = 32 * kb + 8 * grp + 4 * hi;
-                        const u32x4 klo = *(const u32x4*)&sKlo[cur][koff];
-                        const u32x4 khi = *(const u32x4*)&sKhi[cur][koff];
+                        const u32x4 k01 = *(const u32x4*)&sKbf[cur][koff];      // lo0 hi0 lo1 hi1
+                        const u32x4 k23 = *(const u32x4*)&sKbf[cur][koff + 2];  // lo2 hi2 lo3 hi3
+                        const unsigned klo[4] = {k01[0], k01[2], k23[0], k23[2]};
+                        const unsigned khi[4] = {k01[1], k01[3], k23[1], k23[3]};
 #pragma unroll
                         for (int x = 0; x < 4; ++x) {
                             const bool a = allow_pair(qb, klo[x], khi[x], kt0 + koff + x);
@@ -215,10 +220,6 @@ __global__ __launch_bounds__(FWD_THREADS, 2) void fwd_kernel(const AttnParams p)
                 sched_pipeline_mfma_lds<4 * DB, (DB >= 2 ? 3 : 2), 2>();
             }
 
-            if (more && tid < FWD_KT) {
-                sKlo[cur ^ 1][tid] = (unsigned)(kf_stage & 0xFFFFFFFFll);
-                sKhi[cur ^ 1][tid] = ((unsigned)((uint64_t)kf_stage >> 32)) & HI_MODALITY_MASK;
-            }
             wait_async();
             __syncthreads();
         }
