@@ -83,7 +83,7 @@ extern "C" {
 
 const char* bam_last_error(void) { return g_error; }
 
-int bam_abi_version(void) { return 1; }
+int bam_abi_version(void) { return 2; }
 
 int bam_tile_flags(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int64_t flags_stride_b,
                    int64_t flags_stride_m, int B, int S, void* stream) {
@@ -151,19 +151,28 @@ int bam_bwd_preprocess(const void* o, const void* dout, float* delta, int64_t o_
 }
 
 static int bwd_params(bam::AttnParams& p, const void* q, const void* k, const void* v, const void* dout,
-                      const float* lse, const float* delta, float* dq, float* dk, float* dv, const int64_t* bf,
+                      const float* lse, const float* delta, void* dq, void* dk, void* dv, const int64_t* bf,
                       const int8_t* flags, const int64_t* st, int B, int S, int Hq, int Hkv, int D, float scale,
-                      int dtype, bool need_dq, bool need_dkdv) {
+                      int dtype, int accumulate, bool need_dq, bool need_dkdv) {
     BAM_TRY(check_problem(B, S, Hq, Hkv, D, dtype));
     BAM_TRY(check_half_tensor("q", q, st[0], st[1], st[2]));
     BAM_TRY(check_half_tensor("k", k, st[3], st[4], st[5]));
     BAM_TRY(check_half_tensor("v", v, st[6], st[7], st[8]));
     BAM_TRY(check_half_tensor("do", dout, st[9], st[10], st[11]));
-    if (need_dq) BAM_TRY(check_f32_tensor("dq", dq, st[12], st[13], st[14]));
-    if (need_dkdv) {
-        BAM_TRY(check_f32_tensor("dk", dk, st[15], st[16], st[17]));
-        BAM_TRY(check_f32_tensor("dv", dv, st[18], st[19], st[20]));
+    if (accumulate) {
+        if (need_dq) BAM_TRY(check_f32_tensor("dq", dq, st[12], st[13], st[14]));
+        if (need_dkdv) {
+            BAM_TRY(check_f32_tensor("dk", dk, st[15], st[16], st[17]));
+            BAM_TRY(check_f32_tensor("dv", dv, st[18], st[19], st[20]));
+        }
+    } else {
+        if (need_dq) BAM_TRY(check_half_tensor("dq", dq, st[12], st[13], st[14]));
+        if (need_dkdv) {
+            BAM_TRY(check_half_tensor("dk", dk, st[15], st[16], st[17]));
+            BAM_TRY(check_half_tensor("dv", dv, st[18], st[19], st[20]));
+        }
     }
+    p.grad_typed = accumulate ? 0 : 1;
     if (lse == nullptr || delta == nullptr || bf == nullptr || flags == nullptr)
         return fail(BAM_ERR_INVALID_ARGUMENT, "bam_bwd: lse, delta, bf and flags must not be null");
     if (!(scale > 0.f)) return fail(BAM_ERR_INVALID_ARGUMENT, "bam_bwd: softmax scale must be > 0 (got %g)", scale);
@@ -192,51 +201,51 @@ static int bwd_params(bam::AttnParams& p, const void* q, const void* k, const vo
      dk_stride_s, dk_stride_h, dv_stride_b, dv_stride_s, dv_stride_h, bf_stride_b, flags_stride_b, flags_stride_m}
 
 int bam_bwd(const void* q, const void* k, const void* v, const void* dout, const float* lse,
-            const float* delta, float* dq, float* dk, float* dv, const int64_t* bf, const int8_t* flags,
+            const float* delta, void* dq, void* dk, void* dv, const int64_t* bf, const int8_t* flags,
             int64_t q_stride_b, int64_t q_stride_s, int64_t q_stride_h, int64_t k_stride_b,
             int64_t k_stride_s, int64_t k_stride_h, int64_t v_stride_b, int64_t v_stride_s,
             int64_t v_stride_h, int64_t do_stride_b, int64_t do_stride_s, int64_t do_stride_h,
             int64_t dq_stride_b, int64_t dq_stride_s, int64_t dq_stride_h, int64_t dk_stride_b,
             int64_t dk_stride_s, int64_t dk_stride_h, int64_t dv_stride_b, int64_t dv_stride_s,
             int64_t dv_stride_h, int64_t bf_stride_b, int64_t flags_stride_b, int64_t flags_stride_m, int B,
-            int S, int Hq, int Hkv, int D, float scale, int dtype, void* stream) {
+            int S, int Hq, int Hkv, int D, float scale, int dtype, int accumulate, void* stream) {
     const int64_t st[24] = BAM_BWD_STRIDES;
     bam::AttnParams p = {};
-    BAM_TRY(bwd_params(p, q, k, v, dout, lse, delta, dq, dk, dv, bf, flags, st, B, S, Hq, Hkv, D, scale, dtype, true, true));
+    BAM_TRY(bwd_params(p, q, k, v, dout, lse, delta, dq, dk, dv, bf, flags, st, B, S, Hq, Hkv, D, scale, dtype, accumulate, true, true));
     BAM_TRY(launched(bam::launch_bwd_dkdv(p, dtype, (hipStream_t)stream), "bam_bwd (dk/dv)"));
     return launched(bam::launch_bwd_dq(p, dtype, (hipStream_t)stream), "bam_bwd (dq)");
 }
 
 int bam_bwd_dkdv(const void* q, const void* k, const void* v, const void* dout, const float* lse,
-                 const float* delta, float* dk, float* dv, const int64_t* bf, const int8_t* flags,
+                 const float* delta, void* dk, void* dv, const int64_t* bf, const int8_t* flags,
                  int64_t q_stride_b, int64_t q_stride_s, int64_t q_stride_h, int64_t k_stride_b,
                  int64_t k_stride_s, int64_t k_stride_h, int64_t v_stride_b, int64_t v_stride_s,
                  int64_t v_stride_h, int64_t do_stride_b, int64_t do_stride_s, int64_t do_stride_h,
                  int64_t dk_stride_b, int64_t dk_stride_s, int64_t dk_stride_h, int64_t dv_stride_b,
                  int64_t dv_stride_s, int64_t dv_stride_h, int64_t bf_stride_b, int64_t flags_stride_b,
                  int64_t flags_stride_m, int B, int S, int Hq, int Hkv, int D, float scale, int dtype,
-                 void* stream) {
-    float* dq = nullptr;
+                 int accumulate, void* stream) {
+    void* dq = nullptr;
     const int64_t dq_stride_b = 0, dq_stride_s = 0, dq_stride_h = 0;
     const int64_t st[24] = BAM_BWD_STRIDES;
     bam::AttnParams p = {};
-    BAM_TRY(bwd_params(p, q, k, v, dout, lse, delta, dq, dk, dv, bf, flags, st, B, S, Hq, Hkv, D, scale, dtype, false, true));
+    BAM_TRY(bwd_params(p, q, k, v, dout, lse, delta, dq, dk, dv, bf, flags, st, B, S, Hq, Hkv, D, scale, dtype, accumulate, false, true));
     return launched(bam::launch_bwd_dkdv(p, dtype, (hipStream_t)stream), "bam_bwd_dkdv");
 }
 
 int bam_bwd_dq(const void* q, const void* k, const void* v, const void* dout, const float* lse,
-               const float* delta, float* dq, const int64_t* bf, const int8_t* flags, int64_t q_stride_b,
+               const float* delta, void* dq, const int64_t* bf, const int8_t* flags, int64_t q_stride_b,
                int64_t q_stride_s, int64_t q_stride_h, int64_t k_stride_b, int64_t k_stride_s,
                int64_t k_stride_h, int64_t v_stride_b, int64_t v_stride_s, int64_t v_stride_h,
                int64_t do_stride_b, int64_t do_stride_s, int64_t do_stride_h, int64_t dq_stride_b,
                int64_t dq_stride_s, int64_t dq_stride_h, int64_t bf_stride_b, int64_t flags_stride_b,
                int64_t flags_stride_m, int B, int S, int Hq, int Hkv, int D, float scale, int dtype,
-               void* stream) {
-    float *dk = nullptr, *dv = nullptr;
+               int accumulate, void* stream) {
+    void *dk = nullptr, *dv = nullptr;
     const int64_t dk_stride_b = 0, dk_stride_s = 0, dk_stride_h = 0, dv_stride_b = 0, dv_stride_s = 0, dv_stride_h = 0;
     const int64_t st[24] = BAM_BWD_STRIDES;
     bam::AttnParams p = {};
-    BAM_TRY(bwd_params(p, q, k, v, dout, lse, delta, dq, dk, dv, bf, flags, st, B, S, Hq, Hkv, D, scale, dtype, true, false));
+    BAM_TRY(bwd_params(p, q, k, v, dout, lse, delta, dq, dk, dv, bf, flags, st, B, S, Hq, Hkv, D, scale, dtype, accumulate, true, false));
     return launched(bam::launch_bwd_dq(p, dtype, (hipStream_t)stream), "bam_bwd_dq");
 }
 

@@ -15,7 +15,8 @@ struct Tensor4 {  // logical (B, S, H, D), unit stride along D, strides in eleme
 
 struct AttnParams {
     Tensor4 q, k, v, o, dout;  // 16-bit tensors
-    Tensor4 dq, dk, dv;        // fp32 accumulators (backward)
+    Tensor4 dq, dk, dv;        // gradients: fp32 accumulated into, or (grad_typed) input dtype, overwritten
+    int grad_typed;
     float* lse;                // (B, Hq, S_rounded)
     float* delta;              // (B, Hq, S_rounded)
     const int64_t* bf;

@@ -31,16 +31,18 @@ struct TileStage {
             goff[i] = (unsigned)(row * row_stride_bytes + (pc ^ swz<D>(row)) * 16);
         }
     }
-    // tile_base: first row of the tile in global memory; rows_valid: rows of it inside the sequence
+    // tile_base: first row of the tile in global memory (wave-uniform); rows_valid: rows of it
+    // inside the sequence (wave-uniform)
     __device__ __forceinline__ void load(const char* tile_base, u32x4* tile, int rows_valid, int tid) const {
         typedef __attribute__((address_space(1))) const void* gptr;
         typedef __attribute__((address_space(3))) void* lptr;
         if (rows_valid >= ROWS) {
+            const int wave_first = __builtin_amdgcn_readfirstlane(tid & ~63);
 #pragma unroll
             for (int i = 0; i < CPT; ++i)
-                if (EXACT || (tid & ~63) + THREADS * i < CHUNKS)  // wave-uniform
+                if (EXACT || wave_first + THREADS * i < CHUNKS)
                     __builtin_amdgcn_global_load_lds((gptr)(tile_base + goff[i]),
-                                                     (lptr)(tile + THREADS * i + (tid & ~63)), 16, 0, 0);
+                                                     (lptr)(tile + THREADS * i + wave_first), 16, 0, 0);
         } else {
 #pragma unroll
             for (int i = 0; i < CPT; ++i) {

@@ -128,7 +128,7 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
     // Query blocks are visited from the LAST one down: the workgroups of one kv head that are
     // resident together then read the same Q / dO tile at about the same time, and all but the
     // first of them find it in L2.
-    auto list_at = [&](int rem, int n) { return sList[n - 1 - (rem >> 1)]; };
+    auto list_at = [&](int rem, int n) { return __builtin_amdgcn_readfirstlane(sList[n - 1 - (rem >> 1)]); };
     auto tile_row0 = [&](int rem, int n) { return (list_at(rem, n) >> 8) * BLOCK_M + (1 - (rem & 1)) * DKDV_QT; };
     // Everything a tile needs (Q, dO rows, their lse, delta and bitfields) is copied global -> LDS
     // without passing through registers; only the ragged last tile of a sequence is staged
@@ -274,8 +274,51 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
         }
     }
 
-    // ---- epilogue: the two waves of a key group add their partial sums to the caller's fp32
-    // buffers in turn (this workgroup is the sole owner of these rows)
+    // ---- epilogue.  The two waves of a key group hold partial sums.
+    if (p.grad_typed) {
+        // Overwrite mode: dk/dv have the input dtype.  The K, V, Q, dO tiles are dead now; the
+        // stream-1 wave of key group kg parks its partial sums in tile array number kg (exactly
+        // the right size: 2 * D/32 * 16 floats per lane), its stream-0 partner adds its own and
+        // stores the converted result.
+        float* park = (float*)(kg == 0 ? sK : kg == 1 ? sV : kg == 2 ? &sQ[0][0] : &sDO[0][0]);
+        if (st == 1) {
+#pragma unroll
+            for (int db = 0; db < DB; ++db)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    park[(db * 16 + i) * 64 + lane] = dk[db][i];
+                    park[((DB + db) * 16 + i) * 64 + lane] = dv[db][i];
+                }
+        }
+        __syncthreads();
+        if (st == 0 && kvalid) {
+            char* dkp = (char*)p.dk.ptr + 2 * ((int64_t)b * p.dk.sb + (int64_t)key * p.dk.ss + (int64_t)hk * p.dk.sh);
+            char* dvp = (char*)p.dv.ptr + 2 * ((int64_t)b * p.dv.sb + (int64_t)key * p.dv.ss + (int64_t)hk * p.dv.sh);
+#pragma unroll
+            for (int db = 0; db < DB; ++db)
+#pragma unroll
+                for (int grp = 0; grp < 4; ++grp) {
+                    float a[4], c[4];
+#pragma unroll
+                    for (int x = 0; x < 4; ++x) {
+                        const int i = 4 * grp + x;
+                        a[x] = (dk[db][i] + park[(db * 16 + i) * 64 + lane]) * p.scale;
+                        c[x] = dv[db][i] + park[((DB + db) * 16 + i) * 64 + lane];
+                    }
+                    const int d0 = 32 * db + 8 * grp + 4 * hi;
+                    u32x2 wk, wv;
+                    wk[0] = T::pack2(a[0], a[1]);
+                    wk[1] = T::pack2(a[2], a[3]);
+                    wv[0] = T::pack2(c[0], c[1]);
+                    wv[1] = T::pack2(c[2], c[3]);
+                    *(u32x2*)(dkp + d0 * 2) = wk;
+                    *(u32x2*)(dvp + d0 * 2) = wv;
+                }
+        }
+        return;
+    }
+    // Accumulate mode: both waves add to the caller's fp32 buffers in turn (this workgroup is
+    // the sole owner of these rows).
     float* dkp = (float*)p.dk.ptr + ((int64_t)b * p.dk.sb + (int64_t)key * p.dk.ss + (int64_t)hk * p.dk.sh);
     float* dvp = (float*)p.dv.ptr + ((int64_t)b * p.dv.sb + (int64_t)key * p.dv.ss + (int64_t)hk * p.dv.sh);
 #pragma unroll
@@ -390,7 +433,7 @@ __global__ __launch_bounds__(DQ_THREADS, 2) void bwd_dq_kernel(const AttnParams 
     const int n = sCount;
     if (n > 0) {
         {
-            const int kt = sList[0] >> 2;
+            const int kt = __builtin_amdgcn_readfirstlane(sList[0]) >> 2;
             stK.load(kbase + kt * k_ts, sK[0], S - kt * DQ_KT, tid);
             stV.load(vbase + kt * v_ts, sV[0], S - kt * DQ_KT, tid);
             stage_key_bits(kt, 0);
@@ -399,11 +442,11 @@ __global__ __launch_bounds__(DQ_THREADS, 2) void bwd_dq_kernel(const AttnParams 
         __syncthreads();
         for (int it = 0; it < n; ++it) {
             const int cur = it & 1;
-            const int entry = sList[it];
+            const int entry = __builtin_amdgcn_readfirstlane(sList[it]);
             const int kt = entry >> 2, cls = entry & 3;
             const bool more = it + 1 < n;
             if (more) {
-                const int kt1 = sList[it + 1] >> 2;
+                const int kt1 = __builtin_amdgcn_readfirstlane(sList[it + 1]) >> 2;
                 stK.load(kbase + kt1 * k_ts, sK[cur ^ 1], S - kt1 * DQ_KT, tid);
                 stV.load(vbase + kt1 * v_ts, sV[cur ^ 1], S - kt1 * DQ_KT, tid);
                 stage_key_bits(kt1, cur ^ 1);
@@ -472,7 +515,18 @@ __global__ __launch_bounds__(DQ_THREADS, 2) void bwd_dq_kernel(const AttnParams 
         }
     }
 
-    if (qvalid) {
+    if (qvalid && p.grad_typed) {  // overwrite mode: dq has the input dtype
+        char* dqp = (char*)p.dq.ptr + 2 * ((int64_t)b * p.dq.sb + (int64_t)qrow * p.dq.ss + (int64_t)h * p.dq.sh);
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int grp = 0; grp < 4; ++grp) {
+                u32x2 w;
+                w[0] = T::pack2(dq[db][4 * grp + 0] * p.scale, dq[db][4 * grp + 1] * p.scale);
+                w[1] = T::pack2(dq[db][4 * grp + 2] * p.scale, dq[db][4 * grp + 3] * p.scale);
+                *(u32x2*)(dqp + (32 * db + 8 * grp + 4 * hi) * 2) = w;
+            }
+    } else if (qvalid) {
         float* dqp = (float*)p.dq.ptr + ((int64_t)b * p.dq.sb + (int64_t)qrow * p.dq.ss + (int64_t)h * p.dq.sh);
 #pragma unroll
         for (int db = 0; db < DB; ++db)

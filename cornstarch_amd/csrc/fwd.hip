@@ -107,7 +107,7 @@ __global__ __launch_bounds__(FWD_THREADS, 2) void fwd_kernel(const AttnParams p)
     const int n = sCount;
     if (n > 0) {
         {
-            const int kt = sList[0] >> 2;
+            const int kt = __builtin_amdgcn_readfirstlane(sList[0]) >> 2;
             stK.load(kbase + kt * k_ts, sK[0], S - kt * FWD_KT, tid);
             stV.load(vbase + kt * v_ts, sV[0], S - kt * FWD_KT, tid);
             stage_key_bits(kt, 0);
@@ -116,11 +116,11 @@ __global__ __launch_bounds__(FWD_THREADS, 2) void fwd_kernel(const AttnParams p)
         __syncthreads();
         for (int it = 0; it < n; ++it) {
             const int cur = it & 1;
-            const int entry = sList[it];
+            const int entry = __builtin_amdgcn_readfirstlane(sList[it]);
             const int kt = entry >> 2, cls = entry & 3;
             const bool more = it + 1 < n;
             if (more) {
-                const int kt1 = sList[it + 1] >> 2;
+                const int kt1 = __builtin_amdgcn_readfirstlane(sList[it + 1]) >> 2;
                 stK.load(kbase + kt1 * k_ts, sK[cur ^ 1], S - kt1 * FWD_KT, tid);
                 stV.load(vbase + kt1 * v_ts, sV[cur ^ 1], S - kt1 * FWD_KT, tid);
                 stage_key_bits(kt1, cur ^ 1);

@@ -14,7 +14,7 @@ LIB_PATH = os.path.join(_PKG_DIR, "libbam_hip.so")
 BAM_DTYPE_F16 = 0
 BAM_DTYPE_BF16 = 1
 BAM_MAX_SEQLEN = 131072
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 _i64 = ctypes.c_int64
 _int = ctypes.c_int
@@ -27,9 +27,9 @@ SIGNATURES = {
     "bam_materialize_mask": [_ptr, _i64, _ptr, _int, _int, _ptr],
     "bam_fwd": [_ptr] * 7 + [_i64] * 15 + [_int] * 5 + [_f32, _int, _ptr],
     "bam_bwd_preprocess": [_ptr] * 3 + [_i64] * 6 + [_int] * 5 + [_ptr],
-    "bam_bwd": [_ptr] * 11 + [_i64] * 24 + [_int] * 5 + [_f32, _int, _ptr],
-    "bam_bwd_dkdv": [_ptr] * 10 + [_i64] * 21 + [_int] * 5 + [_f32, _int, _ptr],
-    "bam_bwd_dq": [_ptr] * 9 + [_i64] * 18 + [_int] * 5 + [_f32, _int, _ptr],
+    "bam_bwd": [_ptr] * 11 + [_i64] * 24 + [_int] * 5 + [_f32, _int, _int, _ptr],
+    "bam_bwd_dkdv": [_ptr] * 10 + [_i64] * 21 + [_int] * 5 + [_f32, _int, _int, _ptr],
+    "bam_bwd_dq": [_ptr] * 9 + [_i64] * 18 + [_int] * 5 + [_f32, _int, _int, _ptr],
 }
 
 _lib = None

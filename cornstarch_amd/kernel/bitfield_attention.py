@@ -201,7 +201,8 @@ def _launch_bwd_preprocess(o, do, delta):
         )
 
 
-def _launch_bwd_dkdv(q, k, v, do, lse, delta, dk, dv, bf, flags, softmax_scale):
+def _launch_bwd_dkdv(q, k, v, do, lse, delta, dk, dv, bf, flags, softmax_scale, accumulate=True):
+    """accumulate=True: dk/dv are fp32 and added to; False: dk/dv have q's dtype and are overwritten."""
     B, S, Hq, D = q.shape
     with torch.cuda.device(q.device):
         _bam_hip.call(
@@ -209,11 +210,12 @@ def _launch_bwd_dkdv(q, k, v, do, lse, delta, dk, dv, bf, flags, softmax_scale):
             q.data_ptr(), k.data_ptr(), v.data_ptr(), do.data_ptr(), lse.data_ptr(), delta.data_ptr(),
             dk.data_ptr(), dv.data_ptr(), bf.data_ptr(), flags.data_ptr(),
             *_strides3(q, k, v, do, dk, dv), bf.stride(0), flags.stride(0), flags.stride(1),
-            B, S, Hq, k.shape[2], D, float(softmax_scale), _dtype_code(q.dtype), _stream_ptr(q.device),
+            B, S, Hq, k.shape[2], D, float(softmax_scale), _dtype_code(q.dtype), int(accumulate),
+            _stream_ptr(q.device),
         )
 
 
-def _launch_bwd_dq(q, k, v, do, lse, delta, dq, bf, flags, softmax_scale):
+def _launch_bwd_dq(q, k, v, do, lse, delta, dq, bf, flags, softmax_scale, accumulate=True):
     B, S, Hq, D = q.shape
     with torch.cuda.device(q.device):
         _bam_hip.call(
@@ -221,8 +223,38 @@ def _launch_bwd_dq(q, k, v, do, lse, delta, dq, bf, flags, softmax_scale):
             q.data_ptr(), k.data_ptr(), v.data_ptr(), do.data_ptr(), lse.data_ptr(), delta.data_ptr(),
             dq.data_ptr(), bf.data_ptr(), flags.data_ptr(),
             *_strides3(q, k, v, do, dq), bf.stride(0), flags.stride(0), flags.stride(1),
-            B, S, Hq, k.shape[2], D, float(softmax_scale), _dtype_code(q.dtype), _stream_ptr(q.device),
+            B, S, Hq, k.shape[2], D, float(softmax_scale), _dtype_code(q.dtype), int(accumulate),
+            _stream_ptr(q.device),
         )
+
+
+def _is_kernel_ready(x: torch.Tensor, elems_per_16b: int = 8) -> bool:
+    return _kernel_ready(x, elems_per_16b) is x
+
+
+def _bitfield_attn_backward_overwrite(do, q, k, v, o, bitfield_mask, compressed_mask, lse, softmax_scale):
+    """Gradients in the input dtype, written (not accumulated) by the kernels: what
+    ``BitfieldAttentionFunction.backward`` needs, without the reference's zero-filled fp32
+    staging buffers and the final cast (bitfield_attention.py:1248-1266).  Returns None when the
+    layout needs the general path (padded head dimension, unaligned views)."""
+    d = q.shape[-1]
+    if d not in _SUPPORTED_HEAD_DIMS:
+        return None
+    if do.stride(-1) != 1 or not _is_kernel_ready(do):
+        do = do.contiguous()
+    if not all(_is_kernel_ready(x) for x in (q, k, v, o)):
+        return None
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    if not all(_is_kernel_ready(x) for x in (dq, dk, dv)):
+        return None
+    lse = lse.contiguous()
+    bf = bitfield_mask if bitfield_mask.stride(1) == 1 else bitfield_mask.contiguous()
+    flags = compressed_mask if compressed_mask.stride(-1) == 1 else compressed_mask.contiguous()
+    delta = torch.empty_like(lse)
+    _launch_bwd_preprocess(o, do, delta)
+    _launch_bwd_dkdv(q, k, v, do, lse, delta, dk, dv, bf, flags, softmax_scale, accumulate=False)
+    _launch_bwd_dq(q, k, v, do, lse, delta, dq, bf, flags, softmax_scale, accumulate=False)
+    return dq, dk, dv
 
 
 def _bitfield_attn_backward(
@@ -312,6 +344,11 @@ class BitfieldAttentionFunction(torch.autograd.Function):
         q, k, v, o, lse, bias, bitfield_mask, compressed_mask = ctx.saved_tensors
         assert not ctx.needs_input_grad[3], "the bitfield mask is not differentiable"
         with torch.no_grad():
+            direct = _bitfield_attn_backward_overwrite(
+                do, q, k, v, o, bitfield_mask, compressed_mask, lse, ctx.softmax_scale
+            ) if bias is None else None
+            if direct is not None:
+                return (*direct, None, None, None)
             dq = torch.zeros_like(q, dtype=torch.float32)
             dk = torch.zeros_like(k, dtype=torch.float32)
             dv = torch.zeros_like(v, dtype=torch.float32)

@@ -83,20 +83,24 @@ int bam_bwd_preprocess(const void* o, const void* dout, float* delta, int64_t o_
 
 /*
  * Backward.  Replaces `_bwd_kernel[grid]` (bitfield_attention.py:598-929, 1145-1199).
- * dq, dk, dv are fp32 and are ACCUMULATED INTO (the caller zeroes them,
- * bitfield_attention.py:1248-1250); dk/dv receive the sum over the q heads of a group.
- * No atomics are used: each output element is owned by exactly one workgroup, so the
- * result is deterministic.
+ * accumulate != 0: dq, dk, dv are fp32 and are ACCUMULATED INTO (the caller zeroes them,
+ *   bitfield_attention.py:1248-1250) -- the contract of `_bitfield_attn_backward`.
+ * accumulate == 0: dq, dk, dv have the input dtype (16-byte aligned rows like q) and are
+ *   OVERWRITTEN with the final gradients, which spares the autograd path
+ *   (BitfieldAttentionFunction.backward, bitfield_attention.py:1240-1266) the zero fill and
+ *   the fp32 -> dtype cast.
+ * dk/dv receive the sum over the q heads of a group.  No atomics are used: each output
+ * element is owned by exactly one workgroup, so the result is deterministic.
  */
 int bam_bwd(const void* q, const void* k, const void* v, const void* dout, const float* lse,
-            const float* delta, float* dq, float* dk, float* dv, const int64_t* bf, const int8_t* flags,
+            const float* delta, void* dq, void* dk, void* dv, const int64_t* bf, const int8_t* flags,
             int64_t q_stride_b, int64_t q_stride_s, int64_t q_stride_h, int64_t k_stride_b,
             int64_t k_stride_s, int64_t k_stride_h, int64_t v_stride_b, int64_t v_stride_s,
             int64_t v_stride_h, int64_t do_stride_b, int64_t do_stride_s, int64_t do_stride_h,
             int64_t dq_stride_b, int64_t dq_stride_s, int64_t dq_stride_h, int64_t dk_stride_b,
             int64_t dk_stride_s, int64_t dk_stride_h, int64_t dv_stride_b, int64_t dv_stride_s,
             int64_t dv_stride_h, int64_t bf_stride_b, int64_t flags_stride_b, int64_t flags_stride_m, int B,
-            int S, int Hq, int Hkv, int D, float scale, int dtype, void* stream);
+            int S, int Hq, int Hkv, int D, float scale, int dtype, int accumulate, void* stream);
 
 /*
  * The two halves of bam_bwd as separate launches (same reference kernel,
@@ -106,23 +110,23 @@ int bam_bwd(const void* q, const void* k, const void* v, const void* dout, const
  * (frozen encoder outputs, for instance) does not pay for the other.
  */
 int bam_bwd_dkdv(const void* q, const void* k, const void* v, const void* dout, const float* lse,
-                 const float* delta, float* dk, float* dv, const int64_t* bf, const int8_t* flags,
+                 const float* delta, void* dk, void* dv, const int64_t* bf, const int8_t* flags,
                  int64_t q_stride_b, int64_t q_stride_s, int64_t q_stride_h, int64_t k_stride_b,
                  int64_t k_stride_s, int64_t k_stride_h, int64_t v_stride_b, int64_t v_stride_s,
                  int64_t v_stride_h, int64_t do_stride_b, int64_t do_stride_s, int64_t do_stride_h,
                  int64_t dk_stride_b, int64_t dk_stride_s, int64_t dk_stride_h, int64_t dv_stride_b,
                  int64_t dv_stride_s, int64_t dv_stride_h, int64_t bf_stride_b, int64_t flags_stride_b,
                  int64_t flags_stride_m, int B, int S, int Hq, int Hkv, int D, float scale, int dtype,
-                 void* stream);
+                 int accumulate, void* stream);
 
 int bam_bwd_dq(const void* q, const void* k, const void* v, const void* dout, const float* lse,
-               const float* delta, float* dq, const int64_t* bf, const int8_t* flags, int64_t q_stride_b,
+               const float* delta, void* dq, const int64_t* bf, const int8_t* flags, int64_t q_stride_b,
                int64_t q_stride_s, int64_t q_stride_h, int64_t k_stride_b, int64_t k_stride_s,
                int64_t k_stride_h, int64_t v_stride_b, int64_t v_stride_s, int64_t v_stride_h,
                int64_t do_stride_b, int64_t do_stride_s, int64_t do_stride_h, int64_t dq_stride_b,
                int64_t dq_stride_s, int64_t dq_stride_h, int64_t bf_stride_b, int64_t flags_stride_b,
                int64_t flags_stride_m, int B, int S, int Hq, int Hkv, int D, float scale, int dtype,
-               void* stream);
+               int accumulate, void* stream);
 
 #ifdef __cplusplus
 }
