@@ -32,7 +32,9 @@ def parse():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="C2", choices=["C2", "C3", "C4", "C5"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--traffic", default=None, help="JSON file with measured HBM bytes per launch (from rocprofv3 --pmc)")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="after the timed region, run a plain 1 GiB device copy (reads 1 GiB, writes 1 GiB) so that "
+                         "a rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run of this command also holds a kernel of known traffic")
     return ap.parse_args()
 
 
@@ -68,6 +70,20 @@ def cpu_baseline(name):
         "sample": f"{name} q-heads 0..{G - 1} + kv-head 0" + (", sequence 0" if name == "C4" else "")
         + ", fwd+bwd fp32 materialized-mask SDPA, best of 2",
     }
+
+
+def measured_traffic(workload, kernel):
+    """HBM bytes per launch of `kernel`, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and
+    recorded in profiles/hbm_traffic.txt as lines `<workload> <kernel> <bytes>`; None if absent."""
+    path = os.path.join(ROOT, "profiles", "hbm_traffic.txt")
+    if not os.path.exists(path):
+        return None
+    with open(path) as f:
+        for line in f:
+            parts = line.split()
+            if len(parts) >= 3 and parts[0] == workload and parts[1] == kernel:
+                return float(parts[2])
+    return None
 
 
 def main():
@@ -133,6 +149,14 @@ def main():
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
 
+    if args.copy_calibration:
+        src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
     ms_per_step = wall * 1e3 / args.steps
     stage_ms = {}
     for si, s in enumerate(stages):
@@ -146,10 +170,7 @@ def main():
     kname = {"fwd": "fwd_kernel", "dkdv": "bwd_dkdv_kernel", "dq": "bwd_dq_kernel"}
     dom = max(algo, key=lambda s: stage_ms[s])
     achieved = algo[dom] / (stage_ms[dom] * 1e-3) / 1e12
-    traffic = None
-    if args.traffic and os.path.exists(args.traffic):
-        with open(args.traffic) as f:
-            traffic = json.load(f).get(kname[dom])
+    traffic = measured_traffic(name, kname[dom])
 
     value = (f_fwd + f_bwd) / (ms_per_step * 1e-3) / 1e12
     result = {
