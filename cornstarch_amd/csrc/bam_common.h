@@ -63,6 +63,12 @@ __device__ __forceinline__ bool allow_pair(const QueryBits& q, unsigned klo, uns
     return (nz == q.text) & pos_ok;
 }
 
+// The part of the rule that does not depend on the key's position.
+__device__ __forceinline__ bool allow_bits(const QueryBits& q, unsigned klo, unsigned khi) {
+    const unsigned v = ((klo & q.a_lo) ^ q.x_lo) | ((khi & q.a_hi) ^ q.x_hi);
+    return (v != 0u) == q.text;
+}
+
 // ---------------------------------------------------------------------------------
 // Element types: raw 16-byte operands, MFMA and float -> T conversion.
 struct BF16 {

@@ -1,4 +1,4 @@
-// Global -> register -> LDS tile staging and the flag-driven tile lists shared by the
+// Global -> LDS tile staging and the flag-driven tile lists shared by the
 // forward and backward kernels.
 #pragma once
 #include "bam_common.h"
@@ -6,15 +6,39 @@
 
 namespace bam {
 
+// LDS byte address of a __shared__ object (what the LDS-DMA base register M0 wants).
+__device__ __forceinline__ unsigned lds_addr(const void* p) {
+    return (unsigned)(unsigned long long)(const __attribute__((address_space(3))) void*)p;
+}
+
+// One direct global -> LDS copy instruction.  Lane l fetches `bytes` (16 or 4) from
+// sbase + voff and the hardware writes them to LDS byte address lds_base + l * bytes;
+// sbase and lds_base must be wave-uniform.  Issued as inline asm on purpose: the compiler
+// then neither tracks the copy in vmcnt nor makes later LDS reads wait for it, which is what
+// lets a tile load stay in flight across a whole loop iteration.  The price is that the
+// caller owns the synchronization: wait_async() (or wait_async_but<N>()) + a workgroup
+// barrier before anyone reads the destination.
+__device__ __forceinline__ void dma_b128(const void* sbase, unsigned voff, unsigned lds_base) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_base)
+                 : "memory");
+}
+__device__ __forceinline__ void dma_b32(const void* sbase, unsigned voff, unsigned lds_base) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_base)
+                 : "memory");
+}
+
+// All direct global-to-LDS copies this wave has issued have landed (pair with a barrier).
+__device__ __forceinline__ void wait_async() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
 // ROWS x D tile of 2-byte elements copied global -> LDS by THREADS threads, 16 bytes per lane.
 // Full tiles use the direct global-to-LDS load (no staging registers, no LDS write
 // instructions): a wave's 64 lanes fill 64 consecutive chunk slots of the LDS tile, so the
 // XOR swizzle is applied on the SOURCE side -- lane `id` fetches the chunk that belongs in
-// slot `id`.  `setup` fixes those source offsets once per kernel.  The copy is asynchronous:
-// the caller waits with wait_async() and a workgroup barrier before anyone reads the tile.
-// The last, ragged tile of a sequence takes the synchronous path, which zero-fills the rows
-// past the end.  Row strides are limited to 2^24 elements by the host checks, so the
-// offsets fit 32 bits.
+// slot `id`.  `setup` fixes those source offsets once per kernel; `issue(i, ...)` emits copy
+// instruction i of CPT so that callers can spread a tile's copies between other work.
+// The last, ragged tile of a sequence takes the synchronous path (`load_ragged`), which
+// zero-fills the rows past the end.  Row strides are limited to 2^24 elements by the host
+// checks, so the offsets fit 32 bits.
 template <int D, int ROWS, int THREADS>
 struct TileStage {
     static constexpr int NCH = D / 8;
@@ -22,8 +46,10 @@ struct TileStage {
     static constexpr int CPT = (CHUNKS + THREADS - 1) / THREADS;
     static constexpr bool EXACT = (CHUNKS % THREADS) == 0;
     unsigned goff[CPT];
+    int wave_first;  // first chunk slot this wave fills with instruction 0
 
     __device__ __forceinline__ void setup(int64_t row_stride_bytes, int tid) {
+        wave_first = __builtin_amdgcn_readfirstlane(tid & ~63);
 #pragma unroll
         for (int i = 0; i < CPT; ++i) {
             const int id = tid + THREADS * i;
@@ -31,43 +57,42 @@ struct TileStage {
             goff[i] = (unsigned)(row * row_stride_bytes + (pc ^ swz<D>(row)) * 16);
         }
     }
-    // tile_base: first row of the tile in global memory (wave-uniform); rows_valid: rows of it
-    // inside the sequence (wave-uniform)
-    __device__ __forceinline__ void load(const char* tile_base, u32x4* tile, int rows_valid, int tid) const {
-        typedef __attribute__((address_space(1))) const void* gptr;
-        typedef __attribute__((address_space(3))) void* lptr;
-        if (rows_valid >= ROWS) {
-            const int wave_first = __builtin_amdgcn_readfirstlane(tid & ~63);
+    // tile_base: first row of the tile in global memory, tile_lds: lds_addr() of the LDS tile
+    // (both wave-uniform)
+    __device__ __forceinline__ void issue(int i, const char* tile_base, unsigned tile_lds) const {
+        if (EXACT || wave_first + THREADS * i < CHUNKS)
+            dma_b128(tile_base, goff[i], tile_lds + (unsigned)(THREADS * i + wave_first) * 16u);
+    }
+    __device__ __forceinline__ void load_full(const char* tile_base, unsigned tile_lds) const {
 #pragma unroll
-            for (int i = 0; i < CPT; ++i)
-                if (EXACT || wave_first + THREADS * i < CHUNKS)
-                    __builtin_amdgcn_global_load_lds((gptr)(tile_base + goff[i]),
-                                                     (lptr)(tile + THREADS * i + wave_first), 16, 0, 0);
-        } else {
+        for (int i = 0; i < CPT; ++i) issue(i, tile_base, tile_lds);
+    }
+    // synchronous, zero-filling copy of a tile with only rows_valid (< ROWS) rows in range
+    __device__ __forceinline__ void load_ragged(const char* tile_base, u32x4* tile, int rows_valid, int tid) const {
 #pragma unroll
-            for (int i = 0; i < CPT; ++i) {
-                const int id = tid + THREADS * i;
-                u32x4 z = {0u, 0u, 0u, 0u};
-                if ((EXACT || id < CHUNKS) && id / NCH < rows_valid) z = *(const u32x4*)(tile_base + goff[i]);
-                if (EXACT || id < CHUNKS) tile[id] = z;
-            }
+        for (int i = 0; i < CPT; ++i) {
+            const int id = tid + THREADS * i;
+            u32x4 z = {0u, 0u, 0u, 0u};
+            if ((EXACT || id < CHUNKS) && id / NCH < rows_valid) z = *(const u32x4*)(tile_base + goff[i]);
+            if (EXACT || id < CHUNKS) tile[id] = z;
         }
+    }
+    // tile_base / rows_valid wave-uniform
+    __device__ __forceinline__ void load(const char* tile_base, u32x4* tile, int rows_valid, int tid) const {
+        if (rows_valid >= ROWS)
+            load_full(tile_base, lds_addr(tile));
+        else
+            load_ragged(tile_base, tile, rows_valid, tid);
     }
 };
 
 // One wave copies `DWORDS` consecutive dwords (a multiple of 64) global -> LDS asynchronously.
 template <int DWORDS>
 __device__ __forceinline__ void copy_dwords_async(const void* src, void* dst_lds, int lane) {
-    typedef __attribute__((address_space(1))) const void* gptr;
-    typedef __attribute__((address_space(3))) void* lptr;
+    const unsigned dst = lds_addr(dst_lds);
 #pragma unroll
-    for (int i = 0; i < DWORDS / 64; ++i)
-        __builtin_amdgcn_global_load_lds((gptr)((const unsigned*)src + 64 * i + lane),
-                                         (lptr)((unsigned*)dst_lds + 64 * i), 4, 0, 0);
+    for (int i = 0; i < DWORDS / 64; ++i) dma_b32(src, (unsigned)(lane * 4 + 256 * i), dst + 256u * i);
 }
-
-// All direct global-to-LDS copies this wave has issued have landed (pair with a barrier).
-__device__ __forceinline__ void wait_async() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
 // List, in ascending order, the 64-key tiles a 128-row query block has to visit.
 // entry = (tile << 2) | cls ; cls 1: evaluate the mask, cls 2: every pair allowed.

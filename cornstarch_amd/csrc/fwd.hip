@@ -19,6 +19,7 @@
 #include "bam_common.h"
 #include "bam_launch.h"
 #include "bam_tiles.h"
+#include <type_traits>
 
 namespace bam {
 
@@ -34,7 +35,7 @@ __global__ __launch_bounds__(FWD_THREADS, 2) void fwd_kernel(const AttnParams p)
     __shared__ int sList[MAX_LIST];
     __shared__ int sCount;
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int hi = lane >> 5, l32 = lane & 31, half16 = (lane >> 4) & 1;
     const int S = p.S;
     const int G = p.Hq / p.Hkv;
@@ -90,64 +91,73 @@ __global__ __launch_bounds__(FWD_THREADS, 2) void fwd_kernel(const AttnParams p)
     const int64_t k_ts = 2 * p.k.ss * FWD_KT, v_ts = 2 * p.v.ss * FWD_KT;  // bytes per tile
     const int64_t* bfrow = p.bf + (int64_t)b * p.bf_sb;
 
-    TileStage<D, FWD_KT, FWD_THREADS> stK, stV;
+    typedef TileStage<D, FWD_KT, FWD_THREADS> Stage;
+    constexpr int CPT = Stage::CPT;
+    constexpr int NLOADS = 2 * CPT + 1;  // copy instructions per wave and tile: K, V and the key bitfields
+    static_assert(NLOADS <= 2 * KK + 1, "one copy per MFMA gap");
+    Stage stK, stV;
     stK.setup(2 * p.k.ss, tid);
     stV.setup(2 * p.v.ss, tid);
-    // bitfields of a tile's keys: direct global -> LDS copy by wave 1; the ragged last tile is
-    // staged synchronously with 0 (never allowed) for the keys past the end
-    auto stage_key_bits = [&](int kt, int buf) {
-        if (S - kt * FWD_KT >= FWD_KT) {
-            if (wave == 1) copy_dwords_async<2 * FWD_KT>(bfrow + kt * FWD_KT, sKbf[buf], lane);
-        } else if (tid < FWD_KT) {
-            sKbf[buf][tid] = (kt * FWD_KT + tid < S) ? bfrow[kt * FWD_KT + tid] : 0;
-        }
+    const unsigned ldsK = lds_addr(sK), ldsV = lds_addr(sV), ldsB = lds_addr(sKbf);
+    constexpr unsigned TILE_BYTES = FWD_KT * NCH * 16, BITS_BYTES = FWD_KT * 8;
+    // Copy instruction j (0 <= j < NLOADS) of full tile kt into buffer buf.  The 128 dwords of key
+    // bitfields are copied 64 dwords per wave (waves 2, 3 repeat what waves 0, 1 write), so that every
+    // wave issues the same number of copies.
+    auto issue_copy = [&](int j, int kt, int buf) {
+        if (j < CPT)
+            stK.issue(j, kbase + kt * k_ts, ldsK + buf * TILE_BYTES);
+        else if (j < 2 * CPT)
+            stV.issue(j - CPT, vbase + kt * v_ts, ldsV + buf * TILE_BYTES);
+        else
+            dma_b32(bfrow + kt * FWD_KT, (unsigned)((wave & 1) * 256 + lane * 4), ldsB + buf * BITS_BYTES + (wave & 1) * 256u);
     };
 
-    __syncthreads();
-    const int n = sCount;
-    if (n > 0) {
+    // One 64-key tile held in buffer `cur`.  With PREFETCH the copies of tile `kt_next` into the other
+    // buffer are issued one per MFMA of the S phase, where the wave has nothing else to wait for.
+    auto tile_step = [&](auto prefetch, int cur, int entry, int kt_next) {
+        constexpr bool PREFETCH = decltype(prefetch)::value;
+        const int kt = entry >> 2, cls = entry & 3;
+        const u32x4* tK = sK[cur];
+        const u32x4* tV = sV[cur];
+
+        // ---- S^T = K Q^T : 64 keys x 32 queries per wave ----------------------------------
+        // two independent accumulator chains (key blocks 0 and 1) alternate; operand reads run AHEAD
+        // MFMAs in front of their use; the first MFMA of a chain takes C = 0
+        f32x16 s[2];
         {
-            const int kt = __builtin_amdgcn_readfirstlane(sList[0]) >> 2;
-            stK.load(kbase + kt * k_ts, sK[0], S - kt * FWD_KT, tid);
-            stV.load(vbase + kt * v_ts, sV[0], S - kt * FWD_KT, tid);
-            stage_key_bits(kt, 0);
+            constexpr int NOP = 2 * KK, AHEAD = 4;
+            u32x4 ka[NOP];
+#pragma unroll
+            for (int j = 0; j < AHEAD; ++j) ka[j] = lds_read_chunk<D>(tK, 32 * (j & 1) + l32, 2 * (j >> 1) + hi);
+#pragma unroll
+            for (int j = 0; j < NOP; ++j) {
+                __builtin_amdgcn_sched_barrier(0);
+                if (j + AHEAD < NOP)
+                    ka[j + AHEAD] = lds_read_chunk<D>(tK, 32 * ((j + AHEAD) & 1) + l32, 2 * ((j + AHEAD) >> 1) + hi);
+                s[j & 1] = T::mfma(ka[j], qreg[j >> 1], j < 2 ? zero16 : s[j & 1]);
+                if (PREFETCH && j < NLOADS) issue_copy(j, kt_next, cur ^ 1);
+            }
+            __builtin_amdgcn_sched_barrier(0);
         }
-        wait_async();
-        __syncthreads();
-        for (int it = 0; it < n; ++it) {
-            const int cur = it & 1;
-            const int entry = __builtin_amdgcn_readfirstlane(sList[it]);
-            const int kt = entry >> 2, cls = entry & 3;
-            const bool more = it + 1 < n;
-            if (more) {
-                const int kt1 = __builtin_amdgcn_readfirstlane(sList[it + 1]) >> 2;
-                stK.load(kbase + kt1 * k_ts, sK[cur ^ 1], S - kt1 * FWD_KT, tid);
-                stV.load(vbase + kt1 * v_ts, sV[cur ^ 1], S - kt1 * FWD_KT, tid);
-                stage_key_bits(kt1, cur ^ 1);
-            }
 
-            // ---- S^T = K Q^T : 64 keys x 32 queries per wave ----------------------------
-            // two independent accumulator chains (key blocks 0 and 1) alternate; operand reads
-            // run a few MFMAs ahead of their use; the first MFMA of a chain takes C = 0
-            f32x16 s[2];
-            {
-                u32x4 ka[KK][2];
+        // ---- bitfield rule in registers (partial tiles only) ------------------------------
+        if (cls == 1) {
+            const int kt0 = kt * FWD_KT;
+            // Most partial tiles are partial only through causality: all 64 keys carry the same bitfield.
+            // Then the bit test is a per-query constant and the rule reduces to one position compare.
+            const int64_t mine = sKbf[cur][lane];
+            const unsigned mlo = (unsigned)mine, mhi = (unsigned)((uint64_t)mine >> 32);
+            const unsigned flo = __builtin_amdgcn_readfirstlane(mlo), fhi = __builtin_amdgcn_readfirstlane(mhi);
+            if (__all((mlo == flo) & (mhi == fhi))) {
+                const int rel = allow_bits(qb, flo, fhi) ? qb.lim - kt0 : -1;  // last allowed key, relative to the tile
 #pragma unroll
-                for (int kk = 0; kk < KK; ++kk)
+                for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-                    for (int kb = 0; kb < 2; ++kb) ka[kk][kb] = lds_read_chunk<D>(sK[cur], 32 * kb + l32, 2 * kk + hi);
-#pragma unroll
-                for (int kb = 0; kb < 2; ++kb) s[kb] = T::mfma(ka[0][kb], qreg[0], zero16);
-#pragma unroll
-                for (int kk = 1; kk < KK; ++kk)
-#pragma unroll
-                    for (int kb = 0; kb < 2; ++kb) s[kb] = T::mfma(ka[kk][kb], qreg[kk], s[kb]);
-                sched_pipeline_mfma_lds<2 * KK, 4, 1>();
-            }
-
-            // ---- bitfield rule in registers (partial tiles only) ------------------------
-            if (cls == 1) {
-                const int kt0 = kt * FWD_KT;
+                    for (int i = 0; i < 16; ++i) {
+                        const int koff = 32 * kb + 8 * (i >> 2) + 4 * hi + (i & 3);
+                        s[kb][i] = (koff <= rel) ? s[kb][i] : -INFINITY;
+                    }
+            } else {
 #pragma unroll
                 for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
@@ -164,65 +174,97 @@ __global__ __launch_bounds__(FWD_THREADS, 2) void fwd_kernel(const AttnParams p)
                         }
                     }
             }
+        }
 
-            // ---- online softmax (per-lane scalars) ----------------------------------------
-            float mloc = fmaxf(s[0][0], s[1][0]);
+        // ---- online softmax (per-lane scalars) ----------------------------------------------
+        float mloc = fmaxf(s[0][0], s[1][0]);
 #pragma unroll
-            for (int i = 1; i < 16; ++i) mloc = fmaxf(mloc, fmaxf(s[0][i], s[1][i]));
-            mloc = half_swap_max(mloc);
-            if (__any(mloc > m_i + rescale_thr)) {  // wave-uniform; rare after the first tiles
-                const float mnew = fmaxf(m_i, mloc);
-                const float muse = (mnew == -INFINITY) ? 0.f : mnew;
-                const float alpha = __builtin_amdgcn_exp2f((m_i - muse) * c2);  // 0 when m_i = -inf
-                m_i = mnew;
-                nb = -muse * c2;
-                l_i *= alpha;
+        for (int i = 1; i < 16; ++i) mloc = fmaxf(mloc, fmaxf(s[0][i], s[1][i]));
+        mloc = half_swap_max(mloc);
+        if (__any(mloc > m_i + rescale_thr)) {  // wave-uniform; rare after the first tiles
+            const float mnew = fmaxf(m_i, mloc);
+            const float muse = (mnew == -INFINITY) ? 0.f : mnew;
+            const float alpha = __builtin_amdgcn_exp2f((m_i - muse) * c2);  // 0 when m_i = -inf
+            m_i = mnew;
+            nb = -muse * c2;
+            l_i *= alpha;
 #pragma unroll
-                for (int db = 0; db < DB; ++db)
+            for (int db = 0; db < DB; ++db)
 #pragma unroll
-                    for (int i = 0; i < 16; ++i) o[db][i] *= alpha;
-            }
-            float psum0 = 0.f, psum1 = 0.f;
+                for (int i = 0; i < 16; ++i) o[db][i] *= alpha;
+        }
+        float psum0 = 0.f, psum1 = 0.f;
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const float e0 = __builtin_amdgcn_exp2f(fmaf(s[0][i], c2, nb));
-                const float e1 = __builtin_amdgcn_exp2f(fmaf(s[1][i], c2, nb));
-                s[0][i] = e0;
-                s[1][i] = e1;
-                psum0 += e0;
-                psum1 += e1;
-            }
-            l_i += psum0 + psum1;
+        for (int i = 0; i < 16; ++i) {
+            const float e0 = __builtin_amdgcn_exp2f(fmaf(s[0][i], c2, nb));
+            const float e1 = __builtin_amdgcn_exp2f(fmaf(s[1][i], c2, nb));
+            s[0][i] = e0;
+            s[1][i] = e1;
+            psum0 += e0;
+            psum1 += e1;
+        }
+        l_i += psum0 + psum1;
 
-            u32x4 pb[2][2];
+        u32x4 pb[2][2];
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int t = 0; t < 2; ++t) pb[kb][t] = pack8<T>(s[kb], 8 * t);
+
+        // ---- O^T += V^T P^T -------------------------------------------------------------------
+        {
+            u32x4 va[2][2][DB];
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-                for (int t = 0; t < 2; ++t) pb[kb][t] = pack8<T>(s[kb], 8 * t);
+                for (int t = 0; t < 2; ++t)
+#pragma unroll
+                    for (int db = 0; db < DB; ++db)
+                        va[kb][t][db] = lds_read_transposed<D>(tV, lane, 32 * kb + 16 * t + 4 * hi, 32 * db + 16 * half16);
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+#pragma unroll
+                    for (int db = 0; db < DB; ++db) o[db] = T::mfma(va[kb][t][db], pb[kb][t], o[db]);
+            sched_pipeline_mfma_lds<4 * DB, (DB >= 2 ? 3 : 2), 2>();
+        }
+    };
 
-            // ---- O^T += V^T P^T ---------------------------------------------------------------
-            {
-                u32x4 va[2][2][DB];
+    __syncthreads();
+    const int n_all = sCount;
+    // A tile that holds the end of a sequence whose length is not a multiple of 64 is always the last
+    // entry of the list; it is staged synchronously (zero fill past the end) after the main loop.
+    const bool ragged = (S & (FWD_KT - 1)) != 0 && n_all > 0 &&
+                        (__builtin_amdgcn_readfirstlane(sList[n_all > 0 ? n_all - 1 : 0]) >> 2) == ((S - 1) >> 6);
+    const int n = n_all - (ragged ? 1 : 0);
+    if (n > 0) {
+        int entry = __builtin_amdgcn_readfirstlane(sList[0]);
+        int next = __builtin_amdgcn_readfirstlane(sList[n > 1 ? 1 : 0]);
 #pragma unroll
-                for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-                    for (int t = 0; t < 2; ++t)
-#pragma unroll
-                        for (int db = 0; db < DB; ++db)
-                            va[kb][t][db] = lds_read_transposed<D>(sV[cur], lane, 32 * kb + 16 * t + 4 * hi,
-                                                                   32 * db + 16 * half16);
-#pragma unroll
-                for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-                    for (int t = 0; t < 2; ++t)
-#pragma unroll
-                        for (int db = 0; db < DB; ++db) o[db] = T::mfma(va[kb][t][db], pb[kb][t], o[db]);
-                sched_pipeline_mfma_lds<4 * DB, (DB >= 2 ? 3 : 2), 2>();
-            }
-
+        for (int j = 0; j < NLOADS; ++j) issue_copy(j, entry >> 2, 0);
+        wait_async();
+        __syncthreads();
+        for (int it = 0; it < n; ++it) {
+            const int cur = it & 1;
+            // entry after next, requested now and picked up at the end of the iteration; past the end of the
+            // list the last tile is simply copied again (into the buffer nobody reads any more)
+            const int after = sList[it + 2 < n ? it + 2 : n - 1];
+            tile_step(std::true_type{}, cur, entry, next >> 2);
+            entry = next;
+            next = __builtin_amdgcn_readfirstlane(after);
             wait_async();
             __syncthreads();
         }
+    }
+    if (ragged) {
+        const int entry = __builtin_amdgcn_readfirstlane(sList[n_all - 1]);
+        const int kt = entry >> 2, rows = S - kt * FWD_KT;
+        stK.load_ragged(kbase + kt * k_ts, sK[0], rows, tid);
+        stV.load_ragged(vbase + kt * v_ts, sV[0], rows, tid);
+        if (tid < FWD_KT) sKbf[0][tid] = (tid < rows) ? bfrow[kt * FWD_KT + tid] : 0;
+        __syncthreads();
+        tile_step(std::false_type{}, 0, entry, 0);
     }
 
     // ---- epilogue: normalize, write O (q dtype) and LSE (natural log) -------------------
