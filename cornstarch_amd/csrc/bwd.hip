@@ -10,6 +10,7 @@
 #include "bam_common.h"
 #include "bam_launch.h"
 #include "bam_tiles.h"
+#include <type_traits>
 
 namespace bam {
 
@@ -74,7 +75,7 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
     __shared__ int sList[MAX_LIST / 2];
     __shared__ int sCount;
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int kg = wave & 3, st = wave >> 2;
     const int hi = lane >> 5, l32 = lane & 31, half16 = (lane >> 4) & 1;
     const int S = p.S;
@@ -120,159 +121,246 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
     for (int i = 0; i < 16; ++i) zero16[i] = 0.f;
     const float c2 = p.scale * LOG2E;
 
-    TileStage<D, DKDV_QT, DKDV_THREADS> stQ, stDO;
+    typedef TileStage<D, DKDV_QT, DKDV_THREADS> Stage;
+    constexpr int CPT = Stage::CPT;
+    constexpr int NLOADS = 2 * CPT + 1;  // copy instructions per wave and tile: Q, dO and one of the four small rows
+    static_assert(NLOADS <= 2 * KK + 1, "one copy per MFMA gap");
+    Stage stQ, stDO;
     stQ.setup(2 * p.q.ss, tid);
     stDO.setup(2 * p.dout.ss, tid);
+    const unsigned ldsQ = lds_addr(sQ), ldsDO = lds_addr(sDO);
+    constexpr unsigned TILE_BYTES = DKDV_QT * NCH * 16;
+    // small rows of a tile: lse, delta and the two halves of the 64 int64 bitfields, 64 dwords each;
+    // wave w copies row w & 3 (waves 4..7 repeat what waves 0..3 write, so that every wave issues the same
+    // number of copies)
+    const int small = wave & 3;
+    const unsigned ldsSmall = small == 0 ? lds_addr(sLse) : small == 1 ? lds_addr(sDelta) : lds_addr(sQbf) + (small - 2) * 256u;
+    const unsigned smallBytes = small < 2 ? DKDV_QT * 4u : DKDV_QT * 8u;  // per buffer
+    // Copy instruction j of the full 64-row tile (head h, first row row0) into buffer buf.
+    auto issue_copy = [&](int j, int h, int row0, int buf) {
+        if (j < CPT) {
+            const char* qbase = (const char*)p.q.ptr + 2 * ((int64_t)b * p.q.sb + (int64_t)h * p.q.sh + (int64_t)row0 * p.q.ss);
+            stQ.issue(j, qbase, ldsQ + buf * TILE_BYTES);
+        } else if (j < 2 * CPT) {
+            const char* gbase = (const char*)p.dout.ptr + 2 * ((int64_t)b * p.dout.sb + (int64_t)h * p.dout.sh + (int64_t)row0 * p.dout.ss);
+            stDO.issue(j - CPT, gbase, ldsDO + buf * TILE_BYTES);
+        } else {
+            const int64_t off = ((int64_t)b * p.Hq + h) * p.S_rounded + row0;
+            const void* src = small == 0 ? (const void*)(p.lse + off)
+                              : small == 1 ? (const void*)(p.delta + off)
+                                           : (const void*)((const char*)(bfrow + row0) + (small - 2) * 256);
+            dma_b32(src, (unsigned)(lane * 4), ldsSmall + buf * smallBytes);
+        }
+    };
 
-    // iteration `it` -> (q head of the group, list entry, 64-row half of the 128-row block).
-    // Query blocks are visited from the LAST one down: the workgroups of one kv head that are
-    // resident together then read the same Q / dO tile at about the same time, and all but the
-    // first of them find it in L2.
-    auto list_at = [&](int rem, int n) { return __builtin_amdgcn_readfirstlane(sList[n - 1 - (rem >> 1)]); };
-    auto tile_row0 = [&](int rem, int n) { return (list_at(rem, n) >> 8) * BLOCK_M + (1 - (rem & 1)) * DKDV_QT; };
-    // Everything a tile needs (Q, dO rows, their lse, delta and bitfields) is copied global -> LDS
-    // without passing through registers; only the ragged last tile of a sequence is staged
-    // synchronously, with neutral values for the rows past the end (lse = +inf gives P = 0).
-    auto stage = [&](int it, int n, int buf) {
-        const int g = it / (2 * n);
-        const int row0 = tile_row0(it - g * 2 * n, n);
-        const int h = hk * G + g;
-        const char* qbase = (const char*)p.q.ptr + 2 * ((int64_t)b * p.q.sb + (int64_t)h * p.q.sh);
-        const char* gbase = (const char*)p.dout.ptr + 2 * ((int64_t)b * p.dout.sb + (int64_t)h * p.dout.sh);
-        stQ.load(qbase + (int64_t)row0 * 2 * p.q.ss, sQ[buf], S - row0, tid);
-        stDO.load(gbase + (int64_t)row0 * 2 * p.dout.ss, sDO[buf], S - row0, tid);
-        const int64_t off = ((int64_t)b * p.Hq + h) * p.S_rounded + row0;
-        if (S - row0 >= DKDV_QT) {
-            if (wave == 1) copy_dwords_async<DKDV_QT>(p.lse + off, sLse[buf], lane);
-            if (wave == 2) copy_dwords_async<DKDV_QT>(p.delta + off, sDelta[buf], lane);
-            if (wave == 3) copy_dwords_async<2 * DKDV_QT>(bfrow + row0, sQbf[buf], lane);
-        } else if (tid < DKDV_QT) {
-            const bool ok = row0 + tid < S;
-            sLse[buf][tid] = ok ? p.lse[off + tid] : INFINITY;
-            sDelta[buf][tid] = ok ? p.delta[off + tid] : 0.f;
-            sQbf[buf][tid] = ok ? bfrow[row0 + tid] : 0;
+    // One 64-row tile (rows row0.., held in buffer cur) against this wave's 32 keys.  With PREFETCH the
+    // copies of the next tile (head h_next, rows row0_next..) into the other buffer are issued one per MFMA
+    // of the S / dP phase, or back to back when this wave's own flag says there is nothing to compute.
+    const int qr = 32 * st;  // this wave's rows inside the 64-row tile
+    // The wave's flag class is extracted with a per-lane copy of the key group number on purpose: a branch
+    // condition the compiler can prove wave-uniform makes it restructure the loop around that branch, and the
+    // result needs far more registers than a wave has.
+    const int kg_lane = (tid >> 6) & 3;
+    auto tile_step = [&](auto prefetch, int cur, int cls, int row0, int h_next, int row0_next) {
+        constexpr bool PREFETCH = decltype(prefetch)::value;
+        if (cls == 0) {
+            if (PREFETCH) {
+#pragma unroll
+                for (int j = 0; j < NLOADS; ++j) issue_copy(j, h_next, row0_next, cur ^ 1);
+            }
+            return;
+        }
+        const u32x4* tQ = sQ[cur];
+        const u32x4* tG = sDO[cur];
+        // ---- S = Q K^T and dP = dO V^T : 32 queries x 32 keys, two accumulator chains; both operands of
+        // every MFMA come from LDS and are requested AHEAD MFMAs in front of their use
+        f32x16 s, dp;
+        {
+            constexpr int NOP = 2 * KK, AHEAD = 2;  // MFMA j: S (j even) or dP (j odd), k-slice j / 2
+            u32x4 a[NOP], bb[NOP];
+#pragma unroll
+            for (int j = 0; j < AHEAD; ++j) {
+                a[j] = lds_read_chunk<D>((j & 1) ? tG : tQ, qr + l32, 2 * (j >> 1) + hi);
+                bb[j] = lds_read_chunk<D>((j & 1) ? sV : sK, 32 * kg + l32, 2 * (j >> 1) + hi);
+            }
+#pragma unroll
+            for (int j = 0; j < NOP; ++j) {
+                __builtin_amdgcn_sched_barrier(0);
+                if (j + AHEAD < NOP) {
+                    a[j + AHEAD] = lds_read_chunk<D>(((j + AHEAD) & 1) ? tG : tQ, qr + l32, 2 * ((j + AHEAD) >> 1) + hi);
+                    bb[j + AHEAD] = lds_read_chunk<D>(((j + AHEAD) & 1) ? sV : sK, 32 * kg + l32, 2 * ((j + AHEAD) >> 1) + hi);
+                }
+                if (j & 1)
+                    dp = T::mfma(a[j], bb[j], j < 2 ? zero16 : dp);
+                else
+                    s = T::mfma(a[j], bb[j], j < 2 ? zero16 : s);
+                if (PREFETCH && j < NLOADS) issue_copy(j, h_next, row0_next, cur ^ 1);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // ---- P = exp(scale s - lse) on allowed pairs, dS/scale = P (dP - delta)   (the factor `scale` of dS
+        // is applied once to dK in the epilogue).  C fragment: register i <-> query row
+        // 8*(i/4) + 4*hi + i%4 of this wave's 32 rows.
+#pragma unroll
+        for (int grp = 0; grp < 4; ++grp) {
+            const f32x4 l4 = *(const f32x4*)&sLse[cur][qr + 8 * grp + 4 * hi];
+#pragma unroll
+            for (int x = 0; x < 4; ++x) s[4 * grp + x] = __builtin_amdgcn_exp2f(fmaf(s[4 * grp + x], c2, l4[x] * -LOG2E));
+        }
+        if (cls == 1) {
+            // Most partial tiles are partial only through causality: the 32 rows carry the same bitfield.
+            // Then the bit test is a per-key constant and the rule reduces to one position compare.
+            const int64_t mine = sQbf[cur][qr + l32];
+            const unsigned mlo = (unsigned)mine, mhi = (unsigned)((uint64_t)mine >> 32);
+            const unsigned flo = __builtin_amdgcn_readfirstlane(mlo), fhi = __builtin_amdgcn_readfirstlane(mhi);
+            if (__all((mlo == flo) & (mhi == fhi))) {
+                const QueryBits qu = make_query_bits(((int64_t)fhi << 32) | (int64_t)flo, 0);
+                const bool ok = allow_bits(qu, klo, khi) & (qu.text | (qu.lim >= 0));
+                // allowed iff krel <= 8 * grp + x  (text rows: key position <= row position)
+                const int krel = !ok ? 0x7FFFFFFF : qu.text ? key - (row0 + qr) - 4 * hi : (int)0x80000000;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) s[i] = (krel <= 8 * (i >> 2) + (i & 3)) ? s[i] : 0.f;
+            } else {
+                // rule constants of this wave's 32 rows, derived once per row (lane r < 32 takes row r) and
+                // handed to all lanes through a wave-private LDS scratch
+                {
+                    const QueryBits qb = make_query_bits(mine, row0 + qr + l32);
+                    if (hi == 0) {
+                        sWq[wave][0][l32] = qb.a_lo;
+                        sWq[wave][1][l32] = qb.a_hi;
+                        sWq[wave][2][l32] = qb.x_lo;
+                        sWq[wave][3][l32] = qb.x_hi;
+                        sWq[wave][4][l32] = (unsigned)qb.lim;
+                    }
+                }
+#pragma unroll
+                for (int grp = 0; grp < 4; ++grp) {
+                    const int roff = 8 * grp + 4 * hi;
+                    const u32x4 qalo = *(const u32x4*)&sWq[wave][0][roff];
+                    const u32x4 qahi = *(const u32x4*)&sWq[wave][1][roff];
+                    const u32x4 qxlo = *(const u32x4*)&sWq[wave][2][roff];
+                    const u32x4 qxhi = *(const u32x4*)&sWq[wave][3][roff];
+                    const u32x4 qlim = *(const u32x4*)&sWq[wave][4][roff];
+#pragma unroll
+                    for (int x = 0; x < 4; ++x) {
+                        QueryBits qb;
+                        qb.a_lo = qalo[x];
+                        qb.a_hi = qahi[x];
+                        qb.x_lo = qxlo[x];
+                        qb.x_hi = qxhi[x];
+                        qb.lim = (int)qlim[x];
+                        qb.text = qlim[x] < 0x7FFFFFFFu;  // text rows carry their position, modality rows INT_MAX or -1
+                        s[4 * grp + x] = allow_pair(qb, klo, khi, key) ? s[4 * grp + x] : 0.f;
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int grp = 0; grp < 4; ++grp) {
+            const f32x4 d4 = *(const f32x4*)&sDelta[cur][qr + 8 * grp + 4 * hi];
+#pragma unroll
+            for (int x = 0; x < 4; ++x) dp[4 * grp + x] = s[4 * grp + x] * (dp[4 * grp + x] - d4[x]);
+        }
+        u32x4 pb[2], dsb[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            pb[t] = pack8<T>(s, 8 * t);
+            dsb[t] = pack8<T>(dp, 8 * t);
+        }
+        // ---- dV^T += dO^T P ; dK^T += Q^T dS -------------------------------------------------
+        {
+            u32x4 tg[2][DB], tq[2][DB];
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int db = 0; db < DB; ++db) {
+                    tg[t][db] = lds_read_transposed<D>(tG, lane, qr + 16 * t + 4 * hi, 32 * db + 16 * half16);
+                    tq[t][db] = lds_read_transposed<D>(tQ, lane, qr + 16 * t + 4 * hi, 32 * db + 16 * half16);
+                }
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int db = 0; db < DB; ++db) {
+                    dv[db] = T::mfma(tg[t][db], pb[t], dv[db]);
+                    dk[db] = T::mfma(tq[t][db], dsb[t], dk[db]);
+                }
+            sched_pipeline_mfma_lds<4 * DB, 3, 2>();
         }
     };
 
     __syncthreads();
-    const int n = sCount;
+    const int n_all = sCount;
+    // The last 128-row block of a sequence whose length is not a multiple of 128 (always the last list entry)
+    // is staged synchronously, with neutral values for the rows past the end, after the main loop.
+    const bool ragged = (S & (BLOCK_M - 1)) != 0 && n_all > 0 &&
+                        (__builtin_amdgcn_readfirstlane(sList[n_all > 0 ? n_all - 1 : 0]) >> 8) == p.num_m - 1;
+    const int n = n_all - (ragged ? 1 : 0);
+    // Main loop: tiles t = 0 .. 2 n G - 1 -> (q head g of the group, list entry, 64-row half).  Query blocks are
+    // visited from the LAST one down: the workgroups of one kv head that are resident together then read the
+    // same Q / dO tile at about the same time, and all but the first of them find it in L2.
     const int total = n * 2 * G;
     if (total > 0) {
-        stage(0, n, 0);
+        // (g, r) of the tile being computed and of the next two tiles; r counts 0 .. 2n-1 inside a head
+        auto entry_of = [&](int r) { return sList[n - 1 - (r >> 1)]; };
+        auto row0_of = [&](int entry, int r) { return (entry >> 8) * BLOCK_M + (1 - (r & 1)) * DKDV_QT; };
+        int g_cur = 0, r_cur = 0;
+        int g_nxt = 0, r_nxt = 1;  // 2 n >= 2, so tile 1 is in head 0
+        int entry = __builtin_amdgcn_readfirstlane(entry_of(0));
+        int next = __builtin_amdgcn_readfirstlane(entry_of(1));
+#pragma unroll
+        for (int j = 0; j < NLOADS; ++j) issue_copy(j, hk * G, row0_of(entry, 0), 0);
         wait_async();
         __syncthreads();
-        const int qr = 32 * st;  // this wave's rows inside the 64-row tile
         for (int it = 0; it < total; ++it) {
             const int cur = it & 1;
-            if (it + 1 < total) stage(it + 1, n, cur ^ 1);
-
-            const int rem = it % (2 * n);
-            const int entry = list_at(rem, n);
-            const int cls = (entry >> (2 * kg)) & 3;  // this wave's own 128x32 flag
-            if (cls != 0) {
-                // ---- S = Q K^T and dP = dO V^T : 32 queries x 32 keys; both operands of every MFMA
-                // come from LDS and are requested a few MFMAs ahead of their use
-                f32x16 s, dp;
-                {
-                    u32x4 aq[KK], ag[KK], bk[KK], bv[KK];
-#pragma unroll
-                    for (int kk = 0; kk < KK; ++kk) {
-                        aq[kk] = lds_read_chunk<D>(sQ[cur], qr + l32, 2 * kk + hi);
-                        bk[kk] = lds_read_chunk<D>(sK, 32 * kg + l32, 2 * kk + hi);
-                        ag[kk] = lds_read_chunk<D>(sDO[cur], qr + l32, 2 * kk + hi);
-                        bv[kk] = lds_read_chunk<D>(sV, 32 * kg + l32, 2 * kk + hi);
-                    }
-                    s = T::mfma(aq[0], bk[0], zero16);
-                    dp = T::mfma(ag[0], bv[0], zero16);
-#pragma unroll
-                    for (int kk = 1; kk < KK; ++kk) {
-                        s = T::mfma(aq[kk], bk[kk], s);
-                        dp = T::mfma(ag[kk], bv[kk], dp);
-                    }
-                    sched_pipeline_mfma_lds<2 * KK, 2, 2>();
-                }
-                // ---- P = exp(scale s - lse), dS/scale = P (dP - delta)   (the factor `scale` of dS
-                // is applied once to dK in the epilogue).  C fragment: register i <-> query row
-                // 8*(i/4) + 4*hi + i%4 of this wave's 32 rows.
-#pragma unroll
-                for (int grp = 0; grp < 4; ++grp) {
-                    const int roff = qr + 8 * grp + 4 * hi;
-                    const f32x4 l4 = *(const f32x4*)&sLse[cur][roff];
-                    const f32x4 d4 = *(const f32x4*)&sDelta[cur][roff];
-#pragma unroll
-                    for (int x = 0; x < 4; ++x) {
-                        const float e = __builtin_amdgcn_exp2f(fmaf(s[4 * grp + x], c2, l4[x] * -LOG2E));
-                        s[4 * grp + x] = e;
-                        dp[4 * grp + x] = e * (dp[4 * grp + x] - d4[x]);
-                    }
-                }
-                if (cls == 1) {
-                    // rule constants of this wave's 32 rows, derived once per row (lane r < 32 takes
-                    // row r) and handed to all lanes through a wave-private LDS scratch
-                    {
-                        const int row0 = tile_row0(rem, n);
-                        const QueryBits qb = make_query_bits(sQbf[cur][qr + l32], row0 + qr + l32);
-                        if (hi == 0) {
-                            sWq[wave][0][l32] = qb.a_lo;
-                            sWq[wave][1][l32] = qb.a_hi;
-                            sWq[wave][2][l32] = qb.x_lo;
-                            sWq[wave][3][l32] = qb.x_hi;
-                            sWq[wave][4][l32] = (unsigned)qb.lim;
-                        }
-                    }
-#pragma unroll
-                    for (int grp = 0; grp < 4; ++grp) {
-                        const int roff = 8 * grp + 4 * hi;
-                        const u32x4 qalo = *(const u32x4*)&sWq[wave][0][roff];
-                        const u32x4 qahi = *(const u32x4*)&sWq[wave][1][roff];
-                        const u32x4 qxlo = *(const u32x4*)&sWq[wave][2][roff];
-                        const u32x4 qxhi = *(const u32x4*)&sWq[wave][3][roff];
-                        const u32x4 qlim = *(const u32x4*)&sWq[wave][4][roff];
-#pragma unroll
-                        for (int x = 0; x < 4; ++x) {
-                            QueryBits qb;
-                            qb.a_lo = qalo[x];
-                            qb.a_hi = qahi[x];
-                            qb.x_lo = qxlo[x];
-                            qb.x_hi = qxhi[x];
-                            qb.lim = (int)qlim[x];
-                            qb.text = qlim[x] < 0x7FFFFFFFu;  // text rows carry their position, modality rows INT_MAX or -1
-                            const bool a = allow_pair(qb, klo, khi, key);
-                            s[4 * grp + x] = a ? s[4 * grp + x] : 0.f;
-                            dp[4 * grp + x] = a ? dp[4 * grp + x] : 0.f;
-                        }
-                    }
-                }
-                u32x4 pb[2], dsb[2];
-#pragma unroll
-                for (int t = 0; t < 2; ++t) {
-                    pb[t] = pack8<T>(s, 8 * t);
-                    dsb[t] = pack8<T>(dp, 8 * t);
-                }
-                // ---- dV^T += dO^T P ; dK^T += Q^T dS -------------------------------------------
-                {
-                    u32x4 tg[2][DB], tq[2][DB];
-#pragma unroll
-                    for (int t = 0; t < 2; ++t)
-#pragma unroll
-                        for (int db = 0; db < DB; ++db) {
-                            tg[t][db] = lds_read_transposed<D>(sDO[cur], lane, qr + 16 * t + 4 * hi, 32 * db + 16 * half16);
-                            tq[t][db] = lds_read_transposed<D>(sQ[cur], lane, qr + 16 * t + 4 * hi, 32 * db + 16 * half16);
-                        }
-#pragma unroll
-                    for (int t = 0; t < 2; ++t)
-#pragma unroll
-                        for (int db = 0; db < DB; ++db) {
-                            dv[db] = T::mfma(tg[t][db], pb[t], dv[db]);
-                            dk[db] = T::mfma(tq[t][db], dsb[t], dk[db]);
-                        }
-                    sched_pipeline_mfma_lds<4 * DB, 3, 2>();
-                }
+            // tile after next: its list entry is requested now and picked up at the end of the iteration
+            int g_aft = g_nxt, r_aft = r_nxt + 1;
+            if (r_aft == 2 * n) {
+                r_aft = 0;
+                ++g_aft;
             }
+            const int after = entry_of(g_aft < G ? r_aft : 0);
+            // past the last tile the copies simply fetch it again (into the buffer nobody reads any more)
+            const bool more = it + 1 < total;
+            const int h_next = hk * G + (more ? g_nxt : g_cur);
+            const int row0_next = more ? row0_of(next, r_nxt) : row0_of(entry, r_cur);
+            tile_step(std::true_type{}, cur, (entry >> (2 * kg_lane)) & 3, row0_of(entry, r_cur), h_next, row0_next);
+            g_cur = g_nxt;
+            r_cur = r_nxt;
+            g_nxt = g_aft;
+            r_nxt = r_aft;
+            entry = next;
+            next = __builtin_amdgcn_readfirstlane(after);
             wait_async();
             __syncthreads();
         }
     }
+    if (ragged) {
+        wait_async();  // K, V of the tile, in case the main loop had nothing to do
+        const int entry = __builtin_amdgcn_readfirstlane(sList[n_all - 1]);
+        for (int t = 0; t < 2 * G; ++t) {
+            const int g = t >> 1;
+            const int row0 = (entry >> 8) * BLOCK_M + (t & 1) * DKDV_QT;
+            const int rows = S - row0;  // rows of the tile inside the sequence
+            if (rows <= 0) continue;
+            const int h = hk * G + g;
+            __syncthreads();  // everybody is done with buffer 0
+            stQ.load_ragged((const char*)p.q.ptr + 2 * ((int64_t)b * p.q.sb + (int64_t)h * p.q.sh + (int64_t)row0 * p.q.ss), sQ[0], rows, tid);
+            stDO.load_ragged((const char*)p.dout.ptr + 2 * ((int64_t)b * p.dout.sb + (int64_t)h * p.dout.sh + (int64_t)row0 * p.dout.ss), sDO[0], rows, tid);
+            if (tid < DKDV_QT) {
+                const int64_t off = ((int64_t)b * p.Hq + h) * p.S_rounded + row0;
+                const bool ok = tid < rows;
+                sLse[0][tid] = ok ? p.lse[off + tid] : INFINITY;  // lse = +inf gives P = 0
+                sDelta[0][tid] = ok ? p.delta[off + tid] : 0.f;
+                sQbf[0][tid] = ok ? bfrow[row0 + tid] : 0;
+            }
+            __syncthreads();
+            tile_step(std::false_type{}, 0, (entry >> (2 * kg_lane)) & 3, row0, 0, 0);
+        }
+    }
+    // every copy has landed and every wave is done with the tiles: the epilogue reuses the tile arrays
+    wait_async();
+    __syncthreads();
 
     // ---- epilogue.  The two waves of a key group hold partial sums.
     if (p.grad_typed) {
@@ -360,7 +448,7 @@ __global__ __launch_bounds__(DQ_THREADS, 2) void bwd_dq_kernel(const AttnParams 
     __shared__ int sList[MAX_LIST];
     __shared__ int sCount;
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int hi = lane >> 5, l32 = lane & 31, half16 = (lane >> 4) & 1;
     const int S = p.S;
     const int G = p.Hq / p.Hkv;
@@ -409,6 +497,9 @@ __global__ __launch_bounds__(DQ_THREADS, 2) void bwd_dq_kernel(const AttnParams 
     for (int db = 0; db < DB; ++db)
 #pragma unroll
         for (int i = 0; i < 16; ++i) dq[db][i] = 0.f;
+    f32x16 zero16;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) zero16[i] = 0.f;
     const float c2 = p.scale * LOG2E;
 
     const char* kbase = (const char*)p.k.ptr + 2 * ((int64_t)b * p.k.sb + (int64_t)hk * p.k.sh);
@@ -416,69 +507,78 @@ __global__ __launch_bounds__(DQ_THREADS, 2) void bwd_dq_kernel(const AttnParams 
     const int64_t k_ts = 2 * p.k.ss * DQ_KT, v_ts = 2 * p.v.ss * DQ_KT;  // bytes per tile
     const int64_t* bfrow = p.bf + (int64_t)b * p.bf_sb;
 
-    TileStage<D, DQ_KT, DQ_THREADS> stK, stV;
+    typedef TileStage<D, DQ_KT, DQ_THREADS> Stage;
+    constexpr int CPT = Stage::CPT;
+    constexpr int NLOADS = 2 * CPT + 1;  // copy instructions per wave and tile: K, V and the key bitfields
+    static_assert(NLOADS <= 2 * KK + 1, "one copy per MFMA gap");
+    Stage stK, stV;
     stK.setup(2 * p.k.ss, tid);
     stV.setup(2 * p.v.ss, tid);
-    // bitfields of a tile's keys: direct global -> LDS copy by wave 1; the ragged last tile is
-    // staged synchronously with 0 (never allowed) for the keys past the end
-    auto stage_key_bits = [&](int kt, int buf) {
-        if (S - kt * DQ_KT >= DQ_KT) {
-            if (wave == 1) copy_dwords_async<2 * DQ_KT>(bfrow + kt * DQ_KT, sKbf[buf], lane);
-        } else if (tid < DQ_KT) {
-            sKbf[buf][tid] = (kt * DQ_KT + tid < S) ? bfrow[kt * DQ_KT + tid] : 0;
-        }
+    const unsigned ldsK = lds_addr(sK), ldsV = lds_addr(sV), ldsB = lds_addr(sKbf);
+    constexpr unsigned TILE_BYTES = DQ_KT * NCH * 16, BITS_BYTES = DQ_KT * 8;
+    // copy instruction j of full tile kt into buffer buf (key bitfields: 64 dwords per wave, waves 2, 3
+    // repeat what waves 0, 1 write, so that every wave issues the same number of copies)
+    auto issue_copy = [&](int j, int kt, int buf) {
+        if (j < CPT)
+            stK.issue(j, kbase + kt * k_ts, ldsK + buf * TILE_BYTES);
+        else if (j < 2 * CPT)
+            stV.issue(j - CPT, vbase + kt * v_ts, ldsV + buf * TILE_BYTES);
+        else
+            dma_b32(bfrow + kt * DQ_KT, (unsigned)((wave & 1) * 256 + lane * 4), ldsB + buf * BITS_BYTES + (wave & 1) * 256u);
     };
 
-    __syncthreads();
-    const int n = sCount;
-    if (n > 0) {
-        {
-            const int kt = __builtin_amdgcn_readfirstlane(sList[0]) >> 2;
-            stK.load(kbase + kt * k_ts, sK[0], S - kt * DQ_KT, tid);
-            stV.load(vbase + kt * v_ts, sV[0], S - kt * DQ_KT, tid);
-            stage_key_bits(kt, 0);
+    // One 64-key tile held in buffer `cur`; with PREFETCH the copies of tile kt_next into the other buffer
+    // are issued one per MFMA of the first S / dP block.
+    auto tile_step = [&](auto prefetch, int cur, int entry, int kt_next) {
+        constexpr bool PREFETCH = decltype(prefetch)::value;
+        const int kt = entry >> 2, cls = entry & 3;
+        const u32x4* tK = sK[cur];
+        const u32x4* tV = sV[cur];
+        // partial tile whose 64 keys all carry the same bitfield: the rule is one position compare
+        bool uniform_keys = false;
+        int rel = 0;
+        if (cls == 1) {
+            const int64_t mine = sKbf[cur][lane];
+            const unsigned mlo = (unsigned)mine, mhi = (unsigned)((uint64_t)mine >> 32);
+            const unsigned flo = __builtin_amdgcn_readfirstlane(mlo), fhi = __builtin_amdgcn_readfirstlane(mhi);
+            uniform_keys = __all((mlo == flo) & (mhi == fhi));
+            rel = allow_bits(qb, flo, fhi) ? qb.lim - kt * DQ_KT : -1;  // last allowed key, relative to the tile
         }
-        wait_async();
-        __syncthreads();
-        for (int it = 0; it < n; ++it) {
-            const int cur = it & 1;
-            const int entry = __builtin_amdgcn_readfirstlane(sList[it]);
-            const int kt = entry >> 2, cls = entry & 3;
-            const bool more = it + 1 < n;
-            if (more) {
-                const int kt1 = __builtin_amdgcn_readfirstlane(sList[it + 1]) >> 2;
-                stK.load(kbase + kt1 * k_ts, sK[cur ^ 1], S - kt1 * DQ_KT, tid);
-                stV.load(vbase + kt1 * v_ts, sV[cur ^ 1], S - kt1 * DQ_KT, tid);
-                stage_key_bits(kt1, cur ^ 1);
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) {
+            // ---- S^T = K Q^T and dP^T = V dO^T : 32 keys x 32 queries, two accumulator chains
+            f32x16 s, dp;
+            {
+                constexpr int NOP = 2 * KK, AHEAD = 4;  // operand j: K chunk (j even) or V chunk (j odd) of k-slice j / 2
+                u32x4 a[NOP];
+#pragma unroll
+                for (int j = 0; j < AHEAD; ++j) a[j] = lds_read_chunk<D>((j & 1) ? tV : tK, 32 * kb + l32, 2 * (j >> 1) + hi);
+#pragma unroll
+                for (int j = 0; j < NOP; ++j) {
+                    __builtin_amdgcn_sched_barrier(0);
+                    if (j + AHEAD < NOP)
+                        a[j + AHEAD] = lds_read_chunk<D>(((j + AHEAD) & 1) ? tV : tK, 32 * kb + l32, 2 * ((j + AHEAD) >> 1) + hi);
+                    if (j & 1)
+                        dp = T::mfma(a[j], greg[j >> 1], j < 2 ? zero16 : dp);
+                    else
+                        s = T::mfma(a[j], qreg[j >> 1], j < 2 ? zero16 : s);
+                    if (PREFETCH && kb == 0 && j < NLOADS) issue_copy(j, kt_next, cur ^ 1);
+                }
+                __builtin_amdgcn_sched_barrier(0);
             }
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb) {
-                f32x16 s, dp;
+            for (int i = 0; i < 16; ++i) {
+                const float e = __builtin_amdgcn_exp2f(fmaf(s[i], c2, -lse2));
+                dp[i] = e * (dp[i] - dlt);  // the factor `scale` of dS is applied to dQ in the epilogue
+            }
+            if (cls == 1) {
+                if (uniform_keys) {
 #pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    s[i] = 0.f;
-                    dp[i] = 0.f;
-                }
-                {
-                    u32x4 ka[KK], va[KK];
-#pragma unroll
-                    for (int kk = 0; kk < KK; ++kk) {
-                        ka[kk] = lds_read_chunk<D>(sK[cur], 32 * kb + l32, 2 * kk + hi);
-                        va[kk] = lds_read_chunk<D>(sV[cur], 32 * kb + l32, 2 * kk + hi);
+                    for (int i = 0; i < 16; ++i) {
+                        const int koff = 32 * kb + 8 * (i >> 2) + 4 * hi + (i & 3);
+                        dp[i] = (koff <= rel) ? dp[i] : 0.f;
                     }
-#pragma unroll
-                    for (int kk = 0; kk < KK; ++kk) {
-                        s = T::mfma(ka[kk], qreg[kk], s);
-                        dp = T::mfma(va[kk], greg[kk], dp);
-                    }
-                    sched_pipeline_mfma_lds<2 * KK, 4, 1>();
-                }
-#pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    const float e = __builtin_amdgcn_exp2f(fmaf(s[i], c2, -lse2));
-                    dp[i] = e * (dp[i] - dlt);  // the factor `scale` of dS is applied to dQ in the epilogue
-                }
-                if (cls == 1) {
+                } else {
                     const int kt0 = kt * DQ_KT;
 #pragma unroll
                     for (int grp = 0; grp < 4; ++grp) {
@@ -492,27 +592,61 @@ __global__ __launch_bounds__(DQ_THREADS, 2) void bwd_dq_kernel(const AttnParams 
                             dp[4 * grp + x] = allow_pair(qb, klo[x], khi[x], kt0 + koff + x) ? dp[4 * grp + x] : 0.f;
                     }
                 }
-                u32x4 dsb[2];
-#pragma unroll
-                for (int t = 0; t < 2; ++t) dsb[t] = pack8<T>(dp, 8 * t);
-                {
-                    u32x4 ta[2][DB];
-#pragma unroll
-                    for (int t = 0; t < 2; ++t)
-#pragma unroll
-                        for (int db = 0; db < DB; ++db)
-                            ta[t][db] = lds_read_transposed<D>(sK[cur], lane, 32 * kb + 16 * t + 4 * hi,
-                                                               32 * db + 16 * half16);
-#pragma unroll
-                    for (int t = 0; t < 2; ++t)
-#pragma unroll
-                        for (int db = 0; db < DB; ++db) dq[db] = T::mfma(ta[t][db], dsb[t], dq[db]);
-                    sched_pipeline_mfma_lds<2 * DB, 2, 2>();
-                }
             }
+            u32x4 dsb[2];
+#pragma unroll
+            for (int t = 0; t < 2; ++t) dsb[t] = pack8<T>(dp, 8 * t);
+            // ---- dQ^T += K^T dS^T
+            {
+                u32x4 ta[2][DB];
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+#pragma unroll
+                    for (int db = 0; db < DB; ++db)
+                        ta[t][db] = lds_read_transposed<D>(tK, lane, 32 * kb + 16 * t + 4 * hi, 32 * db + 16 * half16);
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+#pragma unroll
+                    for (int db = 0; db < DB; ++db) dq[db] = T::mfma(ta[t][db], dsb[t], dq[db]);
+                sched_pipeline_mfma_lds<2 * DB, 2, 2>();
+            }
+        }
+    };
+
+    __syncthreads();
+    const int n_all = sCount;
+    // A tile that holds the end of a sequence whose length is not a multiple of 64 is always the last
+    // entry of the list; it is staged synchronously (zero fill past the end) after the main loop.
+    const bool ragged = (S & (DQ_KT - 1)) != 0 && n_all > 0 &&
+                        (__builtin_amdgcn_readfirstlane(sList[n_all > 0 ? n_all - 1 : 0]) >> 2) == ((S - 1) >> 6);
+    const int n = n_all - (ragged ? 1 : 0);
+    if (n > 0) {
+        int entry = __builtin_amdgcn_readfirstlane(sList[0]);
+        int next = __builtin_amdgcn_readfirstlane(sList[n > 1 ? 1 : 0]);
+#pragma unroll
+        for (int j = 0; j < NLOADS; ++j) issue_copy(j, entry >> 2, 0);
+        wait_async();
+        __syncthreads();
+        for (int it = 0; it < n; ++it) {
+            const int cur = it & 1;
+            // entry after next, requested now and picked up at the end of the iteration; past the end of the
+            // list the last tile is simply copied again (into the buffer nobody reads any more)
+            const int after = sList[it + 2 < n ? it + 2 : n - 1];
+            tile_step(std::true_type{}, cur, entry, next >> 2);
+            entry = next;
+            next = __builtin_amdgcn_readfirstlane(after);
             wait_async();
             __syncthreads();
         }
+    }
+    if (ragged) {
+        const int entry = __builtin_amdgcn_readfirstlane(sList[n_all - 1]);
+        const int kt = entry >> 2, rows = S - kt * DQ_KT;
+        stK.load_ragged(kbase + kt * k_ts, sK[0], rows, tid);
+        stV.load_ragged(vbase + kt * v_ts, sV[0], rows, tid);
+        if (tid < DQ_KT) sKbf[0][tid] = (tid < rows) ? bfrow[kt * DQ_KT + tid] : 0;
+        __syncthreads();
+        tile_step(std::false_type{}, 0, entry, 0);
     }
 
     if (qvalid && p.grad_typed) {  // overwrite mode: dq has the input dtype
