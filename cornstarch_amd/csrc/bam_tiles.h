@@ -18,12 +18,19 @@ __device__ __forceinline__ unsigned lds_addr(const void* p) {
 // lets a tile load stay in flight across a whole loop iteration.  The price is that the
 // caller owns the synchronization: wait_async() (or wait_async_but<N>()) + a workgroup
 // barrier before anyone reads the destination.
+// SITE only labels the instruction (as an assembler comment): copies issued from different places of a
+// kernel get different labels, which keeps the compiler from merging them into one hoisted copy and so
+// keeps each where the schedule wants it.
+template <int SITE = 0>
 __device__ __forceinline__ void dma_b128(const void* sbase, unsigned voff, unsigned lds_base) {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_base)
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 ; site %3" ::"v"(voff), "s"(sbase),
+                 "s"(lds_base), "n"(SITE)
                  : "memory");
 }
+template <int SITE = 0>
 __device__ __forceinline__ void dma_b32(const void* sbase, unsigned voff, unsigned lds_base) {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_base)
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1 ; site %3" ::"v"(voff), "s"(sbase),
+                 "s"(lds_base), "n"(SITE)
                  : "memory");
 }
 
@@ -59,9 +66,10 @@ struct TileStage {
     }
     // tile_base: first row of the tile in global memory, tile_lds: lds_addr() of the LDS tile
     // (both wave-uniform)
+    template <int SITE = 0>
     __device__ __forceinline__ void issue(int i, const char* tile_base, unsigned tile_lds) const {
         if (EXACT || wave_first + THREADS * i < CHUNKS)
-            dma_b128(tile_base, goff[i], tile_lds + (unsigned)(THREADS * i + wave_first) * 16u);
+            dma_b128<SITE>(tile_base, goff[i], tile_lds + (unsigned)(THREADS * i + wave_first) * 16u);
     }
     __device__ __forceinline__ void load_full(const char* tile_base, unsigned tile_lds) const {
 #pragma unroll

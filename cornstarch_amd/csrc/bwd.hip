@@ -105,8 +105,11 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
     const bool kvalid = key < S;
     const int64_t* bfrow = p.bf + (int64_t)b * p.bf_sb;
     const int64_t kf = kvalid ? bfrow[key] : 0;
-    const unsigned klo = (unsigned)(kf & 0xFFFFFFFFll);
-    const unsigned khi = (unsigned)((uint64_t)kf >> 32);
+    unsigned klo = (unsigned)(kf & 0xFFFFFFFFll);
+    unsigned khi = (unsigned)((uint64_t)kf >> 32);
+    // Pin the arrival of this load here.  Left alone, the compiler waits for it at the first use inside the
+    // main loop, with a vmcnt that also (and every time round) drains the tile copies it does not know about.
+    asm volatile("" : "+v"(klo), "+v"(khi));
 
     f32x16 dk[DB], dv[DB];
 #pragma unroll
