@@ -41,15 +41,19 @@ int check_f32_tensor(const char* name, const void* ptr, int64_t sb, int64_t ss, 
     return BAM_OK;
 }
 
-int check_problem(int B, int S, int Hq, int Hkv, int D, int dtype) {
-    if (B <= 0 || S <= 0 || Hq <= 0 || Hkv <= 0)
-        return fail(BAM_ERR_INVALID_ARGUMENT, "B, S, Hq, Hkv must be positive (got %d, %d, %d, %d)", B, S, Hq, Hkv);
+int check_problem(int B, int Sq, int Sk, int Hq, int Hkv, int D, int dtype) {
+    if (B <= 0 || Sq <= 0 || Sk <= 0 || Hq <= 0 || Hkv <= 0)
+        return fail(BAM_ERR_INVALID_ARGUMENT, "B, S, Hq, Hkv must be positive (got B %d, Sq %d, Sk %d, Hq %d, Hkv %d)", B,
+                    Sq, Sk, Hq, Hkv);
     if (Hq % Hkv) return fail(BAM_ERR_INVALID_ARGUMENT, "Hq (%d) must be a multiple of Hkv (%d)", Hq, Hkv);
     if (D != 32 && D != 64 && D != 128)
         return fail(BAM_ERR_UNSUPPORTED, "head dimension %d is not supported (32, 64 or 128)", D);
     if (dtype != BAM_DTYPE_F16 && dtype != BAM_DTYPE_BF16)
         return fail(BAM_ERR_INVALID_ARGUMENT, "dtype %d is neither BAM_DTYPE_F16 nor BAM_DTYPE_BF16", dtype);
-    if (S > BAM_MAX_SEQLEN) return fail(BAM_ERR_UNSUPPORTED, "S = %d exceeds BAM_MAX_SEQLEN = %d", S, BAM_MAX_SEQLEN);
+    if (Sq > BAM_MAX_SEQLEN || Sk > BAM_MAX_SEQLEN)
+        return fail(BAM_ERR_UNSUPPORTED, "S = %d exceeds BAM_MAX_SEQLEN = %d", Sq > Sk ? Sq : Sk, BAM_MAX_SEQLEN);
+    if ((int64_t)((Sq + 127) / 128) * B * Hq > 0x7FFFFFFFll || (int64_t)((Sk + 127) / 128) * B * Hkv > 0x7FFFFFFFll)
+        return fail(BAM_ERR_UNSUPPORTED, "grid too large");
     return BAM_OK;
 }
 
@@ -59,17 +63,57 @@ int launched(int hip_err, const char* what) {
     return BAM_OK;
 }
 
-void fill_sizes(bam::AttnParams& p, int B, int S, int Hq, int Hkv, int D, float scale) {
+// Where the kernels find bitfields and positions: one (B, S) tensor for plain attention, gathered
+// per-row / per-key arrays plus positions for index-tensor attention.
+struct MaskSource {
+    const int64_t *bfq, *bfk;
+    int64_t bfq_sb, bfk_sb;
+    const int *posq, *posk;
+    int Sq, Sk;
+};
+
+MaskSource plain_source(const int64_t* bf, int64_t bf_stride_b, int S) {
+    return MaskSource{bf, bf, bf_stride_b, bf_stride_b, nullptr, nullptr, S, S};
+}
+
+int indexed_source(const bam_index_view* iv, MaskSource& m) {
+    if (iv == nullptr) return fail(BAM_ERR_INVALID_ARGUMENT, "index view: null pointer");
+    if (iv->q_bits == nullptr || iv->k_bits == nullptr || iv->q_pos == nullptr || iv->k_pos == nullptr)
+        return fail(BAM_ERR_INVALID_ARGUMENT, "index view: q_bits, k_bits, q_pos and k_pos must not be null");
+    if ((reinterpret_cast<uintptr_t>(iv->q_bits) & 7u) || (reinterpret_cast<uintptr_t>(iv->k_bits) & 7u) ||
+        (reinterpret_cast<uintptr_t>(iv->q_pos) & 3u) || (reinterpret_cast<uintptr_t>(iv->k_pos) & 3u))
+        return fail(BAM_ERR_INVALID_ARGUMENT, "index view: misaligned array");
+    m = MaskSource{iv->q_bits, iv->k_bits, iv->q_bits_stride_b, iv->k_bits_stride_b, iv->q_pos, iv->k_pos, iv->Sq, iv->Sk};
+    return BAM_OK;
+}
+
+void fill_sizes(bam::AttnParams& p, const MaskSource& m, int B, int Hq, int Hkv, int D, float scale) {
+    p.bfq = m.bfq;
+    p.bfk = m.bfk;
+    p.bfq_sb = m.bfq_sb;
+    p.bfk_sb = m.bfk_sb;
+    p.posq = m.posq;
+    p.posk = m.posk;
     p.B = B;
-    p.S = S;
+    p.Sq = m.Sq;
+    p.Sk = m.Sk;
     p.Hq = Hq;
     p.Hkv = Hkv;
     p.D = D;
-    p.num_m = (S + 127) / 128;
-    p.num_n = (S + 31) / 32;
-    p.S_rounded = p.num_m * 128;
+    p.num_m = (m.Sq + 127) / 128;
+    p.num_n = (m.Sk + 31) / 32;
+    p.num_kt = (m.Sk + 127) / 128;
+    p.Sq_rounded = p.num_m * 128;
     p.scale = scale;
 }
+
+int fwd_impl(const char* who, const void* q, const void* k, const void* v, void* o, float* lse, const MaskSource& m,
+             const int8_t* flags, const int64_t* st, int64_t flags_stride_b, int64_t flags_stride_m, int B, int Hq,
+             int Hkv, int D, float scale, int dtype, void* stream);
+int bwd_params(bam::AttnParams& p, const char* who, const void* q, const void* k, const void* v, const void* dout,
+               const float* lse, const float* delta, void* dq, void* dk, void* dv, const MaskSource& m,
+               const int8_t* flags, const int64_t* st, int B, int Hq, int Hkv, int D, float scale, int dtype,
+               int accumulate, bool need_dq, bool need_dkdv);
 
 }  // namespace
 
@@ -79,11 +123,82 @@ void fill_sizes(bam::AttnParams& p, int B, int S, int Hq, int Hkv, int D, float 
         if (rc_ != BAM_OK) return rc_; \
     } while (0)
 
+namespace {
+
+int fwd_impl(const char* who, const void* q, const void* k, const void* v, void* o, float* lse, const MaskSource& m,
+             const int8_t* flags, const int64_t* st, int64_t flags_stride_b, int64_t flags_stride_m, int B, int Hq,
+             int Hkv, int D, float scale, int dtype, void* stream) {
+    BAM_TRY(check_problem(B, m.Sq, m.Sk, Hq, Hkv, D, dtype));
+    BAM_TRY(check_half_tensor("q", q, st[0], st[1], st[2]));
+    BAM_TRY(check_half_tensor("k", k, st[3], st[4], st[5]));
+    BAM_TRY(check_half_tensor("v", v, st[6], st[7], st[8]));
+    BAM_TRY(check_half_tensor("o", o, st[9], st[10], st[11]));
+    if (lse == nullptr || m.bfq == nullptr || m.bfk == nullptr || flags == nullptr)
+        return fail(BAM_ERR_INVALID_ARGUMENT, "%s: lse, bitfields and flags must not be null", who);
+    if (!(scale > 0.f)) return fail(BAM_ERR_INVALID_ARGUMENT, "%s: softmax scale must be > 0 (got %g)", who, scale);
+    bam::AttnParams p = {};
+    p.q = {q, st[0], st[1], st[2]};
+    p.k = {k, st[3], st[4], st[5]};
+    p.v = {v, st[6], st[7], st[8]};
+    p.o = {o, st[9], st[10], st[11]};
+    p.lse = lse;
+    p.flags = flags;
+    p.flags_sb = flags_stride_b;
+    p.flags_sm = flags_stride_m;
+    fill_sizes(p, m, B, Hq, Hkv, D, scale);
+    return launched(bam::launch_fwd(p, dtype, (hipStream_t)stream), who);
+}
+
+// st: strides of q, k, v, do, dq, dk, dv (3 each), then flags_stride_b, flags_stride_m
+int bwd_params(bam::AttnParams& p, const char* who, const void* q, const void* k, const void* v, const void* dout,
+               const float* lse, const float* delta, void* dq, void* dk, void* dv, const MaskSource& m,
+               const int8_t* flags, const int64_t* st, int B, int Hq, int Hkv, int D, float scale, int dtype,
+               int accumulate, bool need_dq, bool need_dkdv) {
+    BAM_TRY(check_problem(B, m.Sq, m.Sk, Hq, Hkv, D, dtype));
+    BAM_TRY(check_half_tensor("q", q, st[0], st[1], st[2]));
+    BAM_TRY(check_half_tensor("k", k, st[3], st[4], st[5]));
+    BAM_TRY(check_half_tensor("v", v, st[6], st[7], st[8]));
+    BAM_TRY(check_half_tensor("do", dout, st[9], st[10], st[11]));
+    if (accumulate) {
+        if (need_dq) BAM_TRY(check_f32_tensor("dq", dq, st[12], st[13], st[14]));
+        if (need_dkdv) {
+            BAM_TRY(check_f32_tensor("dk", dk, st[15], st[16], st[17]));
+            BAM_TRY(check_f32_tensor("dv", dv, st[18], st[19], st[20]));
+        }
+    } else {
+        if (need_dq) BAM_TRY(check_half_tensor("dq", dq, st[12], st[13], st[14]));
+        if (need_dkdv) {
+            BAM_TRY(check_half_tensor("dk", dk, st[15], st[16], st[17]));
+            BAM_TRY(check_half_tensor("dv", dv, st[18], st[19], st[20]));
+        }
+    }
+    p.grad_typed = accumulate ? 0 : 1;
+    if (lse == nullptr || delta == nullptr || m.bfq == nullptr || m.bfk == nullptr || flags == nullptr)
+        return fail(BAM_ERR_INVALID_ARGUMENT, "%s: lse, delta, bitfields and flags must not be null", who);
+    if (!(scale > 0.f)) return fail(BAM_ERR_INVALID_ARGUMENT, "%s: softmax scale must be > 0 (got %g)", who, scale);
+    p.q = {q, st[0], st[1], st[2]};
+    p.k = {k, st[3], st[4], st[5]};
+    p.v = {v, st[6], st[7], st[8]};
+    p.dout = {dout, st[9], st[10], st[11]};
+    p.dq = {dq, st[12], st[13], st[14]};
+    p.dk = {dk, st[15], st[16], st[17]};
+    p.dv = {dv, st[18], st[19], st[20]};
+    p.lse = const_cast<float*>(lse);
+    p.delta = const_cast<float*>(delta);
+    p.flags = flags;
+    p.flags_sb = st[21];
+    p.flags_sm = st[22];
+    fill_sizes(p, m, B, Hq, Hkv, D, scale);
+    return BAM_OK;
+}
+
+}  // namespace
+
 extern "C" {
 
 const char* bam_last_error(void) { return g_error; }
 
-int bam_abi_version(void) { return 2; }
+int bam_abi_version(void) { return 3; }
 
 int bam_tile_flags(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int64_t flags_stride_b,
                    int64_t flags_stride_m, int B, int S, void* stream) {
@@ -105,40 +220,49 @@ int bam_materialize_mask(const int64_t* bf, int64_t bf_stride_b, uint8_t* out, i
                     "bam_materialize_mask");
 }
 
+int bam_gather_bitfields(const int64_t* bf, int64_t bf_stride_b, int L, const int64_t* idx, int n, int64_t* out_bits,
+                         int64_t out_stride_b, int32_t* out_pos, int B, void* stream) {
+    if (bf == nullptr || idx == nullptr || out_bits == nullptr || out_pos == nullptr)
+        return fail(BAM_ERR_INVALID_ARGUMENT, "bam_gather_bitfields: null pointer");
+    if (B <= 0 || L <= 0 || n <= 0) return fail(BAM_ERR_INVALID_ARGUMENT, "bam_gather_bitfields: B, L and n must be positive");
+    if (B > 65535) return fail(BAM_ERR_UNSUPPORTED, "bam_gather_bitfields: B is limited to 65535 (got %d)", B);
+    return launched(bam::launch_gather_bitfields(bf, bf_stride_b, L, idx, n, out_bits, out_stride_b, out_pos, B,
+                                                 (hipStream_t)stream),
+                    "bam_gather_bitfields");
+}
+
+#define BAM_FWD_STRIDES                                                                                     \
+    {q_stride_b, q_stride_s, q_stride_h, k_stride_b, k_stride_s, k_stride_h, v_stride_b, v_stride_s, v_stride_h, \
+     o_stride_b, o_stride_s, o_stride_h}
+
 int bam_fwd(const void* q, const void* k, const void* v, void* o, float* lse, const int64_t* bf,
             const int8_t* flags, int64_t q_stride_b, int64_t q_stride_s, int64_t q_stride_h,
             int64_t k_stride_b, int64_t k_stride_s, int64_t k_stride_h, int64_t v_stride_b,
             int64_t v_stride_s, int64_t v_stride_h, int64_t o_stride_b, int64_t o_stride_s,
             int64_t o_stride_h, int64_t bf_stride_b, int64_t flags_stride_b, int64_t flags_stride_m, int B,
             int S, int Hq, int Hkv, int D, float scale, int dtype, void* stream) {
-    BAM_TRY(check_problem(B, S, Hq, Hkv, D, dtype));
-    BAM_TRY(check_half_tensor("q", q, q_stride_b, q_stride_s, q_stride_h));
-    BAM_TRY(check_half_tensor("k", k, k_stride_b, k_stride_s, k_stride_h));
-    BAM_TRY(check_half_tensor("v", v, v_stride_b, v_stride_s, v_stride_h));
-    BAM_TRY(check_half_tensor("o", o, o_stride_b, o_stride_s, o_stride_h));
-    if (lse == nullptr || bf == nullptr || flags == nullptr)
-        return fail(BAM_ERR_INVALID_ARGUMENT, "bam_fwd: lse, bf and flags must not be null");
-    if (!(scale > 0.f)) return fail(BAM_ERR_INVALID_ARGUMENT, "bam_fwd: softmax scale must be > 0 (got %g)", scale);
-    if ((int64_t)((S + 127) / 128) * B * Hq > 0x7FFFFFFFll) return fail(BAM_ERR_UNSUPPORTED, "bam_fwd: grid too large");
-    bam::AttnParams p = {};
-    p.q = {q, q_stride_b, q_stride_s, q_stride_h};
-    p.k = {k, k_stride_b, k_stride_s, k_stride_h};
-    p.v = {v, v_stride_b, v_stride_s, v_stride_h};
-    p.o = {o, o_stride_b, o_stride_s, o_stride_h};
-    p.lse = lse;
-    p.bf = bf;
-    p.bf_sb = bf_stride_b;
-    p.flags = flags;
-    p.flags_sb = flags_stride_b;
-    p.flags_sm = flags_stride_m;
-    fill_sizes(p, B, S, Hq, Hkv, D, scale);
-    return launched(bam::launch_fwd(p, dtype, (hipStream_t)stream), "bam_fwd");
+    const int64_t st[12] = BAM_FWD_STRIDES;
+    return fwd_impl("bam_fwd", q, k, v, o, lse, plain_source(bf, bf_stride_b, S), flags, st, flags_stride_b,
+                    flags_stride_m, B, Hq, Hkv, D, scale, dtype, stream);
+}
+
+int bam_fwd_indexed(const void* q, const void* k, const void* v, void* o, float* lse, const bam_index_view* iv,
+                    const int8_t* flags, int64_t q_stride_b, int64_t q_stride_s, int64_t q_stride_h,
+                    int64_t k_stride_b, int64_t k_stride_s, int64_t k_stride_h, int64_t v_stride_b,
+                    int64_t v_stride_s, int64_t v_stride_h, int64_t o_stride_b, int64_t o_stride_s,
+                    int64_t o_stride_h, int64_t flags_stride_b, int64_t flags_stride_m, int B, int Hq, int Hkv,
+                    int D, float scale, int dtype, void* stream) {
+    MaskSource m;
+    BAM_TRY(indexed_source(iv, m));
+    const int64_t st[12] = BAM_FWD_STRIDES;
+    return fwd_impl("bam_fwd_indexed", q, k, v, o, lse, m, flags, st, flags_stride_b, flags_stride_m, B, Hq, Hkv, D,
+                    scale, dtype, stream);
 }
 
 int bam_bwd_preprocess(const void* o, const void* dout, float* delta, int64_t o_stride_b, int64_t o_stride_s,
                        int64_t o_stride_h, int64_t do_stride_b, int64_t do_stride_s, int64_t do_stride_h,
                        int B, int S, int Hq, int D, int dtype, void* stream) {
-    BAM_TRY(check_problem(B, S, Hq, Hq, D, dtype));
+    BAM_TRY(check_problem(B, S, S, Hq, Hq, D, dtype));
     BAM_TRY(check_half_tensor("o", o, o_stride_b, o_stride_s, o_stride_h));
     BAM_TRY(check_half_tensor("do", dout, do_stride_b, do_stride_s, do_stride_h));
     if (delta == nullptr) return fail(BAM_ERR_INVALID_ARGUMENT, "bam_bwd_preprocess: delta must not be null");
@@ -146,59 +270,14 @@ int bam_bwd_preprocess(const void* o, const void* dout, float* delta, int64_t o_
     p.o = {o, o_stride_b, o_stride_s, o_stride_h};
     p.dout = {dout, do_stride_b, do_stride_s, do_stride_h};
     p.delta = delta;
-    fill_sizes(p, B, S, Hq, Hq, D, 1.f);
+    fill_sizes(p, plain_source(nullptr, 0, S), B, Hq, Hq, D, 1.f);
     return launched(bam::launch_bwd_preprocess(p, dtype, (hipStream_t)stream), "bam_bwd_preprocess");
-}
-
-static int bwd_params(bam::AttnParams& p, const void* q, const void* k, const void* v, const void* dout,
-                      const float* lse, const float* delta, void* dq, void* dk, void* dv, const int64_t* bf,
-                      const int8_t* flags, const int64_t* st, int B, int S, int Hq, int Hkv, int D, float scale,
-                      int dtype, int accumulate, bool need_dq, bool need_dkdv) {
-    BAM_TRY(check_problem(B, S, Hq, Hkv, D, dtype));
-    BAM_TRY(check_half_tensor("q", q, st[0], st[1], st[2]));
-    BAM_TRY(check_half_tensor("k", k, st[3], st[4], st[5]));
-    BAM_TRY(check_half_tensor("v", v, st[6], st[7], st[8]));
-    BAM_TRY(check_half_tensor("do", dout, st[9], st[10], st[11]));
-    if (accumulate) {
-        if (need_dq) BAM_TRY(check_f32_tensor("dq", dq, st[12], st[13], st[14]));
-        if (need_dkdv) {
-            BAM_TRY(check_f32_tensor("dk", dk, st[15], st[16], st[17]));
-            BAM_TRY(check_f32_tensor("dv", dv, st[18], st[19], st[20]));
-        }
-    } else {
-        if (need_dq) BAM_TRY(check_half_tensor("dq", dq, st[12], st[13], st[14]));
-        if (need_dkdv) {
-            BAM_TRY(check_half_tensor("dk", dk, st[15], st[16], st[17]));
-            BAM_TRY(check_half_tensor("dv", dv, st[18], st[19], st[20]));
-        }
-    }
-    p.grad_typed = accumulate ? 0 : 1;
-    if (lse == nullptr || delta == nullptr || bf == nullptr || flags == nullptr)
-        return fail(BAM_ERR_INVALID_ARGUMENT, "bam_bwd: lse, delta, bf and flags must not be null");
-    if (!(scale > 0.f)) return fail(BAM_ERR_INVALID_ARGUMENT, "bam_bwd: softmax scale must be > 0 (got %g)", scale);
-    if ((int64_t)((S + 127) / 128) * B * Hq > 0x7FFFFFFFll) return fail(BAM_ERR_UNSUPPORTED, "bam_bwd: grid too large");
-    p.q = {q, st[0], st[1], st[2]};
-    p.k = {k, st[3], st[4], st[5]};
-    p.v = {v, st[6], st[7], st[8]};
-    p.dout = {dout, st[9], st[10], st[11]};
-    p.dq = {dq, st[12], st[13], st[14]};
-    p.dk = {dk, st[15], st[16], st[17]};
-    p.dv = {dv, st[18], st[19], st[20]};
-    p.lse = const_cast<float*>(lse);
-    p.delta = const_cast<float*>(delta);
-    p.bf = bf;
-    p.bf_sb = st[21];
-    p.flags = flags;
-    p.flags_sb = st[22];
-    p.flags_sm = st[23];
-    fill_sizes(p, B, S, Hq, Hkv, D, scale);
-    return BAM_OK;
 }
 
 #define BAM_BWD_STRIDES                                                                                      \
     {q_stride_b,  q_stride_s,  q_stride_h,  k_stride_b,  k_stride_s,  k_stride_h,  v_stride_b,  v_stride_s,  \
      v_stride_h,  do_stride_b, do_stride_s, do_stride_h, dq_stride_b, dq_stride_s, dq_stride_h, dk_stride_b, \
-     dk_stride_s, dk_stride_h, dv_stride_b, dv_stride_s, dv_stride_h, bf_stride_b, flags_stride_b, flags_stride_m}
+     dk_stride_s, dk_stride_h, dv_stride_b, dv_stride_s, dv_stride_h, flags_stride_b, flags_stride_m}
 
 int bam_bwd(const void* q, const void* k, const void* v, const void* dout, const float* lse,
             const float* delta, void* dq, void* dk, void* dv, const int64_t* bf, const int8_t* flags,
@@ -209,9 +288,10 @@ int bam_bwd(const void* q, const void* k, const void* v, const void* dout, const
             int64_t dk_stride_s, int64_t dk_stride_h, int64_t dv_stride_b, int64_t dv_stride_s,
             int64_t dv_stride_h, int64_t bf_stride_b, int64_t flags_stride_b, int64_t flags_stride_m, int B,
             int S, int Hq, int Hkv, int D, float scale, int dtype, int accumulate, void* stream) {
-    const int64_t st[24] = BAM_BWD_STRIDES;
+    const int64_t st[23] = BAM_BWD_STRIDES;
     bam::AttnParams p = {};
-    BAM_TRY(bwd_params(p, q, k, v, dout, lse, delta, dq, dk, dv, bf, flags, st, B, S, Hq, Hkv, D, scale, dtype, accumulate, true, true));
+    BAM_TRY(bwd_params(p, "bam_bwd", q, k, v, dout, lse, delta, dq, dk, dv, plain_source(bf, bf_stride_b, S), flags, st, B,
+                       Hq, Hkv, D, scale, dtype, accumulate, true, true));
     BAM_TRY(launched(bam::launch_bwd_dkdv(p, dtype, (hipStream_t)stream), "bam_bwd (dk/dv)"));
     return launched(bam::launch_bwd_dq(p, dtype, (hipStream_t)stream), "bam_bwd (dq)");
 }
@@ -227,9 +307,10 @@ int bam_bwd_dkdv(const void* q, const void* k, const void* v, const void* dout, 
                  int accumulate, void* stream) {
     void* dq = nullptr;
     const int64_t dq_stride_b = 0, dq_stride_s = 0, dq_stride_h = 0;
-    const int64_t st[24] = BAM_BWD_STRIDES;
+    const int64_t st[23] = BAM_BWD_STRIDES;
     bam::AttnParams p = {};
-    BAM_TRY(bwd_params(p, q, k, v, dout, lse, delta, dq, dk, dv, bf, flags, st, B, S, Hq, Hkv, D, scale, dtype, accumulate, false, true));
+    BAM_TRY(bwd_params(p, "bam_bwd_dkdv", q, k, v, dout, lse, delta, dq, dk, dv, plain_source(bf, bf_stride_b, S), flags,
+                       st, B, Hq, Hkv, D, scale, dtype, accumulate, false, true));
     return launched(bam::launch_bwd_dkdv(p, dtype, (hipStream_t)stream), "bam_bwd_dkdv");
 }
 
@@ -243,10 +324,49 @@ int bam_bwd_dq(const void* q, const void* k, const void* v, const void* dout, co
                int accumulate, void* stream) {
     void *dk = nullptr, *dv = nullptr;
     const int64_t dk_stride_b = 0, dk_stride_s = 0, dk_stride_h = 0, dv_stride_b = 0, dv_stride_s = 0, dv_stride_h = 0;
-    const int64_t st[24] = BAM_BWD_STRIDES;
+    const int64_t st[23] = BAM_BWD_STRIDES;
     bam::AttnParams p = {};
-    BAM_TRY(bwd_params(p, q, k, v, dout, lse, delta, dq, dk, dv, bf, flags, st, B, S, Hq, Hkv, D, scale, dtype, accumulate, true, false));
+    BAM_TRY(bwd_params(p, "bam_bwd_dq", q, k, v, dout, lse, delta, dq, dk, dv, plain_source(bf, bf_stride_b, S), flags, st,
+                       B, Hq, Hkv, D, scale, dtype, accumulate, true, false));
     return launched(bam::launch_bwd_dq(p, dtype, (hipStream_t)stream), "bam_bwd_dq");
+}
+
+int bam_bwd_dkdv_indexed(const void* q, const void* k, const void* v, const void* dout, const float* lse,
+                         const float* delta, void* dk, void* dv, const bam_index_view* iv, const int8_t* flags,
+                         int64_t q_stride_b, int64_t q_stride_s, int64_t q_stride_h, int64_t k_stride_b,
+                         int64_t k_stride_s, int64_t k_stride_h, int64_t v_stride_b, int64_t v_stride_s,
+                         int64_t v_stride_h, int64_t do_stride_b, int64_t do_stride_s, int64_t do_stride_h,
+                         int64_t dk_stride_b, int64_t dk_stride_s, int64_t dk_stride_h, int64_t dv_stride_b,
+                         int64_t dv_stride_s, int64_t dv_stride_h, int64_t flags_stride_b, int64_t flags_stride_m,
+                         int B, int Hq, int Hkv, int D, float scale, int dtype, int accumulate, void* stream) {
+    MaskSource m;
+    BAM_TRY(indexed_source(iv, m));
+    void* dq = nullptr;
+    const int64_t dq_stride_b = 0, dq_stride_s = 0, dq_stride_h = 0;
+    const int64_t st[23] = BAM_BWD_STRIDES;
+    bam::AttnParams p = {};
+    BAM_TRY(bwd_params(p, "bam_bwd_dkdv_indexed", q, k, v, dout, lse, delta, dq, dk, dv, m, flags, st, B, Hq, Hkv, D, scale,
+                       dtype, accumulate, false, true));
+    return launched(bam::launch_bwd_dkdv(p, dtype, (hipStream_t)stream), "bam_bwd_dkdv_indexed");
+}
+
+int bam_bwd_dq_indexed(const void* q, const void* k, const void* v, const void* dout, const float* lse,
+                       const float* delta, void* dq, const bam_index_view* iv, const int8_t* flags,
+                       int64_t q_stride_b, int64_t q_stride_s, int64_t q_stride_h, int64_t k_stride_b,
+                       int64_t k_stride_s, int64_t k_stride_h, int64_t v_stride_b, int64_t v_stride_s,
+                       int64_t v_stride_h, int64_t do_stride_b, int64_t do_stride_s, int64_t do_stride_h,
+                       int64_t dq_stride_b, int64_t dq_stride_s, int64_t dq_stride_h, int64_t flags_stride_b,
+                       int64_t flags_stride_m, int B, int Hq, int Hkv, int D, float scale, int dtype,
+                       int accumulate, void* stream) {
+    MaskSource m;
+    BAM_TRY(indexed_source(iv, m));
+    void *dk = nullptr, *dv = nullptr;
+    const int64_t dk_stride_b = 0, dk_stride_s = 0, dk_stride_h = 0, dv_stride_b = 0, dv_stride_s = 0, dv_stride_h = 0;
+    const int64_t st[23] = BAM_BWD_STRIDES;
+    bam::AttnParams p = {};
+    BAM_TRY(bwd_params(p, "bam_bwd_dq_indexed", q, k, v, dout, lse, delta, dq, dk, dv, m, flags, st, B, Hq, Hkv, D, scale,
+                       dtype, accumulate, true, false));
+    return launched(bam::launch_bwd_dq(p, dtype, (hipStream_t)stream), "bam_bwd_dq_indexed");
 }
 
 }  // extern "C"

@@ -22,15 +22,15 @@ __global__ __launch_bounds__(256) void bwd_preprocess_kernel(const AttnParams p)
     const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
     const int64_t row = gid / LPR;
     const int c = (int)(gid % LPR);
-    const int64_t total = (int64_t)p.B * p.S * p.Hq;
+    const int64_t total = (int64_t)p.B * p.Sq * p.Hq;
     const bool valid = row < total;
     int h = 0, i = 0, b = 0;
     float acc = 0.f;
     if (valid) {
         h = (int)(row % p.Hq);
         const int64_t bi = row / p.Hq;
-        i = (int)(bi % p.S);
-        b = (int)(bi / p.S);
+        i = (int)(bi % p.Sq);
+        b = (int)(bi / p.Sq);
         const u32x4 ov = *(const u32x4*)((const char*)p.o.ptr +
                                          2 * ((int64_t)b * p.o.sb + (int64_t)i * p.o.ss + (int64_t)h * p.o.sh) + c * 16);
         const u32x4 gv = *(const u32x4*)((const char*)p.dout.ptr +
@@ -43,7 +43,7 @@ __global__ __launch_bounds__(256) void bwd_preprocess_kernel(const AttnParams p)
     }
 #pragma unroll
     for (int off = LPR / 2; off > 0; off >>= 1) acc += __shfl_xor(acc, off);
-    if (valid && c == 0) p.delta[((int64_t)b * p.Hq + h) * p.S_rounded + i] = acc;
+    if (valid && c == 0) p.delta[((int64_t)b * p.Hq + h) * p.Sq_rounded + i] = acc;
 }
 
 // ---------------------------------------------------------------------------------------
@@ -61,7 +61,8 @@ __global__ __launch_bounds__(256) void bwd_preprocess_kernel(const AttnParams p)
 constexpr int DKDV_QT = 64;
 constexpr int DKDV_THREADS = 512;
 
-template <typename T, int D>
+// IDX: index-tensor attention (explicit global positions p.posq / p.posk, gathered bitfield arrays).
+template <typename T, int D, bool IDX>
 __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnParams p) {
     constexpr int NCH = D / 8, KK = D / 16, DB = D / 32;
     __shared__ u32x4 sK[128 * NCH];
@@ -71,6 +72,7 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
     __shared__ __attribute__((aligned(16))) float sLse[2][DKDV_QT];      // natural-log lse of the rows
     __shared__ __attribute__((aligned(16))) float sDelta[2][DKDV_QT];
     __shared__ __attribute__((aligned(16))) int64_t sQbf[2][DKDV_QT];    // raw bitfields of the rows
+    __shared__ __attribute__((aligned(16))) int sQpos[2][DKDV_QT];       // their global positions (IDX only)
     __shared__ __attribute__((aligned(16))) unsigned sWq[DKDV_THREADS / 64][5][32];  // per-wave rule constants
     __shared__ int sList[MAX_LIST / 2];
     __shared__ int sCount;
@@ -78,7 +80,7 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int kg = wave & 3, st = wave >> 2;
     const int hi = lane >> 5, l32 = lane & 31, half16 = (lane >> 4) & 1;
-    const int S = p.S;
+    const int Sq = p.Sq, Sk = p.Sk;
     const int G = p.Hq / p.Hkv;
 
     const int unit = blockIdx.x;
@@ -98,18 +100,19 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
         stV.setup(2 * p.v.ss, tid);
         const char* kb = (const char*)p.k.ptr + 2 * ((int64_t)b * p.k.sb + (int64_t)hk * p.k.sh + (int64_t)nt * 128 * p.k.ss);
         const char* vb = (const char*)p.v.ptr + 2 * ((int64_t)b * p.v.sb + (int64_t)hk * p.v.sh + (int64_t)nt * 128 * p.v.ss);
-        stK.load(kb, sK, S - nt * 128, tid);
-        stV.load(vb, sV, S - nt * 128, tid);
+        stK.load(kb, sK, Sk - nt * 128, tid);
+        stV.load(vb, sV, Sk - nt * 128, tid);
     }
     const int key = nt * 128 + kg * 32 + l32;
-    const bool kvalid = key < S;
-    const int64_t* bfrow = p.bf + (int64_t)b * p.bf_sb;
-    const int64_t kf = kvalid ? bfrow[key] : 0;
+    const bool kvalid = key < Sk;
+    const int64_t* bfrow = p.bfq + (int64_t)b * p.bfq_sb;  // bitfields of the query rows
+    const int64_t kf = kvalid ? p.bfk[(int64_t)b * p.bfk_sb + key] : 0;
+    int kpos = (IDX && kvalid) ? p.posk[key] : key;  // global position of this lane's key
     unsigned klo = (unsigned)(kf & 0xFFFFFFFFll);
     unsigned khi = (unsigned)((uint64_t)kf >> 32);
     // Pin the arrival of this load here.  Left alone, the compiler waits for it at the first use inside the
     // main loop, with a vmcnt that also (and every time round) drains the tile copies it does not know about.
-    asm volatile("" : "+v"(klo), "+v"(khi));
+    asm volatile("" : "+v"(klo), "+v"(khi), "+v"(kpos));
 
     f32x16 dk[DB], dv[DB];
 #pragma unroll
@@ -126,8 +129,9 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
 
     typedef TileStage<D, DKDV_QT, DKDV_THREADS> Stage;
     constexpr int CPT = Stage::CPT;
-    constexpr int NLOADS = 2 * CPT + 1;  // copy instructions per wave and tile: Q, dO and one of the four small rows
-    static_assert(NLOADS <= 2 * KK + 1, "one copy per MFMA gap");
+    // copy instructions per wave and tile: Q, dO, one of the four small rows and (IDX) the row positions
+    constexpr int NLOADS = 2 * CPT + 1 + (IDX ? 1 : 0);
+    static_assert(NLOADS <= 2 * KK, "one copy per MFMA of the S / dP phase");
     Stage stQ, stDO;
     stQ.setup(2 * p.q.ss, tid);
     stDO.setup(2 * p.dout.ss, tid);
@@ -147,12 +151,14 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
         } else if (j < 2 * CPT) {
             const char* gbase = (const char*)p.dout.ptr + 2 * ((int64_t)b * p.dout.sb + (int64_t)h * p.dout.sh + (int64_t)row0 * p.dout.ss);
             stDO.issue(j - CPT, gbase, ldsDO + buf * TILE_BYTES);
-        } else {
-            const int64_t off = ((int64_t)b * p.Hq + h) * p.S_rounded + row0;
+        } else if (j == 2 * CPT) {
+            const int64_t off = ((int64_t)b * p.Hq + h) * p.Sq_rounded + row0;
             const void* src = small == 0 ? (const void*)(p.lse + off)
                               : small == 1 ? (const void*)(p.delta + off)
                                            : (const void*)((const char*)(bfrow + row0) + (small - 2) * 256);
             dma_b32(src, (unsigned)(lane * 4), ldsSmall + buf * smallBytes);
+        } else {  // 64 row positions; every wave writes the same values
+            dma_b32(p.posq + row0, (unsigned)(lane * 4), lds_addr(sQpos) + buf * (DKDV_QT * 4u));
         }
     };
 
@@ -216,18 +222,25 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
             const int64_t mine = sQbf[cur][qr + l32];
             const unsigned mlo = (unsigned)mine, mhi = (unsigned)((uint64_t)mine >> 32);
             const unsigned flo = __builtin_amdgcn_readfirstlane(mlo), fhi = __builtin_amdgcn_readfirstlane(mhi);
-            if (__all((mlo == flo) & (mhi == fhi))) {
+            bool uniform = (mlo == flo) & (mhi == fhi);
+            int qpos0 = row0 + qr;  // position of this wave's first row
+            if (IDX) {              // ... and the 32 rows must sit at consecutive positions
+                const int rel0 = sQpos[cur][qr + l32] - l32;
+                qpos0 = __builtin_amdgcn_readfirstlane(rel0);
+                uniform &= rel0 == qpos0;
+            }
+            if (__all(uniform)) {
                 const QueryBits qu = make_query_bits(((int64_t)fhi << 32) | (int64_t)flo, 0);
                 const bool ok = allow_bits(qu, klo, khi) & (qu.text | (qu.lim >= 0));
                 // allowed iff krel <= 8 * grp + x  (text rows: key position <= row position)
-                const int krel = !ok ? 0x7FFFFFFF : qu.text ? key - (row0 + qr) - 4 * hi : (int)0x80000000;
+                const int krel = !ok ? 0x7FFFFFFF : qu.text ? kpos - qpos0 - 4 * hi : (int)0x80000000;
 #pragma unroll
                 for (int i = 0; i < 16; ++i) s[i] = (krel <= 8 * (i >> 2) + (i & 3)) ? s[i] : 0.f;
             } else {
                 // rule constants of this wave's 32 rows, derived once per row (lane r < 32 takes row r) and
                 // handed to all lanes through a wave-private LDS scratch
                 {
-                    const QueryBits qb = make_query_bits(mine, row0 + qr + l32);
+                    const QueryBits qb = make_query_bits(mine, IDX ? sQpos[cur][qr + l32] : row0 + qr + l32);
                     if (hi == 0) {
                         sWq[wave][0][l32] = qb.a_lo;
                         sWq[wave][1][l32] = qb.a_hi;
@@ -253,7 +266,7 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
                         qb.x_hi = qxhi[x];
                         qb.lim = (int)qlim[x];
                         qb.text = qlim[x] < 0x7FFFFFFFu;  // text rows carry their position, modality rows INT_MAX or -1
-                        s[4 * grp + x] = allow_pair(qb, klo, khi, key) ? s[4 * grp + x] : 0.f;
+                        s[4 * grp + x] = allow_pair(qb, klo, khi, kpos) ? s[4 * grp + x] : 0.f;
                     }
                 }
             }
@@ -295,7 +308,7 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
     const int n_all = sCount;
     // The last 128-row block of a sequence whose length is not a multiple of 128 (always the last list entry)
     // is staged synchronously, with neutral values for the rows past the end, after the main loop.
-    const bool ragged = (S & (BLOCK_M - 1)) != 0 && n_all > 0 &&
+    const bool ragged = (Sq & (BLOCK_M - 1)) != 0 && n_all > 0 &&
                         (__builtin_amdgcn_readfirstlane(sList[n_all > 0 ? n_all - 1 : 0]) >> 8) == p.num_m - 1;
     const int n = n_all - (ragged ? 1 : 0);
     // Main loop: tiles t = 0 .. 2 n G - 1 -> (q head g of the group, list entry, 64-row half).  Query blocks are
@@ -344,18 +357,19 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
         for (int t = 0; t < 2 * G; ++t) {
             const int g = t >> 1;
             const int row0 = (entry >> 8) * BLOCK_M + (t & 1) * DKDV_QT;
-            const int rows = S - row0;  // rows of the tile inside the sequence
+            const int rows = Sq - row0;  // rows of the tile inside the sequence
             if (rows <= 0) continue;
             const int h = hk * G + g;
             __syncthreads();  // everybody is done with buffer 0
             stQ.load_ragged((const char*)p.q.ptr + 2 * ((int64_t)b * p.q.sb + (int64_t)h * p.q.sh + (int64_t)row0 * p.q.ss), sQ[0], rows, tid);
             stDO.load_ragged((const char*)p.dout.ptr + 2 * ((int64_t)b * p.dout.sb + (int64_t)h * p.dout.sh + (int64_t)row0 * p.dout.ss), sDO[0], rows, tid);
             if (tid < DKDV_QT) {
-                const int64_t off = ((int64_t)b * p.Hq + h) * p.S_rounded + row0;
+                const int64_t off = ((int64_t)b * p.Hq + h) * p.Sq_rounded + row0;
                 const bool ok = tid < rows;
                 sLse[0][tid] = ok ? p.lse[off + tid] : INFINITY;  // lse = +inf gives P = 0
                 sDelta[0][tid] = ok ? p.delta[off + tid] : 0.f;
                 sQbf[0][tid] = ok ? bfrow[row0 + tid] : 0;
+                if (IDX) sQpos[0][tid] = ok ? p.posq[row0 + tid] : 0;
             }
             __syncthreads();
             tile_step(std::false_type{}, 0, (entry >> (2 * kg_lane)) & 3, row0, 0, 0);
@@ -442,18 +456,19 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
 constexpr int DQ_KT = 64;
 constexpr int DQ_THREADS = 256;
 
-template <typename T, int D>
+template <typename T, int D, bool IDX>
 __global__ __launch_bounds__(DQ_THREADS, 2) void bwd_dq_kernel(const AttnParams p) {
     constexpr int NCH = D / 8, KK = D / 16, DB = D / 32;
     __shared__ u32x4 sK[2][DQ_KT * NCH];
     __shared__ u32x4 sV[2][DQ_KT * NCH];
     __shared__ __attribute__((aligned(16))) int64_t sKbf[2][DQ_KT];  // raw bitfields of the tile's keys
+    __shared__ __attribute__((aligned(16))) int sKpos[2][DQ_KT];     // their global positions (IDX only)
     __shared__ int sList[MAX_LIST];
     __shared__ int sCount;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int hi = lane >> 5, l32 = lane & 31, half16 = (lane >> 4) & 1;
-    const int S = p.S;
+    const int Sq = p.Sq, Sk = p.Sk;
     const int G = p.Hq / p.Hkv;
 
     int unit, g;
@@ -465,11 +480,11 @@ __global__ __launch_bounds__(DQ_THREADS, 2) void bwd_dq_kernel(const AttnParams 
     const int h = hk * G + g;
 
     if (wave == 0)
-        build_key_tile_list(p.flags + (int64_t)b * p.flags_sb + (int64_t)m * p.flags_sm, p.num_n, S, lane,
+        build_key_tile_list(p.flags + (int64_t)b * p.flags_sb + (int64_t)m * p.flags_sm, p.num_n, Sk, lane,
                             sList, &sCount);
 
     const int qrow = m * BLOCK_M + wave * 32 + l32;
-    const bool qvalid = qrow < S;
+    const bool qvalid = qrow < Sq;
     u32x4 qreg[KK], greg[KK];
     {
         const char* qp = (const char*)p.q.ptr + 2 * ((int64_t)b * p.q.sb + (int64_t)qrow * p.q.ss + (int64_t)h * p.q.sh);
@@ -485,11 +500,11 @@ __global__ __launch_bounds__(DQ_THREADS, 2) void bwd_dq_kernel(const AttnParams 
             greg[kk] = zg;
         }
     }
-    const int64_t qf = qvalid ? p.bf[(int64_t)b * p.bf_sb + qrow] : 0;
-    const QueryBits qb = make_query_bits(qf, qrow);
+    const int64_t qf = qvalid ? p.bfq[(int64_t)b * p.bfq_sb + qrow] : 0;
+    const QueryBits qb = make_query_bits(qf, (IDX && qvalid) ? p.posq[qrow] : qrow);
     float lse2 = INFINITY, dlt = 0.f;
     if (qvalid) {
-        const int64_t off = ((int64_t)b * p.Hq + h) * p.S_rounded + qrow;
+        const int64_t off = ((int64_t)b * p.Hq + h) * p.Sq_rounded + qrow;
         const float l = p.lse[off];
         lse2 = (l == -INFINITY) ? INFINITY : l * LOG2E;
         dlt = p.delta[off];
@@ -508,16 +523,17 @@ __global__ __launch_bounds__(DQ_THREADS, 2) void bwd_dq_kernel(const AttnParams 
     const char* kbase = (const char*)p.k.ptr + 2 * ((int64_t)b * p.k.sb + (int64_t)hk * p.k.sh);
     const char* vbase = (const char*)p.v.ptr + 2 * ((int64_t)b * p.v.sb + (int64_t)hk * p.v.sh);
     const int64_t k_ts = 2 * p.k.ss * DQ_KT, v_ts = 2 * p.v.ss * DQ_KT;  // bytes per tile
-    const int64_t* bfrow = p.bf + (int64_t)b * p.bf_sb;
+    const int64_t* bfrow = p.bfk + (int64_t)b * p.bfk_sb;
 
     typedef TileStage<D, DQ_KT, DQ_THREADS> Stage;
     constexpr int CPT = Stage::CPT;
-    constexpr int NLOADS = 2 * CPT + 1;  // copy instructions per wave and tile: K, V and the key bitfields
-    static_assert(NLOADS <= 2 * KK + 1, "one copy per MFMA gap");
+    // copy instructions per wave and tile: K, V, the key bitfields and (IDX) the key positions
+    constexpr int NLOADS = 2 * CPT + 1 + (IDX ? 1 : 0);
+    static_assert(NLOADS <= 2 * KK, "one copy per MFMA of the first S / dP block");
     Stage stK, stV;
     stK.setup(2 * p.k.ss, tid);
     stV.setup(2 * p.v.ss, tid);
-    const unsigned ldsK = lds_addr(sK), ldsV = lds_addr(sV), ldsB = lds_addr(sKbf);
+    const unsigned ldsK = lds_addr(sK), ldsV = lds_addr(sV), ldsB = lds_addr(sKbf), ldsP = lds_addr(sKpos);
     constexpr unsigned TILE_BYTES = DQ_KT * NCH * 16, BITS_BYTES = DQ_KT * 8;
     // copy instruction j of full tile kt into buffer buf (key bitfields: 64 dwords per wave, waves 2, 3
     // repeat what waves 0, 1 write, so that every wave issues the same number of copies)
@@ -526,8 +542,10 @@ __global__ __launch_bounds__(DQ_THREADS, 2) void bwd_dq_kernel(const AttnParams 
             stK.issue(j, kbase + kt * k_ts, ldsK + buf * TILE_BYTES);
         else if (j < 2 * CPT)
             stV.issue(j - CPT, vbase + kt * v_ts, ldsV + buf * TILE_BYTES);
-        else
+        else if (j == 2 * CPT)
             dma_b32(bfrow + kt * DQ_KT, (unsigned)((wave & 1) * 256 + lane * 4), ldsB + buf * BITS_BYTES + (wave & 1) * 256u);
+        else  // 64 positions; every wave writes the same values
+            dma_b32(p.posk + kt * DQ_KT, (unsigned)(lane * 4), ldsP + buf * (DQ_KT * 4u));
     };
 
     // One 64-key tile held in buffer `cur`; with PREFETCH the copies of tile kt_next into the other buffer
@@ -544,8 +562,15 @@ __global__ __launch_bounds__(DQ_THREADS, 2) void bwd_dq_kernel(const AttnParams 
             const int64_t mine = sKbf[cur][lane];
             const unsigned mlo = (unsigned)mine, mhi = (unsigned)((uint64_t)mine >> 32);
             const unsigned flo = __builtin_amdgcn_readfirstlane(mlo), fhi = __builtin_amdgcn_readfirstlane(mhi);
-            uniform_keys = __all((mlo == flo) & (mhi == fhi));
-            rel = allow_bits(qb, flo, fhi) ? qb.lim - kt * DQ_KT : -1;  // last allowed key, relative to the tile
+            bool uniform = (mlo == flo) & (mhi == fhi);
+            int kt0 = kt * DQ_KT;  // position of the tile's first key
+            if (IDX) {             // ... and the 64 keys must sit at consecutive positions
+                const int rel0 = sKpos[cur][lane] - lane;
+                kt0 = __builtin_amdgcn_readfirstlane(rel0);
+                uniform &= rel0 == kt0;
+            }
+            uniform_keys = __all(uniform);
+            rel = allow_bits(qb, flo, fhi) ? qb.lim - kt0 : -1;  // last allowed key, relative to the tile
         }
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) {
@@ -590,9 +615,15 @@ __global__ __launch_bounds__(DQ_THREADS, 2) void bwd_dq_kernel(const AttnParams 
                         const u32x4 k23 = *(const u32x4*)&sKbf[cur][koff + 2];  // lo2 hi2 lo3 hi3
                         const unsigned klo[4] = {k01[0], k01[2], k23[0], k23[2]};
                         const unsigned khi[4] = {k01[1], k01[3], k23[1], k23[3]};
+                        int kpos[4] = {kt0 + koff, kt0 + koff + 1, kt0 + koff + 2, kt0 + koff + 3};
+                        if (IDX) {
+                            const u32x4 kp = *(const u32x4*)&sKpos[cur][koff];
+#pragma unroll
+                            for (int x = 0; x < 4; ++x) kpos[x] = (int)kp[x];
+                        }
 #pragma unroll
                         for (int x = 0; x < 4; ++x)
-                            dp[4 * grp + x] = allow_pair(qb, klo[x], khi[x], kt0 + koff + x) ? dp[4 * grp + x] : 0.f;
+                            dp[4 * grp + x] = allow_pair(qb, klo[x], khi[x], kpos[x]) ? dp[4 * grp + x] : 0.f;
                     }
                 }
             }
@@ -620,8 +651,8 @@ __global__ __launch_bounds__(DQ_THREADS, 2) void bwd_dq_kernel(const AttnParams 
     const int n_all = sCount;
     // A tile that holds the end of a sequence whose length is not a multiple of 64 is always the last
     // entry of the list; it is staged synchronously (zero fill past the end) after the main loop.
-    const bool ragged = (S & (DQ_KT - 1)) != 0 && n_all > 0 &&
-                        (__builtin_amdgcn_readfirstlane(sList[n_all > 0 ? n_all - 1 : 0]) >> 2) == ((S - 1) >> 6);
+    const bool ragged = (Sk & (DQ_KT - 1)) != 0 && n_all > 0 &&
+                        (__builtin_amdgcn_readfirstlane(sList[n_all > 0 ? n_all - 1 : 0]) >> 2) == ((Sk - 1) >> 6);
     const int n = n_all - (ragged ? 1 : 0);
     if (n > 0) {
         int entry = __builtin_amdgcn_readfirstlane(sList[0]);
@@ -644,10 +675,13 @@ __global__ __launch_bounds__(DQ_THREADS, 2) void bwd_dq_kernel(const AttnParams 
     }
     if (ragged) {
         const int entry = __builtin_amdgcn_readfirstlane(sList[n_all - 1]);
-        const int kt = entry >> 2, rows = S - kt * DQ_KT;
+        const int kt = entry >> 2, rows = Sk - kt * DQ_KT;
         stK.load_ragged(kbase + kt * k_ts, sK[0], rows, tid);
         stV.load_ragged(vbase + kt * v_ts, sV[0], rows, tid);
-        if (tid < DQ_KT) sKbf[0][tid] = (tid < rows) ? bfrow[kt * DQ_KT + tid] : 0;
+        if (tid < DQ_KT) {
+            sKbf[0][tid] = (tid < rows) ? bfrow[kt * DQ_KT + tid] : 0;
+            if (IDX) sKpos[0][tid] = (tid < rows) ? p.posk[kt * DQ_KT + tid] : 0;
+        }
         __syncthreads();
         tile_step(std::false_type{}, 0, entry, 0);
     }
@@ -681,21 +715,27 @@ __global__ __launch_bounds__(DQ_THREADS, 2) void bwd_dq_kernel(const AttnParams 
 // ---------------------------------------------------------------------------------------
 template <typename T, int D>
 static int launch_pre_t(const AttnParams& p, hipStream_t stream) {
-    const int64_t threads = (int64_t)p.B * p.S * p.Hq * (D / 8);
+    const int64_t threads = (int64_t)p.B * p.Sq * p.Hq * (D / 8);
     const int64_t blocks = (threads + 255) / 256;
     hipLaunchKernelGGL((bwd_preprocess_kernel<T, D>), dim3((unsigned)blocks), dim3(256), 0, stream, p);
     return (int)hipGetLastError();
 }
 template <typename T, int D>
 static int launch_dkdv_t(const AttnParams& p, hipStream_t stream) {
-    const int blocks = p.num_m * p.B * p.Hkv;  // ceil(S/128) key tiles
-    hipLaunchKernelGGL((bwd_dkdv_kernel<T, D>), dim3(blocks), dim3(DKDV_THREADS), 0, stream, p);
+    const int blocks = p.num_kt * p.B * p.Hkv;  // one workgroup per 128-key tile
+    if (p.posq != nullptr)
+        hipLaunchKernelGGL((bwd_dkdv_kernel<T, D, true>), dim3(blocks), dim3(DKDV_THREADS), 0, stream, p);
+    else
+        hipLaunchKernelGGL((bwd_dkdv_kernel<T, D, false>), dim3(blocks), dim3(DKDV_THREADS), 0, stream, p);
     return (int)hipGetLastError();
 }
 template <typename T, int D>
 static int launch_dq_t(const AttnParams& p, hipStream_t stream) {
     const int blocks = p.num_m * p.B * p.Hq;
-    hipLaunchKernelGGL((bwd_dq_kernel<T, D>), dim3(blocks), dim3(DQ_THREADS), 0, stream, p);
+    if (p.posq != nullptr)
+        hipLaunchKernelGGL((bwd_dq_kernel<T, D, true>), dim3(blocks), dim3(DQ_THREADS), 0, stream, p);
+    else
+        hipLaunchKernelGGL((bwd_dq_kernel<T, D, false>), dim3(blocks), dim3(DQ_THREADS), 0, stream, p);
     return (int)hipGetLastError();
 }
 

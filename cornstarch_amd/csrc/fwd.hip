@@ -26,18 +26,22 @@ namespace bam {
 constexpr int FWD_KT = 64;
 constexpr int FWD_THREADS = 256;
 
-template <typename T, int D>
+// IDX: index-tensor attention -- query rows and keys carry explicit global positions (p.posq, p.posk) and
+// the bitfield arrays are already gathered per local row / key (context-parallel shards, reference
+// bitfield_attention.py:71-81).
+template <typename T, int D, bool IDX>
 __global__ __launch_bounds__(FWD_THREADS, 2) void fwd_kernel(const AttnParams p) {
     constexpr int NCH = D / 8, KK = D / 16, DB = D / 32;
     __shared__ u32x4 sK[2][FWD_KT * NCH];
     __shared__ u32x4 sV[2][FWD_KT * NCH];
     __shared__ __attribute__((aligned(16))) int64_t sKbf[2][FWD_KT];  // raw bitfields of the tile's keys
+    __shared__ __attribute__((aligned(16))) int sKpos[2][FWD_KT];     // their global positions (IDX only)
     __shared__ int sList[MAX_LIST];
     __shared__ int sCount;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int hi = lane >> 5, l32 = lane & 31, half16 = (lane >> 4) & 1;
-    const int S = p.S;
+    const int Sq = p.Sq, Sk = p.Sk;
     const int G = p.Hq / p.Hkv;
 
     int unit, g;
@@ -49,12 +53,12 @@ __global__ __launch_bounds__(FWD_THREADS, 2) void fwd_kernel(const AttnParams p)
     const int h = hk * G + g;
 
     if (wave == 0)
-        build_key_tile_list(p.flags + (int64_t)b * p.flags_sb + (int64_t)m * p.flags_sm, p.num_n, S, lane,
+        build_key_tile_list(p.flags + (int64_t)b * p.flags_sb + (int64_t)m * p.flags_sm, p.num_n, Sk, lane,
                             sList, &sCount);
 
     // ---- per-lane query state -------------------------------------------------------
     const int qrow = m * BLOCK_M + wave * 32 + l32;
-    const bool qvalid = qrow < S;
+    const bool qvalid = qrow < Sq;
     u32x4 qreg[KK];
     {
         const char* qp = (const char*)p.q.ptr + 2 * ((int64_t)b * p.q.sb + (int64_t)qrow * p.q.ss + (int64_t)h * p.q.sh);
@@ -65,8 +69,8 @@ __global__ __launch_bounds__(FWD_THREADS, 2) void fwd_kernel(const AttnParams p)
             qreg[kk] = z;
         }
     }
-    const int64_t qf = qvalid ? p.bf[(int64_t)b * p.bf_sb + qrow] : 0;
-    const QueryBits qb = make_query_bits(qf, qrow);
+    const int64_t qf = qvalid ? p.bfq[(int64_t)b * p.bfq_sb + qrow] : 0;
+    const QueryBits qb = make_query_bits(qf, (IDX && qvalid) ? p.posq[qrow] : qrow);
 
     f32x16 o[DB];
 #pragma unroll
@@ -89,16 +93,17 @@ __global__ __launch_bounds__(FWD_THREADS, 2) void fwd_kernel(const AttnParams p)
     const char* kbase = (const char*)p.k.ptr + 2 * ((int64_t)b * p.k.sb + (int64_t)hk * p.k.sh);
     const char* vbase = (const char*)p.v.ptr + 2 * ((int64_t)b * p.v.sb + (int64_t)hk * p.v.sh);
     const int64_t k_ts = 2 * p.k.ss * FWD_KT, v_ts = 2 * p.v.ss * FWD_KT;  // bytes per tile
-    const int64_t* bfrow = p.bf + (int64_t)b * p.bf_sb;
+    const int64_t* bfrow = p.bfk + (int64_t)b * p.bfk_sb;
 
     typedef TileStage<D, FWD_KT, FWD_THREADS> Stage;
     constexpr int CPT = Stage::CPT;
-    constexpr int NLOADS = 2 * CPT + 1;  // copy instructions per wave and tile: K, V and the key bitfields
-    static_assert(NLOADS <= 2 * KK + 1, "one copy per MFMA gap");
+    // copy instructions per wave and tile: K, V, the key bitfields and (IDX) the key positions
+    constexpr int NLOADS = 2 * CPT + 1 + (IDX ? 1 : 0);
+    static_assert(NLOADS <= 2 * KK, "one copy per MFMA of the S phase");
     Stage stK, stV;
     stK.setup(2 * p.k.ss, tid);
     stV.setup(2 * p.v.ss, tid);
-    const unsigned ldsK = lds_addr(sK), ldsV = lds_addr(sV), ldsB = lds_addr(sKbf);
+    const unsigned ldsK = lds_addr(sK), ldsV = lds_addr(sV), ldsB = lds_addr(sKbf), ldsP = lds_addr(sKpos);
     constexpr unsigned TILE_BYTES = FWD_KT * NCH * 16, BITS_BYTES = FWD_KT * 8;
     // Copy instruction j (0 <= j < NLOADS) of full tile kt into buffer buf.  The 128 dwords of key
     // bitfields are copied 64 dwords per wave (waves 2, 3 repeat what waves 0, 1 write), so that every
@@ -108,8 +113,10 @@ __global__ __launch_bounds__(FWD_THREADS, 2) void fwd_kernel(const AttnParams p)
             stK.issue(j, kbase + kt * k_ts, ldsK + buf * TILE_BYTES);
         else if (j < 2 * CPT)
             stV.issue(j - CPT, vbase + kt * v_ts, ldsV + buf * TILE_BYTES);
-        else
+        else if (j == 2 * CPT)
             dma_b32(bfrow + kt * FWD_KT, (unsigned)((wave & 1) * 256 + lane * 4), ldsB + buf * BITS_BYTES + (wave & 1) * 256u);
+        else  // 64 positions; every wave writes the same values
+            dma_b32(p.posk + kt * FWD_KT, (unsigned)(lane * 4), ldsP + buf * (FWD_KT * 4u));
     };
 
     // One 64-key tile held in buffer `cur`.  With PREFETCH the copies of tile `kt_next` into the other
@@ -142,13 +149,20 @@ __global__ __launch_bounds__(FWD_THREADS, 2) void fwd_kernel(const AttnParams p)
 
         // ---- bitfield rule in registers (partial tiles only) ------------------------------
         if (cls == 1) {
-            const int kt0 = kt * FWD_KT;
-            // Most partial tiles are partial only through causality: all 64 keys carry the same bitfield.
-            // Then the bit test is a per-query constant and the rule reduces to one position compare.
+            // Most partial tiles are partial only through causality: all 64 keys carry the same bitfield (and,
+            // with index tensors, sit at consecutive positions).  Then the bit test is a per-query constant and
+            // the rule reduces to one position compare.
             const int64_t mine = sKbf[cur][lane];
             const unsigned mlo = (unsigned)mine, mhi = (unsigned)((uint64_t)mine >> 32);
             const unsigned flo = __builtin_amdgcn_readfirstlane(mlo), fhi = __builtin_amdgcn_readfirstlane(mhi);
-            if (__all((mlo == flo) & (mhi == fhi))) {
+            bool uniform = (mlo == flo) & (mhi == fhi);
+            int kt0 = kt * FWD_KT;  // position of the tile's first key
+            if (IDX) {
+                const int rel0 = sKpos[cur][lane] - lane;
+                kt0 = __builtin_amdgcn_readfirstlane(rel0);
+                uniform &= rel0 == kt0;
+            }
+            if (__all(uniform)) {
                 const int rel = allow_bits(qb, flo, fhi) ? qb.lim - kt0 : -1;  // last allowed key, relative to the tile
 #pragma unroll
                 for (int kb = 0; kb < 2; ++kb)
@@ -167,9 +181,15 @@ __global__ __launch_bounds__(FWD_THREADS, 2) void fwd_kernel(const AttnParams p)
                         const u32x4 k23 = *(const u32x4*)&sKbf[cur][koff + 2];  // lo2 hi2 lo3 hi3
                         const unsigned klo[4] = {k01[0], k01[2], k23[0], k23[2]};
                         const unsigned khi[4] = {k01[1], k01[3], k23[1], k23[3]};
+                        int kpos[4] = {kt * FWD_KT + koff, kt * FWD_KT + koff + 1, kt * FWD_KT + koff + 2, kt * FWD_KT + koff + 3};
+                        if (IDX) {
+                            const u32x4 kp = *(const u32x4*)&sKpos[cur][koff];
+#pragma unroll
+                            for (int x = 0; x < 4; ++x) kpos[x] = (int)kp[x];
+                        }
 #pragma unroll
                         for (int x = 0; x < 4; ++x) {
-                            const bool a = allow_pair(qb, klo[x], khi[x], kt0 + koff + x);
+                            const bool a = allow_pair(qb, klo[x], khi[x], kpos[x]);
                             s[kb][4 * grp + x] = a ? s[kb][4 * grp + x] : -INFINITY;
                         }
                     }
@@ -235,8 +255,8 @@ __global__ __launch_bounds__(FWD_THREADS, 2) void fwd_kernel(const AttnParams p)
     const int n_all = sCount;
     // A tile that holds the end of a sequence whose length is not a multiple of 64 is always the last
     // entry of the list; it is staged synchronously (zero fill past the end) after the main loop.
-    const bool ragged = (S & (FWD_KT - 1)) != 0 && n_all > 0 &&
-                        (__builtin_amdgcn_readfirstlane(sList[n_all > 0 ? n_all - 1 : 0]) >> 2) == ((S - 1) >> 6);
+    const bool ragged = (Sk & (FWD_KT - 1)) != 0 && n_all > 0 &&
+                        (__builtin_amdgcn_readfirstlane(sList[n_all > 0 ? n_all - 1 : 0]) >> 2) == ((Sk - 1) >> 6);
     const int n = n_all - (ragged ? 1 : 0);
     if (n > 0) {
         int entry = __builtin_amdgcn_readfirstlane(sList[0]);
@@ -259,10 +279,13 @@ __global__ __launch_bounds__(FWD_THREADS, 2) void fwd_kernel(const AttnParams p)
     }
     if (ragged) {
         const int entry = __builtin_amdgcn_readfirstlane(sList[n_all - 1]);
-        const int kt = entry >> 2, rows = S - kt * FWD_KT;
+        const int kt = entry >> 2, rows = Sk - kt * FWD_KT;
         stK.load_ragged(kbase + kt * k_ts, sK[0], rows, tid);
         stV.load_ragged(vbase + kt * v_ts, sV[0], rows, tid);
-        if (tid < FWD_KT) sKbf[0][tid] = (tid < rows) ? bfrow[kt * FWD_KT + tid] : 0;
+        if (tid < FWD_KT) {
+            sKbf[0][tid] = (tid < rows) ? bfrow[kt * FWD_KT + tid] : 0;
+            if (IDX) sKpos[0][tid] = (tid < rows) ? p.posk[kt * FWD_KT + tid] : 0;
+        }
         __syncthreads();
         tile_step(std::false_type{}, 0, entry, 0);
     }
@@ -271,7 +294,7 @@ __global__ __launch_bounds__(FWD_THREADS, 2) void fwd_kernel(const AttnParams p)
     const float ltot = half_swap_sum(l_i);
     const float inv = ltot > 0.f ? 1.f / ltot : 0.f;
     if (hi == 0)
-        p.lse[((int64_t)b * p.Hq + h) * p.S_rounded + qrow] =
+        p.lse[((int64_t)b * p.Hq + h) * p.Sq_rounded + qrow] =
             ltot > 0.f ? (m_i * c2 + __builtin_amdgcn_logf(ltot)) * LN2 : -INFINITY;
     if (qvalid) {
         char* op = (char*)p.o.ptr + 2 * ((int64_t)b * p.o.sb + (int64_t)qrow * p.o.ss + (int64_t)h * p.o.sh);
@@ -290,7 +313,10 @@ __global__ __launch_bounds__(FWD_THREADS, 2) void fwd_kernel(const AttnParams p)
 template <typename T, int D>
 static int launch_fwd_t(const AttnParams& p, hipStream_t stream) {
     const int blocks = p.num_m * p.B * p.Hq;
-    hipLaunchKernelGGL((fwd_kernel<T, D>), dim3(blocks), dim3(FWD_THREADS), 0, stream, p);
+    if (p.posq != nullptr)
+        hipLaunchKernelGGL((fwd_kernel<T, D, true>), dim3(blocks), dim3(FWD_THREADS), 0, stream, p);
+    else
+        hipLaunchKernelGGL((fwd_kernel<T, D, false>), dim3(blocks), dim3(FWD_THREADS), 0, stream, p);
     return (int)hipGetLastError();
 }
 

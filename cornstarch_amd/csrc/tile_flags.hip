@@ -62,6 +62,30 @@ __global__ __launch_bounds__(256) void materialize_mask_kernel(const int64_t* __
         out[((int64_t)b * S + i) * S + j] = allow_rule(qf, row[j], i, j) ? 1 : 0;
 }
 
+// Index-tensor attention, step 0: the bitfield and the 32-bit position of every local row (or key),
+// out_bits[b][i] = bf[b][idx[i]] (0 when idx[i] is outside [0, L)), out_pos[i] = idx[i].
+// Restates the index branch of the reference's mask block (bitfield_attention.py:71-87), hoisted out
+// of the attention kernels so that they read both with unit stride.
+__global__ __launch_bounds__(256) void gather_bitfields_kernel(const int64_t* __restrict__ bf, int64_t bf_stride_b,
+                                                               int L, const int64_t* __restrict__ idx, int n,
+                                                               int64_t* __restrict__ out_bits,
+                                                               int64_t out_stride_b, int* __restrict__ out_pos) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x, b = blockIdx.y;
+    if (i >= n) return;
+    const int64_t pos = idx[i];
+    const bool inside = pos >= 0 && pos < L;
+    out_bits[(int64_t)b * out_stride_b + i] = inside ? bf[(int64_t)b * bf_stride_b + pos] : 0;
+    if (b == 0) out_pos[i] = (int)(pos < 0 ? 0 : pos > 0x7FFFFFFE ? 0x7FFFFFFE : pos);
+}
+
+int launch_gather_bitfields(const int64_t* bf, int64_t bf_stride_b, int L, const int64_t* idx, int n, int64_t* out_bits,
+                            int64_t out_stride_b, int* out_pos, int B, hipStream_t stream) {
+    dim3 grid((n + 255) / 256, B);
+    hipLaunchKernelGGL(gather_bitfields_kernel, grid, dim3(256), 0, stream, bf, bf_stride_b, L, idx, n, out_bits,
+                       out_stride_b, out_pos);
+    return (int)hipGetLastError();
+}
+
 int launch_tile_flags(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int64_t flags_stride_b,
                       int64_t flags_stride_m, int B, int S, hipStream_t stream) {
     const int num_m = (S + BLOCK_M - 1) / BLOCK_M, num_n = (S + BLOCK_N - 1) / BLOCK_N;

@@ -14,12 +14,29 @@ LIB_PATH = os.path.join(_PKG_DIR, "libbam_hip.so")
 BAM_DTYPE_F16 = 0
 BAM_DTYPE_BF16 = 1
 BAM_MAX_SEQLEN = 131072
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 _i64 = ctypes.c_int64
 _int = ctypes.c_int
 _ptr = ctypes.c_void_p
 _f32 = ctypes.c_float
+
+class IndexView(ctypes.Structure):
+    """``bam_index_view`` of include/bam_hip.h (host struct holding device pointers)."""
+
+    _fields_ = [
+        ("q_bits", ctypes.c_void_p),
+        ("k_bits", ctypes.c_void_p),
+        ("q_pos", ctypes.c_void_p),
+        ("k_pos", ctypes.c_void_p),
+        ("q_bits_stride_b", ctypes.c_int64),
+        ("k_bits_stride_b", ctypes.c_int64),
+        ("Sq", ctypes.c_int32),
+        ("Sk", ctypes.c_int32),
+    ]
+
+
+_view = ctypes.POINTER(IndexView)
 
 # name -> argtypes, exactly the prototypes of include/bam_hip.h
 SIGNATURES = {
@@ -30,6 +47,10 @@ SIGNATURES = {
     "bam_bwd": [_ptr] * 11 + [_i64] * 24 + [_int] * 5 + [_f32, _int, _int, _ptr],
     "bam_bwd_dkdv": [_ptr] * 10 + [_i64] * 21 + [_int] * 5 + [_f32, _int, _int, _ptr],
     "bam_bwd_dq": [_ptr] * 9 + [_i64] * 18 + [_int] * 5 + [_f32, _int, _int, _ptr],
+    "bam_gather_bitfields": [_ptr, _i64, _int, _ptr, _int, _ptr, _i64, _ptr, _int, _ptr],
+    "bam_fwd_indexed": [_ptr] * 5 + [_view, _ptr] + [_i64] * 14 + [_int] * 4 + [_f32, _int, _ptr],
+    "bam_bwd_dkdv_indexed": [_ptr] * 8 + [_view, _ptr] + [_i64] * 20 + [_int] * 4 + [_f32, _int, _int, _ptr],
+    "bam_bwd_dq_indexed": [_ptr] * 7 + [_view, _ptr] + [_i64] * 17 + [_int] * 4 + [_f32, _int, _int, _ptr],
 }
 
 _lib = None

@@ -121,11 +121,49 @@ class BitfieldUtils:
         return out
 
 
-def _check_unsupported(offsets_q, offsets_k, bias):
-    if offsets_q is not None or offsets_k is not None:
-        raise NotImplementedError("offsets_q / offsets_k (context-parallel index tensors) are not implemented yet")
+def _check_unsupported(bias):
     if bias is not None:
         raise NotImplementedError("attention bias is not implemented (no caller of the reference passes one)")
+
+
+class _IndexView:
+    """Index-tensor attention (``offsets_q`` / ``offsets_k`` of the reference entry points,
+    bitfield_attention.py:938-939, 1085-1086): local row i of q sits at global position
+    ``offsets_q[i]``, local key j at ``offsets_k[j]``, and ``bitfield_mask`` is indexed by global
+    position (bitfield_attention.py:71-87).  The gather bitfield[offsets] is done once, by a kernel of
+    the library, and the attention kernels read the gathered arrays with unit stride."""
+
+    def __init__(self, bitfield_mask: torch.Tensor, offsets_q: torch.Tensor, offsets_k: torch.Tensor):
+        if offsets_q is None or offsets_k is None:
+            raise ValueError("offsets_q and offsets_k must be given together")
+        dev = bitfield_mask.device
+        bf = bitfield_mask if bitfield_mask.stride(1) == 1 else bitfield_mask.contiguous()
+        batch, length = bf.shape
+        self.seqlen_q, self.seqlen_k = int(offsets_q.numel()), int(offsets_k.numel())
+        assert offsets_q.dim() == 1 and offsets_k.dim() == 1
+        self._keep = []
+        arrays = []
+        with torch.cuda.device(dev):
+            for off in (offsets_q, offsets_k):
+                idx = off.to(device=dev, dtype=torch.int64).contiguous()
+                bits = torch.empty((batch, idx.numel()), dtype=torch.int64, device=dev)
+                pos = torch.empty((idx.numel(),), dtype=torch.int32, device=dev)
+                _bam_hip.call(
+                    "bam_gather_bitfields", bf.data_ptr(), bf.stride(0), length, idx.data_ptr(), idx.numel(),
+                    bits.data_ptr(), bits.stride(0), pos.data_ptr(), batch, _stream_ptr(dev),
+                )
+                arrays.append((bits, pos))
+                self._keep.append(idx)
+        (self.q_bits, self.q_pos), (self.k_bits, self.k_pos) = arrays
+        self.struct = _bam_hip.IndexView(
+            self.q_bits.data_ptr(), self.k_bits.data_ptr(), self.q_pos.data_ptr(), self.k_pos.data_ptr(),
+            self.q_bits.stride(0), self.k_bits.stride(0), self.seqlen_q, self.seqlen_k,
+        )
+
+    def byref(self):
+        import ctypes
+
+        return ctypes.byref(self.struct)
 
 
 def _bitfield_attn_forward(
@@ -148,11 +186,17 @@ def _bitfield_attn_forward(
     assert q.dtype == k.dtype == v.dtype, "All tensors must have the same type"
     assert q.dtype in [torch.float16, torch.bfloat16], "Only support fp16 and bf16"
     assert q.is_cuda and k.is_cuda and v.is_cuda
-    assert seqlen_q == seqlen_k, "self-attention only: query and key sequence lengths must match"
     assert k.shape == v.shape and k.shape[0] == batch and k.shape[3] == d
     assert nheads % nheads_k == 0
-    assert bitfield_mask.dtype == torch.int64 and bitfield_mask.shape == (batch, seqlen_k)
-    _check_unsupported(offsets_q, offsets_k, bias)
+    assert bitfield_mask.dtype == torch.int64 and bitfield_mask.dim() == 2 and bitfield_mask.shape[0] == batch
+    _check_unsupported(bias)
+    view = None
+    if offsets_q is not None or offsets_k is not None:
+        view = _IndexView(bitfield_mask, offsets_q, offsets_k)
+        assert (view.seqlen_q, view.seqlen_k) == (seqlen_q, seqlen_k), "one offset per local query row / key"
+    else:
+        assert seqlen_q == seqlen_k, "without index tensors query and key sequence lengths must match"
+        assert bitfield_mask.shape[1] == seqlen_k
     softmax_scale = softmax_scale or 1.0 / math.sqrt(d)
 
     dp = _padded_head_dim(d)
@@ -168,17 +212,24 @@ def _bitfield_attn_forward(
     lse = torch.empty((batch, nheads, seqlen_q_rounded), device=q.device, dtype=torch.float32)
     o = torch.empty_like(qk)
     with torch.cuda.device(q.device):
-        _bam_hip.call(
-            "bam_fwd",
-            qk.data_ptr(), kk.data_ptr(), vk.data_ptr(), o.data_ptr(), lse.data_ptr(), bf.data_ptr(), flags.data_ptr(),
-            qk.stride(0), qk.stride(1), qk.stride(2),
-            kk.stride(0), kk.stride(1), kk.stride(2),
-            vk.stride(0), vk.stride(1), vk.stride(2),
-            o.stride(0), o.stride(1), o.stride(2),
-            bf.stride(0), flags.stride(0), flags.stride(1),
-            batch, seqlen_q, nheads, nheads_k, dp, float(softmax_scale), _dtype_code(q.dtype),
-            _stream_ptr(q.device),
-        )
+        if view is None:
+            _bam_hip.call(
+                "bam_fwd",
+                qk.data_ptr(), kk.data_ptr(), vk.data_ptr(), o.data_ptr(), lse.data_ptr(), bf.data_ptr(),
+                flags.data_ptr(), *_strides3(qk, kk, vk, o),
+                bf.stride(0), flags.stride(0), flags.stride(1),
+                batch, seqlen_q, nheads, nheads_k, dp, float(softmax_scale), _dtype_code(q.dtype),
+                _stream_ptr(q.device),
+            )
+        else:
+            _bam_hip.call(
+                "bam_fwd_indexed",
+                qk.data_ptr(), kk.data_ptr(), vk.data_ptr(), o.data_ptr(), lse.data_ptr(), view.byref(),
+                flags.data_ptr(), *_strides3(qk, kk, vk, o),
+                flags.stride(0), flags.stride(1),
+                batch, nheads, nheads_k, dp, float(softmax_scale), _dtype_code(q.dtype),
+                _stream_ptr(q.device),
+            )
     if dp != d:
         o = o[..., :d].contiguous()
     return o, lse, softmax_scale
@@ -202,9 +253,20 @@ def _launch_bwd_preprocess(o, do, delta):
 
 
 def _launch_bwd_dkdv(q, k, v, do, lse, delta, dk, dv, bf, flags, softmax_scale, accumulate=True):
-    """accumulate=True: dk/dv are fp32 and added to; False: dk/dv have q's dtype and are overwritten."""
+    """accumulate=True: dk/dv are fp32 and added to; False: dk/dv have q's dtype and are overwritten.
+    ``bf``: the (B, S) bitfield tensor, or an ``_IndexView`` for index-tensor attention."""
     B, S, Hq, D = q.shape
     with torch.cuda.device(q.device):
+        if isinstance(bf, _IndexView):
+            _bam_hip.call(
+                "bam_bwd_dkdv_indexed",
+                q.data_ptr(), k.data_ptr(), v.data_ptr(), do.data_ptr(), lse.data_ptr(), delta.data_ptr(),
+                dk.data_ptr(), dv.data_ptr(), bf.byref(), flags.data_ptr(),
+                *_strides3(q, k, v, do, dk, dv), flags.stride(0), flags.stride(1),
+                B, Hq, k.shape[2], D, float(softmax_scale), _dtype_code(q.dtype), int(accumulate),
+                _stream_ptr(q.device),
+            )
+            return
         _bam_hip.call(
             "bam_bwd_dkdv",
             q.data_ptr(), k.data_ptr(), v.data_ptr(), do.data_ptr(), lse.data_ptr(), delta.data_ptr(),
@@ -218,6 +280,16 @@ def _launch_bwd_dkdv(q, k, v, do, lse, delta, dk, dv, bf, flags, softmax_scale, 
 def _launch_bwd_dq(q, k, v, do, lse, delta, dq, bf, flags, softmax_scale, accumulate=True):
     B, S, Hq, D = q.shape
     with torch.cuda.device(q.device):
+        if isinstance(bf, _IndexView):
+            _bam_hip.call(
+                "bam_bwd_dq_indexed",
+                q.data_ptr(), k.data_ptr(), v.data_ptr(), do.data_ptr(), lse.data_ptr(), delta.data_ptr(),
+                dq.data_ptr(), bf.byref(), flags.data_ptr(),
+                *_strides3(q, k, v, do, dq), flags.stride(0), flags.stride(1),
+                B, Hq, k.shape[2], D, float(softmax_scale), _dtype_code(q.dtype), int(accumulate),
+                _stream_ptr(q.device),
+            )
+            return
         _bam_hip.call(
             "bam_bwd_dq",
             q.data_ptr(), k.data_ptr(), v.data_ptr(), do.data_ptr(), lse.data_ptr(), delta.data_ptr(),
@@ -286,8 +358,14 @@ def _bitfield_attn_backward(
     assert q.stride(-1) == k.stride(-1) == v.stride(-1) == o.stride(-1) == 1
     assert dq.stride(-1) == dk.stride(-1) == dv.stride(-1) == 1
     assert dq.dtype == dk.dtype == dv.dtype == torch.float32
-    assert q.is_cuda and seqlen_q == seqlen_k
-    _check_unsupported(offsets_q, offsets_k, bias)
+    assert q.is_cuda
+    _check_unsupported(bias)
+    view = None
+    if offsets_q is not None or offsets_k is not None:
+        view = _IndexView(bitfield_mask, offsets_q, offsets_k)
+        assert (view.seqlen_q, view.seqlen_k) == (seqlen_q, seqlen_k), "one offset per local query row / key"
+    else:
+        assert seqlen_q == seqlen_k, "without index tensors query and key sequence lengths must match"
     softmax_scale = softmax_scale or 1.0 / math.sqrt(d)
 
     dp = _padded_head_dim(d)
@@ -299,7 +377,10 @@ def _bitfield_attn_backward(
     work = tuple(_kernel_ready(x, 4) for x in acc)
     lse = lse.contiguous()
     bf = bitfield_mask if bitfield_mask.stride(1) == 1 else bitfield_mask.contiguous()
+    if view is not None:
+        bf = view
     flags = compressed_mask if compressed_mask.stride(-1) == 1 else compressed_mask.contiguous()
+    assert flags.shape == (batch, -(-seqlen_q // BLOCK_M), -(-seqlen_k // BLOCK_N))
     delta = torch.empty_like(lse)
     wq, wk, wv = work
     _launch_bwd_preprocess(ok, gk, delta)

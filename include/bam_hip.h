@@ -36,6 +36,27 @@ extern "C" {
 /* Upper bound on S accepted by the attention kernels (tile lists live in LDS). */
 #define BAM_MAX_SEQLEN 131072
 
+/*
+ * Index-tensor attention (context-parallel shards): the local query rows and keys are arbitrary
+ * subsets / permutations of a global sequence.  The reference passes `offsets_q` / `offsets_k`
+ * down to its mask block, which gathers bitfield[offsets] and compares the gathered positions
+ * (bitfield_attention.py:71-101, 938-939, 1085-1086).  Here the gather is a step of its own
+ * (bam_gather_bitfields) and the attention entry points take its outputs:
+ *   q_bits int64 (B, Sq): bitfield of each local query row,   q_pos int32 (Sq): its global position
+ *   k_bits int64 (B, Sk): bitfield of each local key,         k_pos int32 (Sk): its global position
+ * The struct lives in host memory; the arrays it points at are device memory.
+ */
+typedef struct bam_index_view {
+    const int64_t* q_bits;
+    const int64_t* k_bits;
+    const int32_t* q_pos;
+    const int32_t* k_pos;
+    int64_t q_bits_stride_b;
+    int64_t k_bits_stride_b;
+    int32_t Sq;
+    int32_t Sk;
+} bam_index_view;
+
 const char* bam_last_error(void);
 
 /* ABI version of this library (bumped on any signature change). */
@@ -60,6 +81,15 @@ int bam_tile_flags(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int64_
 int bam_materialize_mask(const int64_t* bf, int64_t bf_stride_b, uint8_t* out, int B, int S, void* stream);
 
 /*
+ * Gather for index-tensor attention: out_bits[b][i] = bf[b][idx[i]], or 0 where idx[i] is outside
+ * [0, L) (the `other=0` of the reference's masked loads, bitfield_attention.py:86-87), and
+ * out_pos[i] = idx[i] as int32.  bf: int64 (B, L); idx: int64 (n); out_bits: int64 (B, n) with row
+ * stride out_stride_b; out_pos: int32 (n).
+ */
+int bam_gather_bitfields(const int64_t* bf, int64_t bf_stride_b, int L, const int64_t* idx, int n, int64_t* out_bits,
+                         int64_t out_stride_b, int32_t* out_pos, int B, void* stream);
+
+/*
  * Forward.  Replaces `_fwd_kernel[grid]` + `_aggregate_partial_outputs[grid]` in
  * `_bitfield_attn_forward` (bitfield_attention.py:236-523, 932-1069, 1292-1436):
  *   o = softmax_allowed(scale * q k^T) v,  lse = log sum_allowed exp(scale * q k^T);
@@ -72,6 +102,20 @@ int bam_fwd(const void* q, const void* k, const void* v, void* o, float* lse, co
             int64_t v_stride_s, int64_t v_stride_h, int64_t o_stride_b, int64_t o_stride_s,
             int64_t o_stride_h, int64_t bf_stride_b, int64_t flags_stride_b, int64_t flags_stride_m, int B,
             int S, int Hq, int Hkv, int D, float scale, int dtype, void* stream);
+
+/*
+ * Forward with index tensors (`offsets_q` / `offsets_k` of `_bitfield_attn_forward`,
+ * bitfield_attention.py:938-939, as used by
+ * shardformer/layers/context_parallel_bitfield_attention.py:137-147).  q is (B, Sq, Hq, D),
+ * k / v are (B, Sk, Hkv, D), flags are (B, ceil(Sq/128), ceil(Sk/32)) over LOCAL tiles,
+ * lse is (B, Hq, ceil(Sq/128)*128).
+ */
+int bam_fwd_indexed(const void* q, const void* k, const void* v, void* o, float* lse, const bam_index_view* iv,
+                    const int8_t* flags, int64_t q_stride_b, int64_t q_stride_s, int64_t q_stride_h,
+                    int64_t k_stride_b, int64_t k_stride_s, int64_t k_stride_h, int64_t v_stride_b,
+                    int64_t v_stride_s, int64_t v_stride_h, int64_t o_stride_b, int64_t o_stride_s,
+                    int64_t o_stride_h, int64_t flags_stride_b, int64_t flags_stride_m, int B, int Hq, int Hkv,
+                    int D, float scale, int dtype, void* stream);
 
 /*
  * delta[b,h,i] = sum_d o[b,i,h,d] * do[b,i,h,d] in fp32.  Replaces
@@ -127,6 +171,30 @@ int bam_bwd_dq(const void* q, const void* k, const void* v, const void* dout, co
                int64_t dq_stride_s, int64_t dq_stride_h, int64_t bf_stride_b, int64_t flags_stride_b,
                int64_t flags_stride_m, int B, int S, int Hq, int Hkv, int D, float scale, int dtype,
                int accumulate, void* stream);
+
+/*
+ * bam_bwd_dkdv / bam_bwd_dq with index tensors (`offsets_q` / `offsets_k` of
+ * `_bitfield_attn_backward`, bitfield_attention.py:1085-1086, as used by
+ * shardformer/layers/context_parallel_bitfield_attention.py:270-294).  dk / dv are (B, Sk, Hkv, D)
+ * in LOCAL key order; dq is (B, Sq, Hq, D).
+ */
+int bam_bwd_dkdv_indexed(const void* q, const void* k, const void* v, const void* dout, const float* lse,
+                         const float* delta, void* dk, void* dv, const bam_index_view* iv, const int8_t* flags,
+                         int64_t q_stride_b, int64_t q_stride_s, int64_t q_stride_h, int64_t k_stride_b,
+                         int64_t k_stride_s, int64_t k_stride_h, int64_t v_stride_b, int64_t v_stride_s,
+                         int64_t v_stride_h, int64_t do_stride_b, int64_t do_stride_s, int64_t do_stride_h,
+                         int64_t dk_stride_b, int64_t dk_stride_s, int64_t dk_stride_h, int64_t dv_stride_b,
+                         int64_t dv_stride_s, int64_t dv_stride_h, int64_t flags_stride_b, int64_t flags_stride_m,
+                         int B, int Hq, int Hkv, int D, float scale, int dtype, int accumulate, void* stream);
+
+int bam_bwd_dq_indexed(const void* q, const void* k, const void* v, const void* dout, const float* lse,
+                       const float* delta, void* dq, const bam_index_view* iv, const int8_t* flags,
+                       int64_t q_stride_b, int64_t q_stride_s, int64_t q_stride_h, int64_t k_stride_b,
+                       int64_t k_stride_s, int64_t k_stride_h, int64_t v_stride_b, int64_t v_stride_s,
+                       int64_t v_stride_h, int64_t do_stride_b, int64_t do_stride_s, int64_t do_stride_h,
+                       int64_t dq_stride_b, int64_t dq_stride_s, int64_t dq_stride_h, int64_t flags_stride_b,
+                       int64_t flags_stride_m, int B, int Hq, int Hkv, int D, float scale, int dtype,
+                       int accumulate, void* stream);
 
 #ifdef __cplusplus
 }

@@ -24,6 +24,12 @@ What pins each function (the pins live in ``tests/test_oracle.py``):
 * ``attention_backward`` -- ``torch.autograd.grad`` through the explicit forward,
   pinned against autograd through SDPA (``test_bitfield_attention.py:198-204``)
   and against the closed-form C restatement in ``bam_oracle.c``.
+* index tensors (``idx_q`` / ``idx_k`` of ``allow_rows``, ``attention_forward``,
+  ``attention_backward``, ``tile_flags_indexed``) -- the indexed mask equals a gather of the
+  pinned global mask; indexed attention over permuted keys equals the plain result gathered at
+  ``idx_q`` (what the reference's context-parallel test asserts,
+  ``tests/test_shardformer/test_context_parallel.py:311-376``); for block-aligned index sets the
+  flags equal the reference's gather of the global flags (``shardformer/layers/utils.py:331-353``).
 * ``create_bitfield_attention_mask`` -- golden vectors of
   ``tests/test_models/test_multimodal_merge_outputs.py:94-110``.
 
@@ -121,6 +127,29 @@ def tile_flags(bitfield: torch.Tensor) -> torch.Tensor:
     return out
 
 
+def tile_flags_indexed(bitfield: torch.Tensor, idx_q: torch.Tensor, idx_k: torch.Tensor) -> torch.Tensor:
+    """Flags of the LOCAL tiles of index-tensor attention: int8 (B, ceil(Sq/128), ceil(Sk/32)) over
+    the mask whose row i / column j stand for global positions idx_q[i] / idx_k[j].  When the
+    index sets are made of whole, aligned blocks this equals the reference's recipe of gathering
+    rows and columns of the global flags (shardformer/layers/utils.py:331-353)."""
+    B = bitfield.shape[0]
+    Sq, Sk = idx_q.numel(), idx_k.numel()
+    nm, nn = -(-Sq // BLOCK_M), -(-Sk // BLOCK_N)
+    out = torch.zeros((B, nm, nn), dtype=torch.int8, device=bitfield.device)
+    cols = torch.full((nn,), BLOCK_N, dtype=torch.int64, device=bitfield.device)
+    if Sk % BLOCK_N:
+        cols[-1] = Sk % BLOCK_N
+    for b in range(B):
+        for m in range(nm):
+            r0, r1 = m * BLOCK_M, min((m + 1) * BLOCK_M, Sq)
+            a = allow_rows(bitfield[b], r0, r1, idx_q, idx_k)
+            a = F.pad(a, (0, nn * BLOCK_N - Sk))
+            cnt = a.view(r1 - r0, nn, BLOCK_N).sum(dim=(0, 2))
+            full = cnt == (r1 - r0) * cols
+            out[b, m] = torch.where(cnt == 0, 0, torch.where(full, 2, 1)).to(torch.int8)
+    return out
+
+
 def unmasked_pairs(bitfield: torch.Tensor) -> int:
     """Number of allowed (query, key) pairs over the whole batch."""
     B, S = bitfield.shape
@@ -182,8 +211,12 @@ def _chunk_forward(qc, kb, vb, allow, scale):
     return o, lse
 
 
-def attention_forward(q, k, v, bitfield, softmax_scale=None, row_chunk=1024, dtype=torch.float32):
-    """Explicit masked softmax attention -> (o (B,S,Hq,D), lse (B,Hq,S)) in ``dtype``."""
+def attention_forward(q, k, v, bitfield, softmax_scale=None, row_chunk=1024, dtype=torch.float32,
+                      idx_q=None, idx_k=None):
+    """Explicit masked softmax attention -> (o (B,S,Hq,D), lse (B,Hq,S)) in ``dtype``.
+    With index tensors q holds the rows at global positions ``idx_q`` and k/v the keys at
+    ``idx_k`` (any order); ``bitfield`` stays indexed by global position
+    (bitfield_attention.py:71-87)."""
     B, S, Hq, D = q.shape
     scale = softmax_scale or 1.0 / math.sqrt(D)
     q, k, v = q.to(dtype), k.to(dtype), v.to(dtype)
@@ -192,14 +225,15 @@ def attention_forward(q, k, v, bitfield, softmax_scale=None, row_chunk=1024, dty
     for b in range(B):
         for r0 in range(0, S, row_chunk):
             r1 = min(r0 + row_chunk, S)
-            allow = allow_rows(bitfield[b], r0, r1)
+            allow = allow_rows(bitfield[b], r0, r1, idx_q, idx_k)
             oc, lc = _chunk_forward(q[b, r0:r1], k[b], v[b], allow, scale)
             o[b, r0:r1] = oc
             lse[b, :, r0:r1] = lc
     return o, lse
 
 
-def attention_backward(q, k, v, bitfield, do, softmax_scale=None, row_chunk=1024, dtype=torch.float32):
+def attention_backward(q, k, v, bitfield, do, softmax_scale=None, row_chunk=1024, dtype=torch.float32,
+                       idx_q=None, idx_k=None):
     """dq, dk, dv of sum(o * do) by autograd through the explicit forward, one row
     chunk at a time (bounded memory).  Matches the reference's gradient contract
     (bitfield_attention.py:840-886): dk/dv are summed over the q-heads of a group."""
@@ -212,7 +246,7 @@ def attention_backward(q, k, v, bitfield, do, softmax_scale=None, row_chunk=1024
     for b in range(B):
         for r0 in range(0, S, row_chunk):
             r1 = min(r0 + row_chunk, S)
-            allow = allow_rows(bitfield[b], r0, r1)
+            allow = allow_rows(bitfield[b], r0, r1, idx_q, idx_k)
             qc = q[b, r0:r1].detach().requires_grad_(True)
             kb = k[b].detach().requires_grad_(True)
             vb = v[b].detach().requires_grad_(True)

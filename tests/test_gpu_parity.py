@@ -283,8 +283,10 @@ def test_backward_accumulates_into_caller_buffers():
         assert torch.allclose(a + 1, b, atol=1e-6)
     with pytest.raises(NotImplementedError):
         BA._bitfield_attn_forward(q, k, v, bfg, flags, bias=torch.zeros(1, 2, 1, 256, device=d))
-    with pytest.raises(NotImplementedError):
-        BA._bitfield_attn_forward(q, k, v, bfg, flags, offsets_q=torch.arange(256, device=d))
+    # identity index tensors change nothing
+    ar = torch.arange(256, device=d)
+    o2, lse2, _ = BA._bitfield_attn_forward(q, k, v, bfg, flags, offsets_q=ar, offsets_k=ar)
+    assert torch.equal(o2, o) and torch.equal(lse2, lse)
 
 
 # -------------------------------------------------- the five benchmark configurations

@@ -219,3 +219,57 @@ def test_all_text_bitfield_is_plain_causal_attention():
     ).transpose(1, 2)
     o, _ = O.attention_forward(q, k, v, bf)
     assert torch.allclose(o, want, atol=1e-5)
+
+
+# ------------------------------------------------------------------ index tensors (context-parallel shards)
+def _cp_splits(S, kind):
+    """Index sets of two 'ranks' the way the reference splits a sequence
+    (shardformer/layers/utils.py:108-146, 180-197): contiguous, zigzag, whole 128-row blocks."""
+    if kind == "uniform":
+        chunks = np.array_split(np.arange(S), 2)
+    elif kind == "zigzag":
+        c = np.array_split(np.arange(S), 4)
+        chunks = [np.concatenate([c[0], c[3]]), np.concatenate([c[1], c[2]])]
+    else:  # whole 128-row blocks dealt alternately, sorted per rank
+        blocks = np.arange(-(-S // 128))
+        chunks = [np.concatenate([np.arange(b * 128, min((b + 1) * 128, S)) for b in blocks[r::2]]) for r in range(2)]
+    return [torch.from_numpy(c.astype(np.int64)) for c in chunks]
+
+
+@pytest.mark.parametrize("kind", ["uniform", "zigzag", "blocks"])
+def test_indexed_attention_is_the_plain_result_gathered(kind):
+    # what the reference's context-parallel test asserts (test_context_parallel.py:311-376): each rank's
+    # output / dq equals its rows of the plain result, and dk / dv summed over the ranks equal the plain ones
+    S, Hq, Hkv, D = 300, 4, 2, 16
+    bf = random_bitfield(1, S, seed=5)
+    q, k, v, do = _rand(1, S, Hq, Hkv, D, seed=2, dtype=torch.float64)
+    o, lse = O.attention_forward(q, k, v, bf, dtype=torch.float64)
+    dq, dk, dv = O.attention_backward(q, k, v, bf, do, dtype=torch.float64)
+    ranks = _cp_splits(S, kind)
+    idx_k = torch.cat(ranks)
+    sum_dk, sum_dv = torch.zeros_like(dk), torch.zeros_like(dv)
+    for idx_q in ranks:
+        ql, dol = q[:, idx_q], do[:, idx_q]
+        kl, vl = k[:, idx_k], v[:, idx_k]
+        ol, lsel = O.attention_forward(ql, kl, vl, bf, dtype=torch.float64, idx_q=idx_q, idx_k=idx_k)
+        assert torch.allclose(ol, o[:, idx_q], atol=1e-12, rtol=0)
+        assert torch.allclose(lsel, lse[:, :, idx_q], atol=1e-12, rtol=0)
+        gq, gk, gv = O.attention_backward(ql, kl, vl, bf, dol, dtype=torch.float64, idx_q=idx_q, idx_k=idx_k)
+        assert torch.allclose(gq, dq[:, idx_q], atol=1e-12, rtol=0)
+        sum_dk[:, idx_k] += gk
+        sum_dv[:, idx_k] += gv
+    assert torch.allclose(sum_dk, dk, atol=1e-11, rtol=0) and torch.allclose(sum_dv, dv, atol=1e-11, rtol=0)
+
+
+def test_indexed_flags_equal_the_reference_gather_of_global_flags_for_aligned_blocks():
+    # the recipe of ContextParallelBatchSplitUtils.get_local_compressed_mask (utils.py:331-353):
+    # rows offsets_q[::128] // 128 and columns cat(offsets[::32]) // 32 of the global flags
+    S = 640
+    bf = random_bitfield(2, S, seed=9)
+    glob = O.tile_flags(bf)
+    ranks = _cp_splits(S, "blocks")
+    idx_k = torch.cat(ranks)
+    cols = torch.cat([r[::32] for r in ranks]) // 32
+    for idx_q in ranks:
+        want = glob[:, idx_q[::128] // 128][:, :, cols]
+        assert torch.equal(O.tile_flags_indexed(bf, idx_q, idx_k), want)
