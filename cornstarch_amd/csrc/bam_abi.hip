@@ -66,14 +66,20 @@ int launched(int hip_err, const char* what) {
 // Where the kernels find bitfields and positions: one (B, S) tensor for plain attention, gathered
 // per-row / per-key arrays plus positions for index-tensor attention.
 struct MaskSource {
+    int mode;
     const int64_t *bfq, *bfk;
     int64_t bfq_sb, bfk_sb;
     const int *posq, *posk;
+    const uint8_t* mask;
     int Sq, Sk;
 };
 
 MaskSource plain_source(const int64_t* bf, int64_t bf_stride_b, int S) {
-    return MaskSource{bf, bf, bf_stride_b, bf_stride_b, nullptr, nullptr, S, S};
+    return MaskSource{bam::MASK_BITFIELD, bf, bf, bf_stride_b, bf_stride_b, nullptr, nullptr, nullptr, S, S};
+}
+
+MaskSource dense_source(const uint8_t* mask, int Sq, int Sk) {
+    return MaskSource{bam::MASK_DENSE, nullptr, nullptr, 0, 0, nullptr, nullptr, mask, Sq, Sk};
 }
 
 int indexed_source(const bam_index_view* iv, MaskSource& m) {
@@ -83,7 +89,8 @@ int indexed_source(const bam_index_view* iv, MaskSource& m) {
     if ((reinterpret_cast<uintptr_t>(iv->q_bits) & 7u) || (reinterpret_cast<uintptr_t>(iv->k_bits) & 7u) ||
         (reinterpret_cast<uintptr_t>(iv->q_pos) & 3u) || (reinterpret_cast<uintptr_t>(iv->k_pos) & 3u))
         return fail(BAM_ERR_INVALID_ARGUMENT, "index view: misaligned array");
-    m = MaskSource{iv->q_bits, iv->k_bits, iv->q_bits_stride_b, iv->k_bits_stride_b, iv->q_pos, iv->k_pos, iv->Sq, iv->Sk};
+    m = MaskSource{bam::MASK_INDEXED, iv->q_bits, iv->k_bits, iv->q_bits_stride_b, iv->k_bits_stride_b,
+                   iv->q_pos,         iv->k_pos,  nullptr,             iv->Sq,              iv->Sk};
     return BAM_OK;
 }
 
@@ -94,6 +101,8 @@ void fill_sizes(bam::AttnParams& p, const MaskSource& m, int B, int Hq, int Hkv,
     p.bfk_sb = m.bfk_sb;
     p.posq = m.posq;
     p.posk = m.posk;
+    p.mask = m.mask;
+    p.mask_mode = m.mode;
     p.B = B;
     p.Sq = m.Sq;
     p.Sk = m.Sk;
@@ -133,7 +142,7 @@ int fwd_impl(const char* who, const void* q, const void* k, const void* v, void*
     BAM_TRY(check_half_tensor("k", k, st[3], st[4], st[5]));
     BAM_TRY(check_half_tensor("v", v, st[6], st[7], st[8]));
     BAM_TRY(check_half_tensor("o", o, st[9], st[10], st[11]));
-    if (lse == nullptr || m.bfq == nullptr || m.bfk == nullptr || flags == nullptr)
+    if (lse == nullptr || flags == nullptr || (m.mode != bam::MASK_DENSE && (m.bfq == nullptr || m.bfk == nullptr)))
         return fail(BAM_ERR_INVALID_ARGUMENT, "%s: lse, bitfields and flags must not be null", who);
     if (!(scale > 0.f)) return fail(BAM_ERR_INVALID_ARGUMENT, "%s: softmax scale must be > 0 (got %g)", who, scale);
     bam::AttnParams p = {};
@@ -173,7 +182,8 @@ int bwd_params(bam::AttnParams& p, const char* who, const void* q, const void* k
         }
     }
     p.grad_typed = accumulate ? 0 : 1;
-    if (lse == nullptr || delta == nullptr || m.bfq == nullptr || m.bfk == nullptr || flags == nullptr)
+    if (lse == nullptr || delta == nullptr || flags == nullptr ||
+        (m.mode != bam::MASK_DENSE && (m.bfq == nullptr || m.bfk == nullptr)))
         return fail(BAM_ERR_INVALID_ARGUMENT, "%s: lse, delta, bitfields and flags must not be null", who);
     if (!(scale > 0.f)) return fail(BAM_ERR_INVALID_ARGUMENT, "%s: softmax scale must be > 0 (got %g)", who, scale);
     p.q = {q, st[0], st[1], st[2]};
@@ -198,7 +208,7 @@ extern "C" {
 
 const char* bam_last_error(void) { return g_error; }
 
-int bam_abi_version(void) { return 3; }
+int bam_abi_version(void) { return 4; }
 
 int bam_tile_flags(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int64_t flags_stride_b,
                    int64_t flags_stride_m, int B, int S, void* stream) {
@@ -218,6 +228,16 @@ int bam_materialize_mask(const int64_t* bf, int64_t bf_stride_b, uint8_t* out, i
         return fail(BAM_ERR_UNSUPPORTED, "bam_materialize_mask: B and S are limited to 65535 (got %d, %d)", B, S);
     return launched(bam::launch_materialize_mask(bf, bf_stride_b, out, B, S, (hipStream_t)stream),
                     "bam_materialize_mask");
+}
+
+int bam_flag_row_workloads(const int8_t* flags, int64_t flags_stride_b, int64_t flags_stride_m, int B, int num_m,
+                           int num_n, int32_t* out, void* stream) {
+    if (flags == nullptr || out == nullptr) return fail(BAM_ERR_INVALID_ARGUMENT, "bam_flag_row_workloads: null pointer");
+    if (B <= 0 || num_m <= 0 || num_n <= 0)
+        return fail(BAM_ERR_INVALID_ARGUMENT, "bam_flag_row_workloads: B, num_m and num_n must be positive");
+    return launched(bam::launch_flag_row_workloads(flags, flags_stride_b, flags_stride_m, B, num_m, num_n, out,
+                                                   (hipStream_t)stream),
+                    "bam_flag_row_workloads");
 }
 
 int bam_gather_bitfields(const int64_t* bf, int64_t bf_stride_b, int L, const int64_t* idx, int n, int64_t* out_bits,
@@ -270,7 +290,7 @@ int bam_bwd_preprocess(const void* o, const void* dout, float* delta, int64_t o_
     p.o = {o, o_stride_b, o_stride_s, o_stride_h};
     p.dout = {dout, do_stride_b, do_stride_s, do_stride_h};
     p.delta = delta;
-    fill_sizes(p, plain_source(nullptr, 0, S), B, Hq, Hq, D, 1.f);
+    fill_sizes(p, plain_source(nullptr, 0, S), B, Hq, Hq, D, 1.f);  // the preprocess kernel never looks at the mask
     return launched(bam::launch_bwd_preprocess(p, dtype, (hipStream_t)stream), "bam_bwd_preprocess");
 }
 
@@ -367,6 +387,61 @@ int bam_bwd_dq_indexed(const void* q, const void* k, const void* v, const void* 
     BAM_TRY(bwd_params(p, "bam_bwd_dq_indexed", q, k, v, dout, lse, delta, dq, dk, dv, m, flags, st, B, Hq, Hkv, D, scale,
                        dtype, accumulate, true, false));
     return launched(bam::launch_bwd_dq(p, dtype, (hipStream_t)stream), "bam_bwd_dq_indexed");
+}
+
+int bam_mask_tile_flags(const uint8_t* mask, int8_t* flags, int64_t flags_stride_b, int64_t flags_stride_m, int B,
+                        int Sq, int Sk, void* stream) {
+    if (mask == nullptr || flags == nullptr) return fail(BAM_ERR_INVALID_ARGUMENT, "bam_mask_tile_flags: null pointer");
+    if (B <= 0 || Sq <= 0 || Sk <= 0) return fail(BAM_ERR_INVALID_ARGUMENT, "bam_mask_tile_flags: B, Sq and Sk must be positive");
+    if (B > 65535 || (Sq + 127) / 128 > 65535)
+        return fail(BAM_ERR_UNSUPPORTED, "bam_mask_tile_flags: grid too large (B = %d, Sq = %d)", B, Sq);
+    return launched(bam::launch_mask_tile_flags(mask, flags, flags_stride_b, flags_stride_m, B, Sq, Sk, (hipStream_t)stream),
+                    "bam_mask_tile_flags");
+}
+
+int bam_fwd_masked(const void* q, const void* k, const void* v, void* o, float* lse, const uint8_t* mask,
+                   const int8_t* flags, int64_t q_stride_b, int64_t q_stride_s, int64_t q_stride_h,
+                   int64_t k_stride_b, int64_t k_stride_s, int64_t k_stride_h, int64_t v_stride_b,
+                   int64_t v_stride_s, int64_t v_stride_h, int64_t o_stride_b, int64_t o_stride_s,
+                   int64_t o_stride_h, int64_t flags_stride_b, int64_t flags_stride_m, int B, int Sq, int Sk, int Hq,
+                   int Hkv, int D, float scale, int dtype, void* stream) {
+    const int64_t st[12] = BAM_FWD_STRIDES;
+    return fwd_impl("bam_fwd_masked", q, k, v, o, lse, dense_source(mask, Sq, Sk), flags, st, flags_stride_b,
+                    flags_stride_m, B, Hq, Hkv, D, scale, dtype, stream);
+}
+
+int bam_bwd_dkdv_masked(const void* q, const void* k, const void* v, const void* dout, const float* lse,
+                        const float* delta, void* dk, void* dv, const uint8_t* mask, const int8_t* flags,
+                        int64_t q_stride_b, int64_t q_stride_s, int64_t q_stride_h, int64_t k_stride_b,
+                        int64_t k_stride_s, int64_t k_stride_h, int64_t v_stride_b, int64_t v_stride_s,
+                        int64_t v_stride_h, int64_t do_stride_b, int64_t do_stride_s, int64_t do_stride_h,
+                        int64_t dk_stride_b, int64_t dk_stride_s, int64_t dk_stride_h, int64_t dv_stride_b,
+                        int64_t dv_stride_s, int64_t dv_stride_h, int64_t flags_stride_b, int64_t flags_stride_m,
+                        int B, int Sq, int Sk, int Hq, int Hkv, int D, float scale, int dtype, int accumulate,
+                        void* stream) {
+    void* dq = nullptr;
+    const int64_t dq_stride_b = 0, dq_stride_s = 0, dq_stride_h = 0;
+    const int64_t st[23] = BAM_BWD_STRIDES;
+    bam::AttnParams p = {};
+    BAM_TRY(bwd_params(p, "bam_bwd_dkdv_masked", q, k, v, dout, lse, delta, dq, dk, dv, dense_source(mask, Sq, Sk), flags,
+                       st, B, Hq, Hkv, D, scale, dtype, accumulate, false, true));
+    return launched(bam::launch_bwd_dkdv(p, dtype, (hipStream_t)stream), "bam_bwd_dkdv_masked");
+}
+
+int bam_bwd_dq_masked(const void* q, const void* k, const void* v, const void* dout, const float* lse,
+                      const float* delta, void* dq, const uint8_t* mask, const int8_t* flags, int64_t q_stride_b,
+                      int64_t q_stride_s, int64_t q_stride_h, int64_t k_stride_b, int64_t k_stride_s,
+                      int64_t k_stride_h, int64_t v_stride_b, int64_t v_stride_s, int64_t v_stride_h,
+                      int64_t do_stride_b, int64_t do_stride_s, int64_t do_stride_h, int64_t dq_stride_b,
+                      int64_t dq_stride_s, int64_t dq_stride_h, int64_t flags_stride_b, int64_t flags_stride_m, int B,
+                      int Sq, int Sk, int Hq, int Hkv, int D, float scale, int dtype, int accumulate, void* stream) {
+    void *dk = nullptr, *dv = nullptr;
+    const int64_t dk_stride_b = 0, dk_stride_s = 0, dk_stride_h = 0, dv_stride_b = 0, dv_stride_s = 0, dv_stride_h = 0;
+    const int64_t st[23] = BAM_BWD_STRIDES;
+    bam::AttnParams p = {};
+    BAM_TRY(bwd_params(p, "bam_bwd_dq_masked", q, k, v, dout, lse, delta, dq, dk, dv, dense_source(mask, Sq, Sk), flags, st,
+                       B, Hq, Hkv, D, scale, dtype, accumulate, true, false));
+    return launched(bam::launch_bwd_dq(p, dtype, (hipStream_t)stream), "bam_bwd_dq_masked");
 }
 
 }  // extern "C"

@@ -5,6 +5,11 @@
 
 namespace bam {
 
+// Where the allow / deny decision of a (query, key) pair comes from.
+constexpr int MASK_BITFIELD = 0;  // bitfield rule, position = row / column number
+constexpr int MASK_INDEXED = 1;   // bitfield rule on gathered bitfields and explicit global positions
+constexpr int MASK_DENSE = 2;     // a materialized bool mask (B, Sq, Sk), one byte per pair (or none: all pairs allowed)
+
 // Number of 64-key (forward, dQ) or 128-row (dK/dV) tiles a workgroup can list in LDS.
 constexpr int MAX_LIST = 2048;
 
@@ -27,6 +32,9 @@ struct AttnParams {
     int64_t bfq_sb, bfk_sb;
     const int* posq;
     const int* posk;
+    // MASK_DENSE: bool mask (B, Sq, Sk), contiguous, one byte per pair; null = every in-range pair allowed
+    const uint8_t* mask;
+    int mask_mode;             // MASK_BITFIELD / MASK_INDEXED / MASK_DENSE
     const int8_t* flags;       // (B, num_m, num_n)
     int64_t flags_sb, flags_sm;
     int B, Sq, Sk, Hq, Hkv, D;
@@ -38,6 +46,10 @@ int launch_tile_flags(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int
                       int64_t flags_stride_m, int B, int S, hipStream_t stream);
 int launch_materialize_mask(const int64_t* bf, int64_t bf_stride_b, uint8_t* out, int B, int S,
                             hipStream_t stream);
+int launch_flag_row_workloads(const int8_t* flags, int64_t flags_stride_b, int64_t flags_stride_m, int B, int num_m,
+                              int num_n, int* out, hipStream_t stream);
+int launch_mask_tile_flags(const uint8_t* mask, int8_t* flags, int64_t flags_stride_b, int64_t flags_stride_m, int B,
+                           int Sq, int Sk, hipStream_t stream);
 int launch_gather_bitfields(const int64_t* bf, int64_t bf_stride_b, int L, const int64_t* idx, int n, int64_t* out_bits,
                             int64_t out_stride_b, int* out_pos, int B, hipStream_t stream);
 int launch_fwd(const AttnParams& p, int dtype, hipStream_t stream);

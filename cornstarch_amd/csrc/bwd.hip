@@ -61,9 +61,11 @@ __global__ __launch_bounds__(256) void bwd_preprocess_kernel(const AttnParams p)
 constexpr int DKDV_QT = 64;
 constexpr int DKDV_THREADS = 512;
 
-// IDX: index-tensor attention (explicit global positions p.posq / p.posk, gathered bitfield arrays).
-template <typename T, int D, bool IDX>
+// MODE (MASK_*): MASK_INDEXED = explicit global positions p.posq / p.posk and gathered bitfield arrays;
+// MASK_DENSE = a materialized bool mask read from global memory in partial tiles.
+template <typename T, int D, int MODE>
 __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnParams p) {
+    constexpr bool IDX = MODE == MASK_INDEXED, DENSE = MODE == MASK_DENSE;
     constexpr int NCH = D / 8, KK = D / 16, DB = D / 32;
     __shared__ u32x4 sK[128 * NCH];
     __shared__ u32x4 sV[128 * NCH];
@@ -106,7 +108,7 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
     const int key = nt * 128 + kg * 32 + l32;
     const bool kvalid = key < Sk;
     const int64_t* bfrow = p.bfq + (int64_t)b * p.bfq_sb;  // bitfields of the query rows
-    const int64_t kf = kvalid ? p.bfk[(int64_t)b * p.bfk_sb + key] : 0;
+    const int64_t kf = (!DENSE && kvalid) ? p.bfk[(int64_t)b * p.bfk_sb + key] : 0;
     int kpos = (IDX && kvalid) ? p.posk[key] : key;  // global position of this lane's key
     unsigned klo = (unsigned)(kf & 0xFFFFFFFFll);
     unsigned khi = (unsigned)((uint64_t)kf >> 32);
@@ -140,7 +142,7 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
     // small rows of a tile: lse, delta and the two halves of the 64 int64 bitfields, 64 dwords each;
     // wave w copies row w & 3 (waves 4..7 repeat what waves 0..3 write, so that every wave issues the same
     // number of copies)
-    const int small = wave & 3;
+    const int small = DENSE ? (wave & 1) : (wave & 3);
     const unsigned ldsSmall = small == 0 ? lds_addr(sLse) : small == 1 ? lds_addr(sDelta) : lds_addr(sQbf) + (small - 2) * 256u;
     const unsigned smallBytes = small < 2 ? DKDV_QT * 4u : DKDV_QT * 8u;  // per buffer
     // Copy instruction j of the full 64-row tile (head h, first row row0) into buffer buf.
@@ -216,7 +218,19 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
 #pragma unroll
             for (int x = 0; x < 4; ++x) s[4 * grp + x] = __builtin_amdgcn_exp2f(fmaf(s[4 * grp + x], c2, l4[x] * -LOG2E));
         }
-        if (cls == 1) {
+        if (DENSE) {
+            if (cls == 1) {
+                // mask bytes of this lane's key column, one per row of the C fragment
+                const uint8_t* mcol = p.mask + ((int64_t)b * Sq + row0 + qr) * Sk + key;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const int r = 8 * (i >> 2) + 4 * hi + (i & 3);
+                    bool a = kvalid && row0 + qr + r < Sq;
+                    if (a && p.mask != nullptr) a = mcol[(int64_t)r * Sk] != 0;
+                    s[i] = a ? s[i] : 0.f;
+                }
+            }
+        } else if (cls == 1) {
             // Most partial tiles are partial only through causality: the 32 rows carry the same bitfield.
             // Then the bit test is a per-key constant and the rule reduces to one position compare.
             const int64_t mine = sQbf[cur][qr + l32];
@@ -368,7 +382,7 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
                 const bool ok = tid < rows;
                 sLse[0][tid] = ok ? p.lse[off + tid] : INFINITY;  // lse = +inf gives P = 0
                 sDelta[0][tid] = ok ? p.delta[off + tid] : 0.f;
-                sQbf[0][tid] = ok ? bfrow[row0 + tid] : 0;
+                if (!DENSE) sQbf[0][tid] = ok ? bfrow[row0 + tid] : 0;
                 if (IDX) sQpos[0][tid] = ok ? p.posq[row0 + tid] : 0;
             }
             __syncthreads();
@@ -456,8 +470,9 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
 constexpr int DQ_KT = 64;
 constexpr int DQ_THREADS = 256;
 
-template <typename T, int D, bool IDX>
+template <typename T, int D, int MODE>
 __global__ __launch_bounds__(DQ_THREADS, 2) void bwd_dq_kernel(const AttnParams p) {
+    constexpr bool IDX = MODE == MASK_INDEXED, DENSE = MODE == MASK_DENSE;
     constexpr int NCH = D / 8, KK = D / 16, DB = D / 32;
     __shared__ u32x4 sK[2][DQ_KT * NCH];
     __shared__ u32x4 sV[2][DQ_KT * NCH];
@@ -500,7 +515,7 @@ __global__ __launch_bounds__(DQ_THREADS, 2) void bwd_dq_kernel(const AttnParams 
             greg[kk] = zg;
         }
     }
-    const int64_t qf = qvalid ? p.bfq[(int64_t)b * p.bfq_sb + qrow] : 0;
+    const int64_t qf = (!DENSE && qvalid) ? p.bfq[(int64_t)b * p.bfq_sb + qrow] : 0;
     const QueryBits qb = make_query_bits(qf, (IDX && qvalid) ? p.posq[qrow] : qrow);
     float lse2 = INFINITY, dlt = 0.f;
     if (qvalid) {
@@ -528,7 +543,7 @@ __global__ __launch_bounds__(DQ_THREADS, 2) void bwd_dq_kernel(const AttnParams 
     typedef TileStage<D, DQ_KT, DQ_THREADS> Stage;
     constexpr int CPT = Stage::CPT;
     // copy instructions per wave and tile: K, V, the key bitfields and (IDX) the key positions
-    constexpr int NLOADS = 2 * CPT + 1 + (IDX ? 1 : 0);
+    constexpr int NLOADS = 2 * CPT + (DENSE ? 0 : 1) + (IDX ? 1 : 0);
     static_assert(NLOADS <= 2 * KK, "one copy per MFMA of the first S / dP block");
     Stage stK, stV;
     stK.setup(2 * p.k.ss, tid);
@@ -558,7 +573,7 @@ __global__ __launch_bounds__(DQ_THREADS, 2) void bwd_dq_kernel(const AttnParams 
         // partial tile whose 64 keys all carry the same bitfield: the rule is one position compare
         bool uniform_keys = false;
         int rel = 0;
-        if (cls == 1) {
+        if (!DENSE && cls == 1) {
             const int64_t mine = sKbf[cur][lane];
             const unsigned mlo = (unsigned)mine, mhi = (unsigned)((uint64_t)mine >> 32);
             const unsigned flo = __builtin_amdgcn_readfirstlane(mlo), fhi = __builtin_amdgcn_readfirstlane(mhi);
@@ -599,7 +614,34 @@ __global__ __launch_bounds__(DQ_THREADS, 2) void bwd_dq_kernel(const AttnParams 
                 const float e = __builtin_amdgcn_exp2f(fmaf(s[i], c2, -lse2));
                 dp[i] = e * (dp[i] - dlt);  // the factor `scale` of dS is applied to dQ in the epilogue
             }
-            if (cls == 1) {
+            if (DENSE) {
+                if (cls == 1) {
+                    const int kt0 = kt * DQ_KT;
+                    const uint8_t* mrow = p.mask + ((int64_t)b * Sq + (qvalid ? qrow : 0)) * Sk + kt0;
+                    const bool dwords = (Sk & 3) == 0;  // rows start 4-byte aligned
+#pragma unroll
+                    for (int grp = 0; grp < 4; ++grp) {
+                        const int koff = 32 * kb + 8 * grp + 4 * hi;
+                        unsigned m4 = 0;
+                        if (p.mask == nullptr) {
+                            m4 = 0x01010101u;
+                        } else if (qvalid) {
+                            if (dwords) {
+                                if (kt0 + koff < Sk) m4 = *(const unsigned*)(mrow + koff);
+                            } else {
+#pragma unroll
+                                for (int x = 0; x < 4; ++x)
+                                    if (kt0 + koff + x < Sk) m4 |= (unsigned)mrow[koff + x] << (8 * x);
+                            }
+                        }
+#pragma unroll
+                        for (int x = 0; x < 4; ++x) {
+                            const bool a = ((m4 >> (8 * x)) & 0xFFu) != 0 && kt0 + koff + x < Sk;
+                            dp[4 * grp + x] = a ? dp[4 * grp + x] : 0.f;
+                        }
+                    }
+                }
+            } else if (cls == 1) {
                 if (uniform_keys) {
 #pragma unroll
                     for (int i = 0; i < 16; ++i) {
@@ -678,7 +720,7 @@ __global__ __launch_bounds__(DQ_THREADS, 2) void bwd_dq_kernel(const AttnParams 
         const int kt = entry >> 2, rows = Sk - kt * DQ_KT;
         stK.load_ragged(kbase + kt * k_ts, sK[0], rows, tid);
         stV.load_ragged(vbase + kt * v_ts, sV[0], rows, tid);
-        if (tid < DQ_KT) {
+        if (!DENSE && tid < DQ_KT) {
             sKbf[0][tid] = (tid < rows) ? bfrow[kt * DQ_KT + tid] : 0;
             if (IDX) sKpos[0][tid] = (tid < rows) ? p.posk[kt * DQ_KT + tid] : 0;
         }
@@ -723,19 +765,23 @@ static int launch_pre_t(const AttnParams& p, hipStream_t stream) {
 template <typename T, int D>
 static int launch_dkdv_t(const AttnParams& p, hipStream_t stream) {
     const int blocks = p.num_kt * p.B * p.Hkv;  // one workgroup per 128-key tile
-    if (p.posq != nullptr)
-        hipLaunchKernelGGL((bwd_dkdv_kernel<T, D, true>), dim3(blocks), dim3(DKDV_THREADS), 0, stream, p);
+    if (p.mask_mode == MASK_INDEXED)
+        hipLaunchKernelGGL((bwd_dkdv_kernel<T, D, MASK_INDEXED>), dim3(blocks), dim3(DKDV_THREADS), 0, stream, p);
+    else if (p.mask_mode == MASK_DENSE)
+        hipLaunchKernelGGL((bwd_dkdv_kernel<T, D, MASK_DENSE>), dim3(blocks), dim3(DKDV_THREADS), 0, stream, p);
     else
-        hipLaunchKernelGGL((bwd_dkdv_kernel<T, D, false>), dim3(blocks), dim3(DKDV_THREADS), 0, stream, p);
+        hipLaunchKernelGGL((bwd_dkdv_kernel<T, D, MASK_BITFIELD>), dim3(blocks), dim3(DKDV_THREADS), 0, stream, p);
     return (int)hipGetLastError();
 }
 template <typename T, int D>
 static int launch_dq_t(const AttnParams& p, hipStream_t stream) {
     const int blocks = p.num_m * p.B * p.Hq;
-    if (p.posq != nullptr)
-        hipLaunchKernelGGL((bwd_dq_kernel<T, D, true>), dim3(blocks), dim3(DQ_THREADS), 0, stream, p);
+    if (p.mask_mode == MASK_INDEXED)
+        hipLaunchKernelGGL((bwd_dq_kernel<T, D, MASK_INDEXED>), dim3(blocks), dim3(DQ_THREADS), 0, stream, p);
+    else if (p.mask_mode == MASK_DENSE)
+        hipLaunchKernelGGL((bwd_dq_kernel<T, D, MASK_DENSE>), dim3(blocks), dim3(DQ_THREADS), 0, stream, p);
     else
-        hipLaunchKernelGGL((bwd_dq_kernel<T, D, false>), dim3(blocks), dim3(DQ_THREADS), 0, stream, p);
+        hipLaunchKernelGGL((bwd_dq_kernel<T, D, MASK_BITFIELD>), dim3(blocks), dim3(DQ_THREADS), 0, stream, p);
     return (int)hipGetLastError();
 }
 

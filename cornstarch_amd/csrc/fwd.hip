@@ -26,10 +26,12 @@ namespace bam {
 constexpr int FWD_KT = 64;
 constexpr int FWD_THREADS = 256;
 
-// IDX: index-tensor attention -- query rows and keys carry explicit global positions (p.posq, p.posk) and
-// the bitfield arrays are already gathered per local row / key (context-parallel shards, reference
-// bitfield_attention.py:71-81).
-template <typename T, int D, bool IDX>
+// MODE (MASK_*): where allow / deny comes from.  MASK_INDEXED: query rows and keys carry explicit global
+// positions (p.posq, p.posk) and the bitfield arrays are already gathered per local row / key
+// (context-parallel shards, reference bitfield_attention.py:71-81).  MASK_DENSE: a materialized bool mask
+// (the reference's sibling kernel, cornstarch/kernel/attention.py:184-232), read from global memory in the
+// tiles the flags call partial.
+template <typename T, int D, int MODE>
 __global__ __launch_bounds__(FWD_THREADS, 2) void fwd_kernel(const AttnParams p) {
     constexpr int NCH = D / 8, KK = D / 16, DB = D / 32;
     __shared__ u32x4 sK[2][FWD_KT * NCH];
@@ -41,6 +43,7 @@ __global__ __launch_bounds__(FWD_THREADS, 2) void fwd_kernel(const AttnParams p)
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int hi = lane >> 5, l32 = lane & 31, half16 = (lane >> 4) & 1;
+    constexpr bool IDX = MODE == MASK_INDEXED, DENSE = MODE == MASK_DENSE;
     const int Sq = p.Sq, Sk = p.Sk;
     const int G = p.Hq / p.Hkv;
 
@@ -69,7 +72,7 @@ __global__ __launch_bounds__(FWD_THREADS, 2) void fwd_kernel(const AttnParams p)
             qreg[kk] = z;
         }
     }
-    const int64_t qf = qvalid ? p.bfq[(int64_t)b * p.bfq_sb + qrow] : 0;
+    const int64_t qf = (!DENSE && qvalid) ? p.bfq[(int64_t)b * p.bfq_sb + qrow] : 0;
     const QueryBits qb = make_query_bits(qf, (IDX && qvalid) ? p.posq[qrow] : qrow);
 
     f32x16 o[DB];
@@ -98,7 +101,7 @@ __global__ __launch_bounds__(FWD_THREADS, 2) void fwd_kernel(const AttnParams p)
     typedef TileStage<D, FWD_KT, FWD_THREADS> Stage;
     constexpr int CPT = Stage::CPT;
     // copy instructions per wave and tile: K, V, the key bitfields and (IDX) the key positions
-    constexpr int NLOADS = 2 * CPT + 1 + (IDX ? 1 : 0);
+    constexpr int NLOADS = 2 * CPT + (DENSE ? 0 : 1) + (IDX ? 1 : 0);
     static_assert(NLOADS <= 2 * KK, "one copy per MFMA of the S phase");
     Stage stK, stV;
     stK.setup(2 * p.k.ss, tid);
@@ -113,7 +116,7 @@ __global__ __launch_bounds__(FWD_THREADS, 2) void fwd_kernel(const AttnParams p)
             stK.issue(j, kbase + kt * k_ts, ldsK + buf * TILE_BYTES);
         else if (j < 2 * CPT)
             stV.issue(j - CPT, vbase + kt * v_ts, ldsV + buf * TILE_BYTES);
-        else if (j == 2 * CPT)
+        else if (j == 2 * CPT)  // (never reached with a dense mask: NLOADS == 2 * CPT)
             dma_b32(bfrow + kt * FWD_KT, (unsigned)((wave & 1) * 256 + lane * 4), ldsB + buf * BITS_BYTES + (wave & 1) * 256u);
         else  // 64 positions; every wave writes the same values
             dma_b32(p.posk + kt * FWD_KT, (unsigned)(lane * 4), ldsP + buf * (FWD_KT * 4u));
@@ -148,7 +151,37 @@ __global__ __launch_bounds__(FWD_THREADS, 2) void fwd_kernel(const AttnParams p)
         }
 
         // ---- bitfield rule in registers (partial tiles only) ------------------------------
-        if (cls == 1) {
+        if (DENSE) {
+            if (cls == 1) {
+                // mask bytes of this lane's query row: 4 consecutive keys per C-fragment group
+                const int kt0 = kt * FWD_KT;
+                const uint8_t* mrow = p.mask + ((int64_t)b * Sq + (qvalid ? qrow : 0)) * Sk + kt0;
+                const bool dwords = (Sk & 3) == 0;  // rows start 4-byte aligned
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                    for (int grp = 0; grp < 4; ++grp) {
+                        const int koff = 32 * kb + 8 * grp + 4 * hi;
+                        unsigned m4 = 0;
+                        if (p.mask == nullptr) {
+                            m4 = 0x01010101u;
+                        } else if (qvalid) {
+                            if (dwords) {
+                                if (kt0 + koff < Sk) m4 = *(const unsigned*)(mrow + koff);
+                            } else {
+#pragma unroll
+                                for (int x = 0; x < 4; ++x)
+                                    if (kt0 + koff + x < Sk) m4 |= (unsigned)mrow[koff + x] << (8 * x);
+                            }
+                        }
+#pragma unroll
+                        for (int x = 0; x < 4; ++x) {
+                            const bool a = ((m4 >> (8 * x)) & 0xFFu) != 0 && kt0 + koff + x < Sk;
+                            s[kb][4 * grp + x] = a ? s[kb][4 * grp + x] : -INFINITY;
+                        }
+                    }
+            }
+        } else if (cls == 1) {
             // Most partial tiles are partial only through causality: all 64 keys carry the same bitfield (and,
             // with index tensors, sit at consecutive positions).  Then the bit test is a per-query constant and
             // the rule reduces to one position compare.
@@ -282,7 +315,7 @@ __global__ __launch_bounds__(FWD_THREADS, 2) void fwd_kernel(const AttnParams p)
         const int kt = entry >> 2, rows = Sk - kt * FWD_KT;
         stK.load_ragged(kbase + kt * k_ts, sK[0], rows, tid);
         stV.load_ragged(vbase + kt * v_ts, sV[0], rows, tid);
-        if (tid < FWD_KT) {
+        if (!DENSE && tid < FWD_KT) {
             sKbf[0][tid] = (tid < rows) ? bfrow[kt * FWD_KT + tid] : 0;
             if (IDX) sKpos[0][tid] = (tid < rows) ? p.posk[kt * FWD_KT + tid] : 0;
         }
@@ -313,10 +346,12 @@ __global__ __launch_bounds__(FWD_THREADS, 2) void fwd_kernel(const AttnParams p)
 template <typename T, int D>
 static int launch_fwd_t(const AttnParams& p, hipStream_t stream) {
     const int blocks = p.num_m * p.B * p.Hq;
-    if (p.posq != nullptr)
-        hipLaunchKernelGGL((fwd_kernel<T, D, true>), dim3(blocks), dim3(FWD_THREADS), 0, stream, p);
+    if (p.mask_mode == MASK_INDEXED)
+        hipLaunchKernelGGL((fwd_kernel<T, D, MASK_INDEXED>), dim3(blocks), dim3(FWD_THREADS), 0, stream, p);
+    else if (p.mask_mode == MASK_DENSE)
+        hipLaunchKernelGGL((fwd_kernel<T, D, MASK_DENSE>), dim3(blocks), dim3(FWD_THREADS), 0, stream, p);
     else
-        hipLaunchKernelGGL((fwd_kernel<T, D, false>), dim3(blocks), dim3(FWD_THREADS), 0, stream, p);
+        hipLaunchKernelGGL((fwd_kernel<T, D, MASK_BITFIELD>), dim3(blocks), dim3(FWD_THREADS), 0, stream, p);
     return (int)hipGetLastError();
 }
 

@@ -86,6 +86,68 @@ int launch_gather_bitfields(const int64_t* bf, int64_t bf_stride_b, int L, const
     return (int)hipGetLastError();
 }
 
+// Tile flags of a materialized bool mask (B, Sq, Sk), one byte per pair: the same 0 / 1 / 2 classification
+// over 128 x 32 tiles that the bitfield path uses, so that the attention kernels skip empty tiles and
+// read the mask only in partial ones.  (The reference's materialized-mask kernel decides per tile, inside
+// the attention loop, whether anything is unmasked: cornstarch/kernel/attention.py:188-200.)
+// One workgroup = one row block x 8 column tiles; thread = one column, 128 rows, coalesced byte reads.
+__global__ __launch_bounds__(256) void mask_tile_flags_kernel(const uint8_t* __restrict__ mask, int8_t* __restrict__ flags,
+                                                              int64_t flags_stride_b, int64_t flags_stride_m, int Sq,
+                                                              int Sk, int num_n) {
+    const int b = blockIdx.z, m = blockIdx.y, tid = threadIdx.x;
+    const int col = blockIdx.x * 256 + tid;
+    const int r0 = m * BLOCK_M, r1 = min(r0 + BLOCK_M, Sq);
+    int count = 0;
+    if (col < Sk) {
+        const uint8_t* pcol = mask + (int64_t)b * Sq * Sk + col;
+        for (int r = r0; r < r1; ++r) count += pcol[(int64_t)r * Sk] != 0;
+    }
+#pragma unroll
+    for (int off = 16; off > 0; off >>= 1) count += __shfl_xor(count, off);  // over the 32 columns of a tile
+    const int n = blockIdx.x * 8 + (tid >> 5);
+    if ((tid & 31) == 0 && n < num_n) {
+        const int cells = (r1 - r0) * min(BLOCK_N, Sk - n * BLOCK_N);
+        flags[(int64_t)b * flags_stride_b + (int64_t)m * flags_stride_m + n] = count == 0 ? 0 : count == cells ? 2 : 1;
+    }
+}
+
+int launch_mask_tile_flags(const uint8_t* mask, int8_t* flags, int64_t flags_stride_b, int64_t flags_stride_m, int B,
+                           int Sq, int Sk, hipStream_t stream) {
+    const int num_m = (Sq + BLOCK_M - 1) / BLOCK_M, num_n = (Sk + BLOCK_N - 1) / BLOCK_N;
+    dim3 grid((num_n + 7) / 8, num_m, B);
+    hipLaunchKernelGGL(mask_tile_flags_kernel, grid, dim3(256), 0, stream, mask, flags, flags_stride_b, flags_stride_m,
+                       Sq, Sk, num_n);
+    return (int)hipGetLastError();
+}
+
+// Work per 128-row block for the makespan-minimizing sequence split: the number of non-empty 128x32
+// tiles of each row block, summed over the batch -- `torch.sum(compressed_mask > 0, dim=(0, 2))` of
+// the reference (shardformer/layers/utils.py:161-166), computed where the flags already are instead
+// of after a copy to the host.  One workgroup per row block, no atomics.
+__global__ __launch_bounds__(256) void flag_row_workloads_kernel(const int8_t* __restrict__ flags, int64_t flags_stride_b,
+                                                                 int64_t flags_stride_m, int B, int num_n,
+                                                                 int* __restrict__ out) {
+    __shared__ int partial[4];
+    const int m = blockIdx.x, tid = threadIdx.x;
+    int count = 0;
+    for (int b = 0; b < B; ++b) {
+        const int8_t* row = flags + (int64_t)b * flags_stride_b + (int64_t)m * flags_stride_m;
+        for (int n = tid; n < num_n; n += 256) count += row[n] > 0;
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) count += __shfl_xor(count, off);
+    if ((tid & 63) == 0) partial[tid >> 6] = count;
+    __syncthreads();
+    if (tid == 0) out[m] = partial[0] + partial[1] + partial[2] + partial[3];
+}
+
+int launch_flag_row_workloads(const int8_t* flags, int64_t flags_stride_b, int64_t flags_stride_m, int B, int num_m,
+                              int num_n, int* out, hipStream_t stream) {
+    hipLaunchKernelGGL(flag_row_workloads_kernel, dim3(num_m), dim3(256), 0, stream, flags, flags_stride_b,
+                       flags_stride_m, B, num_n, out);
+    return (int)hipGetLastError();
+}
+
 int launch_tile_flags(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int64_t flags_stride_b,
                       int64_t flags_stride_m, int B, int S, hipStream_t stream) {
     const int num_m = (S + BLOCK_M - 1) / BLOCK_M, num_n = (S + BLOCK_N - 1) / BLOCK_N;

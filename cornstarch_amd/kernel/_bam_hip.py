@@ -14,7 +14,7 @@ LIB_PATH = os.path.join(_PKG_DIR, "libbam_hip.so")
 BAM_DTYPE_F16 = 0
 BAM_DTYPE_BF16 = 1
 BAM_MAX_SEQLEN = 131072
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 _i64 = ctypes.c_int64
 _int = ctypes.c_int
@@ -47,6 +47,11 @@ SIGNATURES = {
     "bam_bwd": [_ptr] * 11 + [_i64] * 24 + [_int] * 5 + [_f32, _int, _int, _ptr],
     "bam_bwd_dkdv": [_ptr] * 10 + [_i64] * 21 + [_int] * 5 + [_f32, _int, _int, _ptr],
     "bam_bwd_dq": [_ptr] * 9 + [_i64] * 18 + [_int] * 5 + [_f32, _int, _int, _ptr],
+    "bam_mask_tile_flags": [_ptr, _ptr, _i64, _i64, _int, _int, _int, _ptr],
+    "bam_fwd_masked": [_ptr] * 7 + [_i64] * 14 + [_int] * 6 + [_f32, _int, _ptr],
+    "bam_bwd_dkdv_masked": [_ptr] * 10 + [_i64] * 20 + [_int] * 6 + [_f32, _int, _int, _ptr],
+    "bam_bwd_dq_masked": [_ptr] * 9 + [_i64] * 17 + [_int] * 6 + [_f32, _int, _int, _ptr],
+    "bam_flag_row_workloads": [_ptr, _i64, _i64, _int, _int, _int, _ptr, _ptr],
     "bam_gather_bitfields": [_ptr, _i64, _int, _ptr, _int, _ptr, _i64, _ptr, _int, _ptr],
     "bam_fwd_indexed": [_ptr] * 5 + [_view, _ptr] + [_i64] * 14 + [_int] * 4 + [_f32, _int, _ptr],
     "bam_bwd_dkdv_indexed": [_ptr] * 8 + [_view, _ptr] + [_i64] * 20 + [_int] * 4 + [_f32, _int, _int, _ptr],

@@ -120,6 +120,23 @@ class BitfieldUtils:
         cls._cache_key = key
         return out
 
+    @classmethod
+    def nonempty_tiles_per_row_block(cls, compressed_mask: torch.Tensor) -> torch.Tensor:
+        """int64 (ceil(S/128),): non-empty 128x32 tiles of each row block, summed over the batch --
+        ``torch.sum(compressed_mask > 0, dim=(0, 2))``, the per-block workload the makespan-minimizing
+        sequence split sorts by (reference shardformer/layers/utils.py:161-171), computed on the GPU so that
+        only this small vector has to travel to the host."""
+        assert compressed_mask.is_cuda and compressed_mask.dtype == torch.int8 and compressed_mask.dim() == 3
+        flags = compressed_mask if compressed_mask.stride(-1) == 1 else compressed_mask.contiguous()
+        batch_size, num_m, num_n = flags.shape
+        out = torch.empty((num_m,), dtype=torch.int32, device=flags.device)
+        with torch.cuda.device(flags.device):
+            _bam_hip.call(
+                "bam_flag_row_workloads", flags.data_ptr(), flags.stride(0), flags.stride(1), batch_size, num_m, num_n,
+                out.data_ptr(), _stream_ptr(flags.device),
+            )
+        return out.to(torch.int64)
+
 
 def _check_unsupported(bias):
     if bias is not None:

@@ -81,6 +81,15 @@ int bam_tile_flags(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int64_
 int bam_materialize_mask(const int64_t* bf, int64_t bf_stride_b, uint8_t* out, int B, int S, void* stream);
 
 /*
+ * Non-empty tiles per 128-row block, summed over the batch: out[m] = sum_{b,n} (flags[b,m,n] > 0), int32 (num_m).
+ * This is the input of the makespan-minimizing sequence split, which the reference computes on the host
+ * after copying the flags there (`torch.sum(compressed_mask > 0, dim=(0, 2))`,
+ * shardformer/layers/utils.py:161-166).
+ */
+int bam_flag_row_workloads(const int8_t* flags, int64_t flags_stride_b, int64_t flags_stride_m, int B, int num_m,
+                           int num_n, int32_t* out, void* stream);
+
+/*
  * Gather for index-tensor attention: out_bits[b][i] = bf[b][idx[i]], or 0 where idx[i] is outside
  * [0, L) (the `other=0` of the reference's masked loads, bitfield_attention.py:86-87), and
  * out_pos[i] = idx[i] as int32.  bf: int64 (B, L); idx: int64 (n); out_bits: int64 (B, n) with row
@@ -195,6 +204,45 @@ int bam_bwd_dq_indexed(const void* q, const void* k, const void* v, const void* 
                        int64_t dq_stride_b, int64_t dq_stride_s, int64_t dq_stride_h, int64_t flags_stride_b,
                        int64_t flags_stride_m, int B, int Hq, int Hkv, int D, float scale, int dtype,
                        int accumulate, void* stream);
+
+/*
+ * Materialized-mask attention: the sibling path of the reference,
+ * cornstarch/kernel/attention.py (`flash_attn_func(q, k, v, bias, mask)`, `_flash_attn_forward` :855-949,
+ * `_flash_attn_backward` :952-1069, forward kernel :77-345, backward kernels :438-852), served by the same
+ * forward / dK,dV / dQ kernels with the allow decision read from a bool mask instead of derived from bitfields.
+ *   mask: uint8 / bool (B, Sq, Sk), contiguous, nonzero = attend; NULL = every pair allowed (then flags
+ *         must be 2 everywhere).
+ *   flags: int8 (B, ceil(Sq/128), ceil(Sk/32)) from bam_mask_tile_flags (0 empty, 1 partial, 2 full).
+ * q is (B, Sq, Hq, D), k / v are (B, Sk, Hkv, D) (the reference requires Hkv == Hq, :867-868; grouped kv heads
+ * work as in the bitfield path), lse / delta are (B, Hq, ceil(Sq/128)*128).
+ */
+int bam_mask_tile_flags(const uint8_t* mask, int8_t* flags, int64_t flags_stride_b, int64_t flags_stride_m, int B,
+                        int Sq, int Sk, void* stream);
+
+int bam_fwd_masked(const void* q, const void* k, const void* v, void* o, float* lse, const uint8_t* mask,
+                   const int8_t* flags, int64_t q_stride_b, int64_t q_stride_s, int64_t q_stride_h,
+                   int64_t k_stride_b, int64_t k_stride_s, int64_t k_stride_h, int64_t v_stride_b,
+                   int64_t v_stride_s, int64_t v_stride_h, int64_t o_stride_b, int64_t o_stride_s,
+                   int64_t o_stride_h, int64_t flags_stride_b, int64_t flags_stride_m, int B, int Sq, int Sk, int Hq,
+                   int Hkv, int D, float scale, int dtype, void* stream);
+
+int bam_bwd_dkdv_masked(const void* q, const void* k, const void* v, const void* dout, const float* lse,
+                        const float* delta, void* dk, void* dv, const uint8_t* mask, const int8_t* flags,
+                        int64_t q_stride_b, int64_t q_stride_s, int64_t q_stride_h, int64_t k_stride_b,
+                        int64_t k_stride_s, int64_t k_stride_h, int64_t v_stride_b, int64_t v_stride_s,
+                        int64_t v_stride_h, int64_t do_stride_b, int64_t do_stride_s, int64_t do_stride_h,
+                        int64_t dk_stride_b, int64_t dk_stride_s, int64_t dk_stride_h, int64_t dv_stride_b,
+                        int64_t dv_stride_s, int64_t dv_stride_h, int64_t flags_stride_b, int64_t flags_stride_m,
+                        int B, int Sq, int Sk, int Hq, int Hkv, int D, float scale, int dtype, int accumulate,
+                        void* stream);
+
+int bam_bwd_dq_masked(const void* q, const void* k, const void* v, const void* dout, const float* lse,
+                      const float* delta, void* dq, const uint8_t* mask, const int8_t* flags, int64_t q_stride_b,
+                      int64_t q_stride_s, int64_t q_stride_h, int64_t k_stride_b, int64_t k_stride_s,
+                      int64_t k_stride_h, int64_t v_stride_b, int64_t v_stride_s, int64_t v_stride_h,
+                      int64_t do_stride_b, int64_t do_stride_s, int64_t do_stride_h, int64_t dq_stride_b,
+                      int64_t dq_stride_s, int64_t dq_stride_h, int64_t flags_stride_b, int64_t flags_stride_m, int B,
+                      int Sq, int Sk, int Hq, int Hkv, int D, float scale, int dtype, int accumulate, void* stream);
 
 #ifdef __cplusplus
 }

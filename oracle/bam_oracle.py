@@ -30,6 +30,10 @@ What pins each function (the pins live in ``tests/test_oracle.py``):
   ``idx_q`` (what the reference's context-parallel test asserts,
   ``tests/test_shardformer/test_context_parallel.py:311-376``); for block-aligned index sets the
   flags equal the reference's gather of the global flags (``shardformer/layers/utils.py:331-353``).
+* ``masked_attention_forward`` / ``masked_attention_backward`` (materialized bool mask, the
+  reference's ``flash_attn_func``) -- library SDPA with the same ``attn_mask`` and autograd through it,
+  which is what the reference's test compares against (``tests/test_kernel/test_attention.py``);
+  ``mask_tile_flags`` -- brute-force classification of random masks.
 * ``create_bitfield_attention_mask`` -- golden vectors of
   ``tests/test_models/test_multimodal_merge_outputs.py:94-110``.
 
@@ -256,6 +260,41 @@ def attention_backward(q, k, v, bitfield, do, softmax_scale=None, row_chunk=1024
             dk[b] += gk
             dv[b] += gv
     return dq, dk, dv
+
+
+def masked_attention_forward(q, k, v, mask, softmax_scale=None, dtype=torch.float32):
+    """Attention with a materialized bool mask (B, Sq, Sk) (None: attend everywhere), the contract of
+    the reference's ``flash_attn_func`` (cornstarch/kernel/attention.py:184-232: pairs whose mask
+    byte is False get -inf before the softmax) -> (o (B,Sq,Hq,D), lse (B,Hq,Sq))."""
+    B, Sq, Hq, D = q.shape
+    Sk = k.shape[1]
+    scale = softmax_scale or 1.0 / math.sqrt(D)
+    q, k, v = q.to(dtype), k.to(dtype), v.to(dtype)
+    o = torch.empty((B, Sq, Hq, D), dtype=dtype, device=q.device)
+    lse = torch.empty((B, Hq, Sq), dtype=dtype, device=q.device)
+    for b in range(B):
+        allow = mask[b] if mask is not None else torch.ones((Sq, Sk), dtype=torch.bool, device=q.device)
+        o[b], lse[b] = _chunk_forward(q[b], k[b], v[b], allow, scale)
+    return o, lse
+
+
+def masked_attention_backward(q, k, v, mask, do, softmax_scale=None, dtype=torch.float32):
+    """dq, dk, dv of sum(o * do) for ``masked_attention_forward`` by autograd."""
+    q, k, v, do = (t.to(dtype) for t in (q, k, v, do))
+    qr, kr, vr = (t.detach().requires_grad_(True) for t in (q, k, v))
+    o, _ = masked_attention_forward(qr, kr, vr, mask, softmax_scale, dtype)
+    return torch.autograd.grad(o, (qr, kr, vr), do)
+
+
+def mask_tile_flags(mask: torch.Tensor) -> torch.Tensor:
+    """int8 (B, ceil(Sq/128), ceil(Sk/32)) classification of a bool mask (B, Sq, Sk): 0 empty,
+    2 every in-range cell set, 1 otherwise."""
+    B, Sq, Sk = mask.shape
+    nm, nn = -(-Sq // BLOCK_M), -(-Sk // BLOCK_N)
+    padded = F.pad(mask, (0, nn * BLOCK_N - Sk, 0, nm * BLOCK_M - Sq))
+    cnt = padded.view(B, nm, BLOCK_M, nn, BLOCK_N).sum(dim=(2, 4))
+    cells = F.pad(torch.ones_like(mask), (0, nn * BLOCK_N - Sk, 0, nm * BLOCK_M - Sq)).view(B, nm, BLOCK_M, nn, BLOCK_N).sum(dim=(2, 4))
+    return torch.where(cnt == 0, 0, torch.where(cnt == cells, 2, 1)).to(torch.int8)
 
 
 def delta(o, do):

@@ -1,0 +1,104 @@
+"""Materialized-mask attention (``flash_attn_func(q, k, v, mask=...)``) on an MI355X, through the C ABI.
+
+The grid follows the reference's test of this entry point (tests/test_kernel/test_attention.py:10-111:
+fp16 / bf16, head dims 32 / 64 / 128, query / key lengths incl. 128x1024 and 1024x128, the tril +
+modality-squares mask, batch 1, 12 heads).  Checked against the fp32 oracle: flags bit exact, forward within
+1e-2 + 1e-2 |x|, gradients within relative L2 5e-2.
+"""
+
+import pytest
+import torch
+
+from cornstarch_amd.kernel import attention as A
+from cornstarch_amd.kernel import interface
+from oracle import bam_oracle as O
+from tests.helpers import rel_l2
+
+pytestmark = pytest.mark.gpu
+
+GRAD_REL_L2 = 5e-2
+
+
+def dev():
+    return torch.device("cuda:0")
+
+
+def reference_mask(B, Sq, Sk):
+    mask = torch.tril(torch.ones(B, Sq, Sk, dtype=torch.bool))
+    mask[:, 12:24, :] = False
+    mask[:, 12:24, 12:24] = True
+    mask[:, 36:56, :] = False
+    mask[:, 36:56, 36:56] = True
+    return mask
+
+
+def inputs(B, Sq, Sk, Hq, Hkv, D, dtype, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    q = (torch.randn(B, Sq, Hq, D, generator=g) * 0.5).to(dtype)
+    k = (torch.randn(B, Sk, Hkv, D, generator=g) * 0.5).to(dtype)
+    v = (torch.randn(B, Sk, Hkv, D, generator=g) * 0.5).to(dtype)
+    do = torch.randn(B, Sq, Hq, D, generator=g).to(dtype)
+    return q, k, v, do
+
+
+def check(q, k, v, do, mask, scale=None):
+    d = dev()
+    qg, kg, vg = (t.to(d).requires_grad_(True) for t in (q, k, v))
+    mg = mask.to(d) if mask is not None else None
+    out = A.flash_attn_func(qg, kg, vg, mask=mg, softmax_scale=scale)
+    gq, gk, gv = torch.autograd.grad(out, (qg, kg, vg), do.to(d))
+    torch.cuda.synchronize()
+    o_ref, _ = O.masked_attention_forward(q, k, v, mask, softmax_scale=scale)
+    assert out.dtype == q.dtype and out.shape == q.shape
+    torch.testing.assert_close(out.float().cpu(), o_ref, atol=1e-2, rtol=1e-2)
+    wq, wk, wv = O.masked_attention_backward(q, k, v, mask, do, softmax_scale=scale)
+    for got, want in ((gq, wq), (gk, wk), (gv, wv)):
+        assert got.dtype == q.dtype
+        assert rel_l2(got.float().cpu(), want) <= GRAD_REL_L2
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["fp16", "bf16"])
+@pytest.mark.parametrize("head_dim", [32, 64, 128])
+@pytest.mark.parametrize(
+    "seqlen", [(128, 128), (128, 1024), (1024, 128), (1024, 1024), (57, 57), (144, 144), (283, 283)],
+    ids=["128x128", "128x1024", "1024x128", "1024x1024", "57x57", "144x144", "283x283"],
+)
+def test_reference_grid(dtype, head_dim, seqlen):
+    Sq, Sk = seqlen
+    q, k, v, do = inputs(1, Sq, Sk, 12, 12, head_dim, dtype)
+    check(q, k, v, do, reference_mask(1, Sq, Sk))
+
+
+@pytest.mark.parametrize("Sq,Sk", [(300, 170), (64, 515), (1, 33)])
+def test_mask_flags_bit_exact_and_random_masks_with_dead_rows(Sq, Sk):
+    g = torch.Generator().manual_seed(Sq)
+    mask = torch.rand(2, Sq, Sk, generator=g) < 0.4
+    mask[:, : Sq // 2, : Sk // 3] = True
+    mask[:, Sq // 2 :, Sk // 2 :] = False
+    mask[:, -1, :] = False  # a row that sees nothing: o = 0, gradients 0
+    flags = A.mask_tile_flags(mask.to(dev()), 2, Sq, Sk, dev())
+    assert torch.equal(flags.cpu(), O.mask_tile_flags(mask))
+    q, k, v, do = inputs(2, Sq, Sk, 4, 2, 64, torch.bfloat16, seed=Sk)  # grouped kv heads as well
+    check(q, k, v, do, mask)
+
+
+def test_no_mask_head_dim_40_custom_scale():
+    q, k, v, do = inputs(2, 200, 333, 4, 4, 40, torch.float16, seed=8)
+    check(q, k, v, do, None, scale=0.2)
+
+
+def test_private_entry_points_and_hf_adapter():
+    d = dev()
+    q, k, v, do = (t.to(d) for t in inputs(1, 144, 144, 4, 4, 64, torch.bfloat16, seed=2))
+    mask = reference_mask(1, 144, 144).to(d)
+    o, lse, scale = A._flash_attn_forward(q, k, v, mask=mask)
+    assert lse.shape == (1, 4, 256) and lse.dtype == torch.float32 and scale == 64 ** -0.5
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    A._flash_attn_backward(do, q, k, v, o, lse, dq, dk, dv, mask=mask, softmax_scale=scale)
+    want = O.masked_attention_backward(q.cpu(), k.cpu(), v.cpu(), mask.cpu(), do.cpu())
+    for got, w in zip((dq, dk, dv), want):
+        assert rel_l2(got.float().cpu(), w) <= GRAD_REL_L2
+    out, none = interface.cornstarch_attention_forward(None, q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), mask)
+    assert none is None and torch.equal(out, o)
+    with pytest.raises(NotImplementedError):
+        A.flash_attn_func(q, k, v, bias=torch.zeros(1, 4, 1, 144, device=d))

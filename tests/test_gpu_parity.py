@@ -103,6 +103,20 @@ def test_flags_rowblock_workloads_of_the_context_parallel_test(S):
     assert (dense == 2).all()
 
 
+@pytest.mark.parametrize("S", [57, 335, 1024, 3712])
+def test_row_block_workloads_for_the_makespan_split(S):
+    # torch.sum(compressed_mask > 0, dim=(0, 2)) of shardformer/layers/utils.py:161-166; for an all-text
+    # sequence block m sees 4 (m + 1) tiles per sequence (test_context_parallel.py:258-272)
+    causal = torch.full((3, S), (1 << 62) | 1, dtype=torch.int64, device=dev())
+    got = BA.BitfieldUtils.nonempty_tiles_per_row_block(flags_of(causal))
+    nm, nn = -(-S // 128), -(-S // 32)
+    want = torch.tensor([3 * min(4 * (m + 1), nn) for m in range(nm)])
+    assert got.dtype == torch.int64 and torch.equal(got.cpu(), want)
+    bf = random_bitfield(2, S, seed=S).to(dev())
+    flags = flags_of(bf)
+    assert torch.equal(BA.BitfieldUtils.nonempty_tiles_per_row_block(flags), torch.sum(flags > 0, dim=(0, 2)))
+
+
 def test_flags_of_a_strided_bitfield_row_view():
     base = random_bitfield(4, 600, seed=11)
     big = torch.zeros((4, 1000), dtype=torch.int64)

@@ -273,3 +273,63 @@ def test_indexed_flags_equal_the_reference_gather_of_global_flags_for_aligned_bl
     for idx_q in ranks:
         want = glob[:, idx_q[::128] // 128][:, :, cols]
         assert torch.equal(O.tile_flags_indexed(bf, idx_q, idx_k), want)
+
+
+# ------------------------------------------------------------------ materialized bool mask (flash_attn_func)
+def _reference_dense_mask(B, Sq, Sk):
+    """mask of the reference's test (tests/test_kernel/test_attention.py:80-88)."""
+    mask = torch.tril(torch.ones(B, Sq, Sk, dtype=torch.bool))
+    mask[:, 12:24, :] = False
+    mask[:, 12:24, 12:24] = True
+    mask[:, 36:56, :] = False
+    mask[:, 36:56, 36:56] = True
+    return mask
+
+
+@pytest.mark.parametrize("Sq,Sk", [(57, 57), (128, 300), (283, 144)])
+def test_dense_mask_attention_against_library_sdpa(Sq, Sk):
+    # ground truth of the reference's test: SDPA with attn_mask = mask (test_attention.py:93-104)
+    B, H, D = 2, 3, 16
+    g = torch.Generator().manual_seed(3)
+    q = torch.randn(B, Sq, H, D, generator=g, dtype=torch.float64) * 0.5
+    k = torch.randn(B, Sk, H, D, generator=g, dtype=torch.float64) * 0.5
+    v = torch.randn(B, Sk, H, D, generator=g, dtype=torch.float64) * 0.5
+    do = torch.randn(B, Sq, H, D, generator=g, dtype=torch.float64)
+    mask = _reference_dense_mask(B, Sq, Sk)
+    live = mask.any(-1)  # rows of the square blocks that fall outside Sk see nothing: SDPA gives NaN there
+    qr, kr, vr = (t.clone().requires_grad_(True) for t in (q, k, v))
+    ref = F.scaled_dot_product_attention(
+        qr.transpose(1, 2), kr.transpose(1, 2), vr.transpose(1, 2), attn_mask=mask.unsqueeze(1)
+    ).transpose(1, 2)
+    ref = torch.where(live[:, :, None, None], ref, torch.zeros_like(ref))
+    o, lse = O.masked_attention_forward(q, k, v, mask, dtype=torch.float64)
+    assert torch.allclose(o, ref, atol=1e-10, rtol=0)
+    s = torch.einsum("bihd,bjhd->bhij", q, k) / math.sqrt(D)
+    want_lse = torch.logsumexp(s.masked_fill(~mask.unsqueeze(1), float("-inf")), dim=-1)
+    assert torch.equal(torch.isfinite(lse), torch.isfinite(want_lse))
+    assert torch.allclose(lse[torch.isfinite(lse)], want_lse[torch.isfinite(want_lse)], atol=1e-10, rtol=0)
+    wq, wk, wv = torch.autograd.grad(ref, (qr, kr, vr), do)
+    dq, dk, dv = O.masked_attention_backward(q, k, v, mask, do, dtype=torch.float64)
+    for got, want in ((dq, wq), (dk, wk), (dv, wv)):
+        assert torch.allclose(got, want, atol=1e-10, rtol=0)
+    # no mask at all == plain softmax attention
+    o2, _ = O.masked_attention_forward(q, k, v, None, dtype=torch.float64)
+    ref2 = F.scaled_dot_product_attention(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2)).transpose(1, 2)
+    assert torch.allclose(o2, ref2, atol=1e-10, rtol=0)
+
+
+def test_dense_mask_tile_flags_against_loops():
+    g = torch.Generator().manual_seed(4)
+    mask = torch.rand(2, 300, 170, generator=g) < 0.5
+    mask[:, :128, :64] = True  # full tiles
+    mask[:, 128:256, 32:96] = False  # empty tiles
+    mask[:, 256:, 160:] = True  # the ragged corner tile, full
+    got = O.mask_tile_flags(mask)
+    assert got.shape == (2, 3, 6)
+    for b in range(2):
+        for m in range(3):
+            for n in range(6):
+                t = mask[b, m * 128 : (m + 1) * 128, n * 32 : (n + 1) * 32]
+                want = 0 if not t.any() else 2 if t.all() else 1
+                assert got[b, m, n] == want
+    assert got[0, 0, 0] == 2 and got[0, 1, 1] == 0 and got[0, 2, 5] == 2
