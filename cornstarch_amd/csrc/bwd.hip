@@ -471,7 +471,7 @@ constexpr int DQ_KT = 64;
 constexpr int DQ_THREADS = 256;
 
 template <typename T, int D, int MODE>
-__global__ __launch_bounds__(DQ_THREADS, 2) void bwd_dq_kernel(const AttnParams p) {
+__global__ __launch_bounds__(DQ_THREADS, D == 128 ? 2 : 3) void bwd_dq_kernel(const AttnParams p) {
     constexpr bool IDX = MODE == MASK_INDEXED, DENSE = MODE == MASK_DENSE;
     constexpr int NCH = D / 8, KK = D / 16, DB = D / 32;
     __shared__ u32x4 sK[2][DQ_KT * NCH];

@@ -32,7 +32,7 @@ constexpr int FWD_THREADS = 256;
 // (the reference's sibling kernel, cornstarch/kernel/attention.py:184-232), read from global memory in the
 // tiles the flags call partial.
 template <typename T, int D, int MODE>
-__global__ __launch_bounds__(FWD_THREADS, 2) void fwd_kernel(const AttnParams p) {
+__global__ __launch_bounds__(FWD_THREADS, D == 128 ? 2 : 3) void fwd_kernel(const AttnParams p) {
     constexpr int NCH = D / 8, KK = D / 16, DB = D / 32;
     __shared__ u32x4 sK[2][FWD_KT * NCH];
     __shared__ u32x4 sV[2][FWD_KT * NCH];
