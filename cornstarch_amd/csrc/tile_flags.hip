@@ -9,6 +9,9 @@ namespace bam {
 // One workgroup = one 128-row block x FLAG_COLS_PER_BLOCK key tiles.  Each wave takes one
 // 128x32 tile at a time: lane l owns key column (l & 31) and the 64 query rows of half
 // (l >> 5); the per-lane counts are summed over the wave.
+// Shortcut: when the 128 rows carry one bitfield and the 32 columns carry one bitfield (and the
+// tile lies inside the sequence) the class follows from one evaluation of the bit test plus the
+// position of the tile relative to the diagonal; long runs of equal bitfields are the common case.
 constexpr int FLAG_WAVES = 4;
 constexpr int FLAG_TILES_PER_WAVE = 8;
 constexpr int FLAG_COLS_PER_BLOCK = FLAG_WAVES * FLAG_TILES_PER_WAVE;
@@ -29,11 +32,31 @@ __global__ __launch_bounds__(FLAG_WAVES * 64) void tile_flags_kernel(const int64
     __syncthreads();
     const int rows_in_range = min(BLOCK_M, S - m * BLOCK_M);
     const int half = lane >> 5;
+    const int64_t q0 = q_bits[0];
+    const bool rows_uniform = rows_in_range == BLOCK_M && __all(q_bits[lane] == q0 && q_bits[lane + 64] == q0);
     for (int t = 0; t < FLAG_TILES_PER_WAVE; ++t) {
         const int n = blockIdx.x * FLAG_COLS_PER_BLOCK + wave * FLAG_TILES_PER_WAVE + t;
         if (n >= num_n) break;  // wave-uniform
         const int j = n * BLOCK_N + (lane & 31);
         const int64_t kf = (j < S) ? row[j] : 0;
+        if (rows_uniform && (n + 1) * BLOCK_N <= S) {
+            const unsigned klo = __builtin_amdgcn_readfirstlane((unsigned)kf);
+            const unsigned khi = __builtin_amdgcn_readfirstlane((unsigned)((uint64_t)kf >> 32));
+            const int64_t k0 = (int64_t)(((uint64_t)khi << 32) | klo);
+            if (__all(kf == k0)) {
+                const int64_t M = (((int64_t)1) << 62) - 1;
+                const int64_t qb = q0 & M, kb = k0 & M;
+                int8_t f;
+                if (q0 & 1) {  // text rows: causal over keys that share a bit
+                    const int r0 = m * BLOCK_M, c0 = n * BLOCK_N;
+                    f = (qb & kb) == 0 ? 0 : r0 >= c0 + BLOCK_N - 1 ? 2 : r0 + BLOCK_M - 1 < c0 ? 0 : 1;
+                } else {
+                    f = (qb == kb && qb != 0) ? 2 : 0;
+                }
+                if (lane == 0) flags[(int64_t)b * flags_stride_b + (int64_t)m * flags_stride_m + n] = f;
+                continue;
+            }
+        }
         int cnt = 0;
 #pragma unroll 8
         for (int r = 0; r < 64; ++r) {
