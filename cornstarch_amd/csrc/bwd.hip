@@ -187,7 +187,7 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
         // every MFMA come from LDS and are requested AHEAD MFMAs in front of their use
         f32x16 s, dp;
         {
-            constexpr int NOP = 2 * KK, AHEAD = 2;  // MFMA j: S (j even) or dP (j odd), k-slice j / 2
+            constexpr int NOP = 2 * KK, AHEAD = 3;  // MFMA j: S (j even) or dP (j odd), k-slice j / 2
             u32x4 a[NOP], bb[NOP];
 #pragma unroll
             for (int j = 0; j < AHEAD; ++j) {
@@ -314,7 +314,7 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
                     dv[db] = T::mfma(tg[t][db], pb[t], dv[db]);
                     dk[db] = T::mfma(tq[t][db], dsb[t], dk[db]);
                 }
-            sched_pipeline_mfma_lds<4 * DB, 3, 2>();
+            sched_pipeline_mfma_lds<4 * DB, 4, 2>();
         }
     };
 
