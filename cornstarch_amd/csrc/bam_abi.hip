@@ -27,8 +27,9 @@ int check_half_tensor(const char* name, const void* ptr, int64_t sb, int64_t ss,
     if ((sb % 8) || (ss % 8) || (sh % 8))
         return fail(BAM_ERR_INVALID_ARGUMENT, "%s: strides (%lld, %lld, %lld) must be multiples of 8 elements", name,
                     (long long)sb, (long long)ss, (long long)sh);
-    if (ss < 0 || ss >= (1ll << 24))
-        return fail(BAM_ERR_UNSUPPORTED, "%s: sequence stride %lld is outside [0, 2^24) elements", name, (long long)ss);
+    // tile copies hold row * stride as 32-bit byte offsets, for up to 128 rows of 2-byte elements
+    if (ss < 0 || ss >= (1ll << 23))
+        return fail(BAM_ERR_UNSUPPORTED, "%s: sequence stride %lld is outside [0, 2^23) elements", name, (long long)ss);
     return BAM_OK;
 }
 
@@ -80,6 +81,12 @@ MaskSource plain_source(const int64_t* bf, int64_t bf_stride_b, int S) {
 
 MaskSource dense_source(const uint8_t* mask, int Sq, int Sk) {
     return MaskSource{bam::MASK_DENSE, nullptr, nullptr, 0, 0, nullptr, nullptr, mask, Sq, Sk};
+}
+
+// the kernels read the mask four bytes at a time when rows are a multiple of four bytes long
+int check_mask(const char* who, const uint8_t* mask) {
+    if (reinterpret_cast<uintptr_t>(mask) & 3u) return fail(BAM_ERR_INVALID_ARGUMENT, "%s: mask is not 4-byte aligned", who);
+    return BAM_OK;
 }
 
 int indexed_source(const bam_index_view* iv, MaskSource& m) {
@@ -405,6 +412,7 @@ int bam_fwd_masked(const void* q, const void* k, const void* v, void* o, float* 
                    int64_t v_stride_s, int64_t v_stride_h, int64_t o_stride_b, int64_t o_stride_s,
                    int64_t o_stride_h, int64_t flags_stride_b, int64_t flags_stride_m, int B, int Sq, int Sk, int Hq,
                    int Hkv, int D, float scale, int dtype, void* stream) {
+    BAM_TRY(check_mask("bam_fwd_masked", mask));
     const int64_t st[12] = BAM_FWD_STRIDES;
     return fwd_impl("bam_fwd_masked", q, k, v, o, lse, dense_source(mask, Sq, Sk), flags, st, flags_stride_b,
                     flags_stride_m, B, Hq, Hkv, D, scale, dtype, stream);
@@ -419,6 +427,7 @@ int bam_bwd_dkdv_masked(const void* q, const void* k, const void* v, const void*
                         int64_t dv_stride_s, int64_t dv_stride_h, int64_t flags_stride_b, int64_t flags_stride_m,
                         int B, int Sq, int Sk, int Hq, int Hkv, int D, float scale, int dtype, int accumulate,
                         void* stream) {
+    BAM_TRY(check_mask("bam_bwd_dkdv_masked", mask));
     void* dq = nullptr;
     const int64_t dq_stride_b = 0, dq_stride_s = 0, dq_stride_h = 0;
     const int64_t st[23] = BAM_BWD_STRIDES;
@@ -435,6 +444,7 @@ int bam_bwd_dq_masked(const void* q, const void* k, const void* v, const void* d
                       int64_t do_stride_b, int64_t do_stride_s, int64_t do_stride_h, int64_t dq_stride_b,
                       int64_t dq_stride_s, int64_t dq_stride_h, int64_t flags_stride_b, int64_t flags_stride_m, int B,
                       int Sq, int Sk, int Hq, int Hkv, int D, float scale, int dtype, int accumulate, void* stream) {
+    BAM_TRY(check_mask("bam_bwd_dq_masked", mask));
     void *dk = nullptr, *dv = nullptr;
     const int64_t dk_stride_b = 0, dk_stride_s = 0, dk_stride_h = 0, dv_stride_b = 0, dv_stride_s = 0, dv_stride_h = 0;
     const int64_t st[23] = BAM_BWD_STRIDES;

@@ -44,7 +44,7 @@ __device__ __forceinline__ void wait_async() { asm volatile("s_waitcnt vmcnt(0)"
 // slot `id`.  `setup` fixes those source offsets once per kernel; `issue(i, ...)` emits copy
 // instruction i of CPT so that callers can spread a tile's copies between other work.
 // The last, ragged tile of a sequence takes the synchronous path (`load_ragged`), which
-// zero-fills the rows past the end.  Row strides are limited to 2^24 elements by the host
+// zero-fills the rows past the end.  Row strides are limited to 2^23 elements by the host
 // checks, so the offsets fit 32 bits.
 template <int D, int ROWS, int THREADS>
 struct TileStage {

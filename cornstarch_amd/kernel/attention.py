@@ -61,7 +61,9 @@ def _checked_mask(mask, batch, seqlen_q, seqlen_k):
     assert mask.shape == (batch, seqlen_q, seqlen_k), (
         f"Expected mask shape ({batch, seqlen_q, seqlen_k}), got {mask.shape}"
     )
-    return mask if mask.is_contiguous() else mask.contiguous()
+    if not mask.is_contiguous() or mask.data_ptr() % 4:
+        mask = mask.clone(memory_format=torch.contiguous_format)
+    return mask
 
 
 def _flash_attn_forward(
