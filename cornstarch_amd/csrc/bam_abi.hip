@@ -101,6 +101,22 @@ int indexed_source(const bam_index_view* iv, MaskSource& m) {
     return BAM_OK;
 }
 
+// bias may be null.  The kernels read groups of four keys with one access when base and strides allow it.
+int fill_bias(bam::AttnParams& p, const char* who, const bam_bias* bias, int Sk) {
+    if (bias == nullptr) return BAM_OK;  // p.bias stays null
+    if (bias->ptr == nullptr) return fail(BAM_ERR_INVALID_ARGUMENT, "%s: bias: null pointer", who);
+    const int esz = bias->is_f32 ? 4 : 2;
+    if (reinterpret_cast<uintptr_t>(bias->ptr) % esz) return fail(BAM_ERR_INVALID_ARGUMENT, "%s: bias: misaligned pointer", who);
+    p.bias = bias->ptr;
+    p.bias_sb = bias->stride_b;
+    p.bias_sh = bias->stride_h;
+    p.bias_sm = bias->stride_m;
+    p.bias_f32 = bias->is_f32 ? 1 : 0;
+    p.bias_vec = (reinterpret_cast<uintptr_t>(bias->ptr) % (4 * esz) == 0) && (bias->stride_b % 4 == 0) &&
+                 (bias->stride_h % 4 == 0) && (bias->stride_m % 4 == 0) && (Sk % 4 == 0);
+    return BAM_OK;
+}
+
 void fill_sizes(bam::AttnParams& p, const MaskSource& m, int B, int Hq, int Hkv, int D, float scale) {
     p.bfq = m.bfq;
     p.bfk = m.bfk;
@@ -125,11 +141,11 @@ void fill_sizes(bam::AttnParams& p, const MaskSource& m, int B, int Hq, int Hkv,
 
 int fwd_impl(const char* who, const void* q, const void* k, const void* v, void* o, float* lse, const MaskSource& m,
              const int8_t* flags, const int64_t* st, int64_t flags_stride_b, int64_t flags_stride_m, int B, int Hq,
-             int Hkv, int D, float scale, int dtype, void* stream);
+             int Hkv, int D, float scale, int dtype, const bam_bias* bias, void* stream);
 int bwd_params(bam::AttnParams& p, const char* who, const void* q, const void* k, const void* v, const void* dout,
                const float* lse, const float* delta, void* dq, void* dk, void* dv, const MaskSource& m,
                const int8_t* flags, const int64_t* st, int B, int Hq, int Hkv, int D, float scale, int dtype,
-               int accumulate, bool need_dq, bool need_dkdv);
+               int accumulate, bool need_dq, bool need_dkdv, const bam_bias* bias);
 
 }  // namespace
 
@@ -143,7 +159,7 @@ namespace {
 
 int fwd_impl(const char* who, const void* q, const void* k, const void* v, void* o, float* lse, const MaskSource& m,
              const int8_t* flags, const int64_t* st, int64_t flags_stride_b, int64_t flags_stride_m, int B, int Hq,
-             int Hkv, int D, float scale, int dtype, void* stream) {
+             int Hkv, int D, float scale, int dtype, const bam_bias* bias, void* stream) {
     BAM_TRY(check_problem(B, m.Sq, m.Sk, Hq, Hkv, D, dtype));
     BAM_TRY(check_half_tensor("q", q, st[0], st[1], st[2]));
     BAM_TRY(check_half_tensor("k", k, st[3], st[4], st[5]));
@@ -162,6 +178,7 @@ int fwd_impl(const char* who, const void* q, const void* k, const void* v, void*
     p.flags_sb = flags_stride_b;
     p.flags_sm = flags_stride_m;
     fill_sizes(p, m, B, Hq, Hkv, D, scale);
+    BAM_TRY(fill_bias(p, who, bias, m.Sk));
     return launched(bam::launch_fwd(p, dtype, (hipStream_t)stream), who);
 }
 
@@ -169,7 +186,7 @@ int fwd_impl(const char* who, const void* q, const void* k, const void* v, void*
 int bwd_params(bam::AttnParams& p, const char* who, const void* q, const void* k, const void* v, const void* dout,
                const float* lse, const float* delta, void* dq, void* dk, void* dv, const MaskSource& m,
                const int8_t* flags, const int64_t* st, int B, int Hq, int Hkv, int D, float scale, int dtype,
-               int accumulate, bool need_dq, bool need_dkdv) {
+               int accumulate, bool need_dq, bool need_dkdv, const bam_bias* bias) {
     BAM_TRY(check_problem(B, m.Sq, m.Sk, Hq, Hkv, D, dtype));
     BAM_TRY(check_half_tensor("q", q, st[0], st[1], st[2]));
     BAM_TRY(check_half_tensor("k", k, st[3], st[4], st[5]));
@@ -206,7 +223,7 @@ int bwd_params(bam::AttnParams& p, const char* who, const void* q, const void* k
     p.flags_sb = st[21];
     p.flags_sm = st[22];
     fill_sizes(p, m, B, Hq, Hkv, D, scale);
-    return BAM_OK;
+    return fill_bias(p, who, bias, m.Sk);
 }
 
 }  // namespace
@@ -215,7 +232,7 @@ extern "C" {
 
 const char* bam_last_error(void) { return g_error; }
 
-int bam_abi_version(void) { return 4; }
+int bam_abi_version(void) { return 5; }
 
 int bam_tile_flags(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int64_t flags_stride_b,
                    int64_t flags_stride_m, int B, int S, void* stream) {
@@ -267,10 +284,10 @@ int bam_fwd(const void* q, const void* k, const void* v, void* o, float* lse, co
             int64_t k_stride_b, int64_t k_stride_s, int64_t k_stride_h, int64_t v_stride_b,
             int64_t v_stride_s, int64_t v_stride_h, int64_t o_stride_b, int64_t o_stride_s,
             int64_t o_stride_h, int64_t bf_stride_b, int64_t flags_stride_b, int64_t flags_stride_m, int B,
-            int S, int Hq, int Hkv, int D, float scale, int dtype, void* stream) {
+            int S, int Hq, int Hkv, int D, float scale, int dtype, const bam_bias* bias, void* stream) {
     const int64_t st[12] = BAM_FWD_STRIDES;
     return fwd_impl("bam_fwd", q, k, v, o, lse, plain_source(bf, bf_stride_b, S), flags, st, flags_stride_b,
-                    flags_stride_m, B, Hq, Hkv, D, scale, dtype, stream);
+                    flags_stride_m, B, Hq, Hkv, D, scale, dtype, bias, stream);
 }
 
 int bam_fwd_indexed(const void* q, const void* k, const void* v, void* o, float* lse, const bam_index_view* iv,
@@ -278,12 +295,12 @@ int bam_fwd_indexed(const void* q, const void* k, const void* v, void* o, float*
                     int64_t k_stride_b, int64_t k_stride_s, int64_t k_stride_h, int64_t v_stride_b,
                     int64_t v_stride_s, int64_t v_stride_h, int64_t o_stride_b, int64_t o_stride_s,
                     int64_t o_stride_h, int64_t flags_stride_b, int64_t flags_stride_m, int B, int Hq, int Hkv,
-                    int D, float scale, int dtype, void* stream) {
+                    int D, float scale, int dtype, const bam_bias* bias, void* stream) {
     MaskSource m;
     BAM_TRY(indexed_source(iv, m));
     const int64_t st[12] = BAM_FWD_STRIDES;
     return fwd_impl("bam_fwd_indexed", q, k, v, o, lse, m, flags, st, flags_stride_b, flags_stride_m, B, Hq, Hkv, D,
-                    scale, dtype, stream);
+                    scale, dtype, bias, stream);
 }
 
 int bam_bwd_preprocess(const void* o, const void* dout, float* delta, int64_t o_stride_b, int64_t o_stride_s,
@@ -314,11 +331,11 @@ int bam_bwd(const void* q, const void* k, const void* v, const void* dout, const
             int64_t dq_stride_b, int64_t dq_stride_s, int64_t dq_stride_h, int64_t dk_stride_b,
             int64_t dk_stride_s, int64_t dk_stride_h, int64_t dv_stride_b, int64_t dv_stride_s,
             int64_t dv_stride_h, int64_t bf_stride_b, int64_t flags_stride_b, int64_t flags_stride_m, int B,
-            int S, int Hq, int Hkv, int D, float scale, int dtype, int accumulate, void* stream) {
+            int S, int Hq, int Hkv, int D, float scale, int dtype, int accumulate, const bam_bias* bias, void* stream) {
     const int64_t st[23] = BAM_BWD_STRIDES;
     bam::AttnParams p = {};
     BAM_TRY(bwd_params(p, "bam_bwd", q, k, v, dout, lse, delta, dq, dk, dv, plain_source(bf, bf_stride_b, S), flags, st, B,
-                       Hq, Hkv, D, scale, dtype, accumulate, true, true));
+                       Hq, Hkv, D, scale, dtype, accumulate, true, true, bias));
     BAM_TRY(launched(bam::launch_bwd_dkdv(p, dtype, (hipStream_t)stream), "bam_bwd (dk/dv)"));
     return launched(bam::launch_bwd_dq(p, dtype, (hipStream_t)stream), "bam_bwd (dq)");
 }
@@ -331,13 +348,13 @@ int bam_bwd_dkdv(const void* q, const void* k, const void* v, const void* dout, 
                  int64_t dk_stride_b, int64_t dk_stride_s, int64_t dk_stride_h, int64_t dv_stride_b,
                  int64_t dv_stride_s, int64_t dv_stride_h, int64_t bf_stride_b, int64_t flags_stride_b,
                  int64_t flags_stride_m, int B, int S, int Hq, int Hkv, int D, float scale, int dtype,
-                 int accumulate, void* stream) {
+                 int accumulate, const bam_bias* bias, void* stream) {
     void* dq = nullptr;
     const int64_t dq_stride_b = 0, dq_stride_s = 0, dq_stride_h = 0;
     const int64_t st[23] = BAM_BWD_STRIDES;
     bam::AttnParams p = {};
     BAM_TRY(bwd_params(p, "bam_bwd_dkdv", q, k, v, dout, lse, delta, dq, dk, dv, plain_source(bf, bf_stride_b, S), flags,
-                       st, B, Hq, Hkv, D, scale, dtype, accumulate, false, true));
+                       st, B, Hq, Hkv, D, scale, dtype, accumulate, false, true, bias));
     return launched(bam::launch_bwd_dkdv(p, dtype, (hipStream_t)stream), "bam_bwd_dkdv");
 }
 
@@ -348,13 +365,13 @@ int bam_bwd_dq(const void* q, const void* k, const void* v, const void* dout, co
                int64_t do_stride_b, int64_t do_stride_s, int64_t do_stride_h, int64_t dq_stride_b,
                int64_t dq_stride_s, int64_t dq_stride_h, int64_t bf_stride_b, int64_t flags_stride_b,
                int64_t flags_stride_m, int B, int S, int Hq, int Hkv, int D, float scale, int dtype,
-               int accumulate, void* stream) {
+               int accumulate, const bam_bias* bias, void* stream) {
     void *dk = nullptr, *dv = nullptr;
     const int64_t dk_stride_b = 0, dk_stride_s = 0, dk_stride_h = 0, dv_stride_b = 0, dv_stride_s = 0, dv_stride_h = 0;
     const int64_t st[23] = BAM_BWD_STRIDES;
     bam::AttnParams p = {};
     BAM_TRY(bwd_params(p, "bam_bwd_dq", q, k, v, dout, lse, delta, dq, dk, dv, plain_source(bf, bf_stride_b, S), flags, st,
-                       B, Hq, Hkv, D, scale, dtype, accumulate, true, false));
+                       B, Hq, Hkv, D, scale, dtype, accumulate, true, false, bias));
     return launched(bam::launch_bwd_dq(p, dtype, (hipStream_t)stream), "bam_bwd_dq");
 }
 
@@ -365,7 +382,7 @@ int bam_bwd_dkdv_indexed(const void* q, const void* k, const void* v, const void
                          int64_t v_stride_h, int64_t do_stride_b, int64_t do_stride_s, int64_t do_stride_h,
                          int64_t dk_stride_b, int64_t dk_stride_s, int64_t dk_stride_h, int64_t dv_stride_b,
                          int64_t dv_stride_s, int64_t dv_stride_h, int64_t flags_stride_b, int64_t flags_stride_m,
-                         int B, int Hq, int Hkv, int D, float scale, int dtype, int accumulate, void* stream) {
+                         int B, int Hq, int Hkv, int D, float scale, int dtype, int accumulate, const bam_bias* bias, void* stream) {
     MaskSource m;
     BAM_TRY(indexed_source(iv, m));
     void* dq = nullptr;
@@ -373,7 +390,7 @@ int bam_bwd_dkdv_indexed(const void* q, const void* k, const void* v, const void
     const int64_t st[23] = BAM_BWD_STRIDES;
     bam::AttnParams p = {};
     BAM_TRY(bwd_params(p, "bam_bwd_dkdv_indexed", q, k, v, dout, lse, delta, dq, dk, dv, m, flags, st, B, Hq, Hkv, D, scale,
-                       dtype, accumulate, false, true));
+                       dtype, accumulate, false, true, bias));
     return launched(bam::launch_bwd_dkdv(p, dtype, (hipStream_t)stream), "bam_bwd_dkdv_indexed");
 }
 
@@ -384,7 +401,7 @@ int bam_bwd_dq_indexed(const void* q, const void* k, const void* v, const void* 
                        int64_t v_stride_h, int64_t do_stride_b, int64_t do_stride_s, int64_t do_stride_h,
                        int64_t dq_stride_b, int64_t dq_stride_s, int64_t dq_stride_h, int64_t flags_stride_b,
                        int64_t flags_stride_m, int B, int Hq, int Hkv, int D, float scale, int dtype,
-                       int accumulate, void* stream) {
+                       int accumulate, const bam_bias* bias, void* stream) {
     MaskSource m;
     BAM_TRY(indexed_source(iv, m));
     void *dk = nullptr, *dv = nullptr;
@@ -392,7 +409,7 @@ int bam_bwd_dq_indexed(const void* q, const void* k, const void* v, const void* 
     const int64_t st[23] = BAM_BWD_STRIDES;
     bam::AttnParams p = {};
     BAM_TRY(bwd_params(p, "bam_bwd_dq_indexed", q, k, v, dout, lse, delta, dq, dk, dv, m, flags, st, B, Hq, Hkv, D, scale,
-                       dtype, accumulate, true, false));
+                       dtype, accumulate, true, false, bias));
     return launched(bam::launch_bwd_dq(p, dtype, (hipStream_t)stream), "bam_bwd_dq_indexed");
 }
 
@@ -411,11 +428,11 @@ int bam_fwd_masked(const void* q, const void* k, const void* v, void* o, float* 
                    int64_t k_stride_b, int64_t k_stride_s, int64_t k_stride_h, int64_t v_stride_b,
                    int64_t v_stride_s, int64_t v_stride_h, int64_t o_stride_b, int64_t o_stride_s,
                    int64_t o_stride_h, int64_t flags_stride_b, int64_t flags_stride_m, int B, int Sq, int Sk, int Hq,
-                   int Hkv, int D, float scale, int dtype, void* stream) {
+                   int Hkv, int D, float scale, int dtype, const bam_bias* bias, void* stream) {
     BAM_TRY(check_mask("bam_fwd_masked", mask));
     const int64_t st[12] = BAM_FWD_STRIDES;
     return fwd_impl("bam_fwd_masked", q, k, v, o, lse, dense_source(mask, Sq, Sk), flags, st, flags_stride_b,
-                    flags_stride_m, B, Hq, Hkv, D, scale, dtype, stream);
+                    flags_stride_m, B, Hq, Hkv, D, scale, dtype, bias, stream);
 }
 
 int bam_bwd_dkdv_masked(const void* q, const void* k, const void* v, const void* dout, const float* lse,
@@ -426,14 +443,14 @@ int bam_bwd_dkdv_masked(const void* q, const void* k, const void* v, const void*
                         int64_t dk_stride_b, int64_t dk_stride_s, int64_t dk_stride_h, int64_t dv_stride_b,
                         int64_t dv_stride_s, int64_t dv_stride_h, int64_t flags_stride_b, int64_t flags_stride_m,
                         int B, int Sq, int Sk, int Hq, int Hkv, int D, float scale, int dtype, int accumulate,
-                        void* stream) {
+                        const bam_bias* bias, void* stream) {
     BAM_TRY(check_mask("bam_bwd_dkdv_masked", mask));
     void* dq = nullptr;
     const int64_t dq_stride_b = 0, dq_stride_s = 0, dq_stride_h = 0;
     const int64_t st[23] = BAM_BWD_STRIDES;
     bam::AttnParams p = {};
     BAM_TRY(bwd_params(p, "bam_bwd_dkdv_masked", q, k, v, dout, lse, delta, dq, dk, dv, dense_source(mask, Sq, Sk), flags,
-                       st, B, Hq, Hkv, D, scale, dtype, accumulate, false, true));
+                       st, B, Hq, Hkv, D, scale, dtype, accumulate, false, true, bias));
     return launched(bam::launch_bwd_dkdv(p, dtype, (hipStream_t)stream), "bam_bwd_dkdv_masked");
 }
 
@@ -443,14 +460,14 @@ int bam_bwd_dq_masked(const void* q, const void* k, const void* v, const void* d
                       int64_t k_stride_h, int64_t v_stride_b, int64_t v_stride_s, int64_t v_stride_h,
                       int64_t do_stride_b, int64_t do_stride_s, int64_t do_stride_h, int64_t dq_stride_b,
                       int64_t dq_stride_s, int64_t dq_stride_h, int64_t flags_stride_b, int64_t flags_stride_m, int B,
-                      int Sq, int Sk, int Hq, int Hkv, int D, float scale, int dtype, int accumulate, void* stream) {
+                      int Sq, int Sk, int Hq, int Hkv, int D, float scale, int dtype, int accumulate, const bam_bias* bias, void* stream) {
     BAM_TRY(check_mask("bam_bwd_dq_masked", mask));
     void *dk = nullptr, *dv = nullptr;
     const int64_t dk_stride_b = 0, dk_stride_s = 0, dk_stride_h = 0, dv_stride_b = 0, dv_stride_s = 0, dv_stride_h = 0;
     const int64_t st[23] = BAM_BWD_STRIDES;
     bam::AttnParams p = {};
     BAM_TRY(bwd_params(p, "bam_bwd_dq_masked", q, k, v, dout, lse, delta, dq, dk, dv, dense_source(mask, Sq, Sk), flags, st,
-                       B, Hq, Hkv, D, scale, dtype, accumulate, true, false));
+                       B, Hq, Hkv, D, scale, dtype, accumulate, true, false, bias));
     return launched(bam::launch_bwd_dq(p, dtype, (hipStream_t)stream), "bam_bwd_dq_masked");
 }
 

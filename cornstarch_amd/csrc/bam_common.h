@@ -116,6 +116,46 @@ __device__ __forceinline__ u32x4 pack8(const f32x16& c, int base) {
     return r;
 }
 
+// Four consecutive elements key .. key + 3 of one row of an attention bias, as floats.  `row` points at the
+// row's element for key 0; keys at or past Sk read as 0.  `vec`: the group is one aligned access that lies
+// completely inside or completely outside the row (key is a multiple of four).
+template <typename T>
+__device__ __forceinline__ f32x4 load_bias4(const void* row, int key, int Sk, bool f32, bool vec) {
+    f32x4 r = {0.f, 0.f, 0.f, 0.f};
+    if (f32) {
+        const float* pf = (const float*)row + key;
+        if (vec) {
+            if (key < Sk) r = *(const f32x4*)pf;
+        } else {
+#pragma unroll
+            for (int x = 0; x < 4; ++x)
+                if (key + x < Sk) r[x] = pf[x];
+        }
+    } else {
+        const unsigned short* ph = (const unsigned short*)row + key;
+        if (vec) {
+            if (key < Sk) {
+                const u32x2 w = *(const u32x2*)ph;
+                r[0] = T::to_float((unsigned short)(w[0] & 0xFFFFu));
+                r[1] = T::to_float((unsigned short)(w[0] >> 16));
+                r[2] = T::to_float((unsigned short)(w[1] & 0xFFFFu));
+                r[3] = T::to_float((unsigned short)(w[1] >> 16));
+            }
+        } else {
+#pragma unroll
+            for (int x = 0; x < 4; ++x)
+                if (key + x < Sk) r[x] = T::to_float(ph[x]);
+        }
+    }
+    return r;
+}
+
+// One element of an attention bias as float.
+template <typename T>
+__device__ __forceinline__ float load_bias1(const void* base, int64_t index, bool f32) {
+    return f32 ? ((const float*)base)[index] : T::to_float(((const unsigned short*)base)[index]);
+}
+
 // ---------------------------------------------------------------------------------
 // LDS tile layout.  A tile is ROWS x D elements of 2 bytes, stored as 16-byte chunks;
 // chunk c of row r lives at chunk slot  r * (D/8) + (c ^ swz(r)).  The XOR pattern is a

@@ -35,6 +35,13 @@ struct AttnParams {
     // MASK_DENSE: bool mask (B, Sq, Sk), contiguous, one byte per pair; null = every in-range pair allowed
     const uint8_t* mask;
     int mask_mode;             // MASK_BITFIELD / MASK_INDEXED / MASK_DENSE
+    // Additive attention bias (reference bitfield_attention.py:321-329, :410-434): a logical (B, Hq, Sq, Sk)
+    // view with unit stride along the keys, added to scale * q.k before the softmax; null = none.  A stride of
+    // 0 broadcasts (the per-key "vector" form has bias_sm == 0).
+    const void* bias;
+    int64_t bias_sb, bias_sh, bias_sm;  // in elements
+    int bias_f32;              // element type: 1 = fp32, 0 = the dtype of q
+    int bias_vec;              // every group of four keys starting at a multiple of four is one aligned, in-range access
     const int8_t* flags;       // (B, num_m, num_n)
     int64_t flags_sb, flags_sm;
     int B, Sq, Sk, Hq, Hkv, D;

@@ -63,7 +63,8 @@ constexpr int DKDV_THREADS = 512;
 
 // MODE (MASK_*): MASK_INDEXED = explicit global positions p.posq / p.posk and gathered bitfield arrays;
 // MASK_DENSE = a materialized bool mask read from global memory in partial tiles.
-template <typename T, int D, int MODE>
+// BIAS: the forward added p.bias to scale * q.k (reference bitfield_attention.py:815-835); P is recomputed with it.
+template <typename T, int D, int MODE, bool BIAS>
 __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnParams p) {
     constexpr bool IDX = MODE == MASK_INDEXED, DENSE = MODE == MASK_DENSE;
     constexpr int NCH = D / 8, KK = D / 16, DB = D / 32;
@@ -127,7 +128,7 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
     f32x16 zero16;
 #pragma unroll
     for (int i = 0; i < 16; ++i) zero16[i] = 0.f;
-    const float c2 = p.scale * LOG2E;
+    const float c2 = BIAS ? LOG2E : p.scale * LOG2E;  // with a bias the scores become scale * s + bias first
 
     typedef TileStage<D, DKDV_QT, DKDV_THREADS> Stage;
     constexpr int CPT = Stage::CPT;
@@ -172,7 +173,7 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
     // condition the compiler can prove wave-uniform makes it restructure the loop around that branch, and the
     // result needs far more registers than a wave has.
     const int kg_lane = (tid >> 6) & 3;
-    auto tile_step = [&](auto prefetch, int cur, int cls, int row0, int h_next, int row0_next) {
+    auto tile_step = [&](auto prefetch, int cur, int cls, int h_cur, int row0, int h_next, int row0_next) {
         constexpr bool PREFETCH = decltype(prefetch)::value;
         if (cls == 0) {
             if (PREFETCH) {
@@ -212,6 +213,17 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
         // ---- P = exp(scale s - lse) on allowed pairs, dS/scale = P (dP - delta)   (the factor `scale` of dS
         // is applied once to dK in the epilogue).  C fragment: register i <-> query row
         // 8*(i/4) + 4*hi + i%4 of this wave's 32 rows.
+        if (BIAS) {
+            // column `key` of the bias, one element per row of the C fragment
+            const int64_t col = (int64_t)b * p.bias_sb + (int64_t)h_cur * p.bias_sh + key;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int row = row0 + qr + 8 * (i >> 2) + 4 * hi + (i & 3);
+                float bv = 0.f;
+                if (kvalid && row < Sq) bv = load_bias1<T>(p.bias, col + (int64_t)row * p.bias_sm, p.bias_f32 != 0);
+                s[i] = fmaf(s[i], p.scale, bv);
+            }
+        }
 #pragma unroll
         for (int grp = 0; grp < 4; ++grp) {
             const f32x4 l4 = *(const f32x4*)&sLse[cur][qr + 8 * grp + 4 * hi];
@@ -354,7 +366,7 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
             const bool more = it + 1 < total;
             const int h_next = hk * G + (more ? g_nxt : g_cur);
             const int row0_next = more ? row0_of(next, r_nxt) : row0_of(entry, r_cur);
-            tile_step(std::true_type{}, cur, (entry >> (2 * kg_lane)) & 3, row0_of(entry, r_cur), h_next, row0_next);
+            tile_step(std::true_type{}, cur, (entry >> (2 * kg_lane)) & 3, hk * G + g_cur, row0_of(entry, r_cur), h_next, row0_next);
             g_cur = g_nxt;
             r_cur = r_nxt;
             g_nxt = g_aft;
@@ -386,7 +398,7 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
                 if (IDX) sQpos[0][tid] = ok ? p.posq[row0 + tid] : 0;
             }
             __syncthreads();
-            tile_step(std::false_type{}, 0, (entry >> (2 * kg_lane)) & 3, row0, 0, 0);
+            tile_step(std::false_type{}, 0, (entry >> (2 * kg_lane)) & 3, h, row0, 0, 0);
         }
     }
     // every copy has landed and every wave is done with the tiles: the epilogue reuses the tile arrays
@@ -470,7 +482,7 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
 constexpr int DQ_KT = 64;
 constexpr int DQ_THREADS = 256;
 
-template <typename T, int D, int MODE>
+template <typename T, int D, int MODE, bool BIAS>
 __global__ __launch_bounds__(DQ_THREADS, D == 128 ? 2 : 3) void bwd_dq_kernel(const AttnParams p) {
     constexpr bool IDX = MODE == MASK_INDEXED, DENSE = MODE == MASK_DENSE;
     constexpr int NCH = D / 8, KK = D / 16, DB = D / 32;
@@ -533,7 +545,11 @@ __global__ __launch_bounds__(DQ_THREADS, D == 128 ? 2 : 3) void bwd_dq_kernel(co
     f32x16 zero16;
 #pragma unroll
     for (int i = 0; i < 16; ++i) zero16[i] = 0.f;
-    const float c2 = p.scale * LOG2E;
+    const float c2 = BIAS ? LOG2E : p.scale * LOG2E;  // with a bias the scores become scale * s + bias first
+    const char* bias_row = nullptr;  // this lane's row of the bias
+    if (BIAS)
+        bias_row = (const char*)p.bias + (p.bias_f32 ? 4 : 2) * ((int64_t)b * p.bias_sb + (int64_t)h * p.bias_sh +
+                                                                (int64_t)(qvalid ? qrow : 0) * p.bias_sm);
 
     const char* kbase = (const char*)p.k.ptr + 2 * ((int64_t)b * p.k.sb + (int64_t)hk * p.k.sh);
     const char* vbase = (const char*)p.v.ptr + 2 * ((int64_t)b * p.v.sb + (int64_t)hk * p.v.sh);
@@ -608,6 +624,14 @@ __global__ __launch_bounds__(DQ_THREADS, D == 128 ? 2 : 3) void bwd_dq_kernel(co
                     if (PREFETCH && kb == 0 && j < NLOADS) issue_copy(j, kt_next, cur ^ 1);
                 }
                 __builtin_amdgcn_sched_barrier(0);
+            }
+            if (BIAS) {
+#pragma unroll
+                for (int grp = 0; grp < 4; ++grp) {
+                    const f32x4 b4 = load_bias4<T>(bias_row, kt * DQ_KT + 32 * kb + 8 * grp + 4 * hi, Sk, p.bias_f32 != 0, p.bias_vec != 0);
+#pragma unroll
+                    for (int x = 0; x < 4; ++x) s[4 * grp + x] = fmaf(s[4 * grp + x], p.scale, b4[x]);
+                }
             }
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
@@ -762,27 +786,35 @@ static int launch_pre_t(const AttnParams& p, hipStream_t stream) {
     hipLaunchKernelGGL((bwd_preprocess_kernel<T, D>), dim3((unsigned)blocks), dim3(256), 0, stream, p);
     return (int)hipGetLastError();
 }
-template <typename T, int D>
-static int launch_dkdv_t(const AttnParams& p, hipStream_t stream) {
+template <typename T, int D, bool BIAS>
+static int launch_dkdv_b(const AttnParams& p, hipStream_t stream) {
     const int blocks = p.num_kt * p.B * p.Hkv;  // one workgroup per 128-key tile
     if (p.mask_mode == MASK_INDEXED)
-        hipLaunchKernelGGL((bwd_dkdv_kernel<T, D, MASK_INDEXED>), dim3(blocks), dim3(DKDV_THREADS), 0, stream, p);
+        hipLaunchKernelGGL((bwd_dkdv_kernel<T, D, MASK_INDEXED, BIAS>), dim3(blocks), dim3(DKDV_THREADS), 0, stream, p);
     else if (p.mask_mode == MASK_DENSE)
-        hipLaunchKernelGGL((bwd_dkdv_kernel<T, D, MASK_DENSE>), dim3(blocks), dim3(DKDV_THREADS), 0, stream, p);
+        hipLaunchKernelGGL((bwd_dkdv_kernel<T, D, MASK_DENSE, BIAS>), dim3(blocks), dim3(DKDV_THREADS), 0, stream, p);
     else
-        hipLaunchKernelGGL((bwd_dkdv_kernel<T, D, MASK_BITFIELD>), dim3(blocks), dim3(DKDV_THREADS), 0, stream, p);
+        hipLaunchKernelGGL((bwd_dkdv_kernel<T, D, MASK_BITFIELD, BIAS>), dim3(blocks), dim3(DKDV_THREADS), 0, stream, p);
+    return (int)hipGetLastError();
+}
+template <typename T, int D>
+static int launch_dkdv_t(const AttnParams& p, hipStream_t stream) {
+    return p.bias != nullptr ? launch_dkdv_b<T, D, true>(p, stream) : launch_dkdv_b<T, D, false>(p, stream);
+}
+template <typename T, int D, bool BIAS>
+static int launch_dq_b(const AttnParams& p, hipStream_t stream) {
+    const int blocks = p.num_m * p.B * p.Hq;
+    if (p.mask_mode == MASK_INDEXED)
+        hipLaunchKernelGGL((bwd_dq_kernel<T, D, MASK_INDEXED, BIAS>), dim3(blocks), dim3(DQ_THREADS), 0, stream, p);
+    else if (p.mask_mode == MASK_DENSE)
+        hipLaunchKernelGGL((bwd_dq_kernel<T, D, MASK_DENSE, BIAS>), dim3(blocks), dim3(DQ_THREADS), 0, stream, p);
+    else
+        hipLaunchKernelGGL((bwd_dq_kernel<T, D, MASK_BITFIELD, BIAS>), dim3(blocks), dim3(DQ_THREADS), 0, stream, p);
     return (int)hipGetLastError();
 }
 template <typename T, int D>
 static int launch_dq_t(const AttnParams& p, hipStream_t stream) {
-    const int blocks = p.num_m * p.B * p.Hq;
-    if (p.mask_mode == MASK_INDEXED)
-        hipLaunchKernelGGL((bwd_dq_kernel<T, D, MASK_INDEXED>), dim3(blocks), dim3(DQ_THREADS), 0, stream, p);
-    else if (p.mask_mode == MASK_DENSE)
-        hipLaunchKernelGGL((bwd_dq_kernel<T, D, MASK_DENSE>), dim3(blocks), dim3(DQ_THREADS), 0, stream, p);
-    else
-        hipLaunchKernelGGL((bwd_dq_kernel<T, D, MASK_BITFIELD>), dim3(blocks), dim3(DQ_THREADS), 0, stream, p);
-    return (int)hipGetLastError();
+    return p.bias != nullptr ? launch_dq_b<T, D, true>(p, stream) : launch_dq_b<T, D, false>(p, stream);
 }
 
 #define BAM_DISPATCH(fn)                                       \

@@ -31,7 +31,8 @@ constexpr int FWD_THREADS = 256;
 // (context-parallel shards, reference bitfield_attention.py:71-81).  MASK_DENSE: a materialized bool mask
 // (the reference's sibling kernel, cornstarch/kernel/attention.py:184-232), read from global memory in the
 // tiles the flags call partial.
-template <typename T, int D, int MODE>
+// BIAS: an additive bias p.bias (reference bitfield_attention.py:410-434) is added to scale * q.k.
+template <typename T, int D, int MODE, bool BIAS>
 __global__ __launch_bounds__(FWD_THREADS, D == 128 ? 2 : 3) void fwd_kernel(const AttnParams p) {
     constexpr int NCH = D / 8, KK = D / 16, DB = D / 32;
     __shared__ u32x4 sK[2][FWD_KT * NCH];
@@ -87,7 +88,13 @@ __global__ __launch_bounds__(FWD_THREADS, D == 128 ? 2 : 3) void fwd_kernel(cons
     // final division by l.
     constexpr float RESCALE_LOG2 = 8.f;
     float m_i = -INFINITY, l_i = 0.f, nb = 0.f;  // nb = -m_i * c2 (0 while m_i is -inf)
-    const float c2 = p.scale * LOG2E;
+    // with a bias the scores are turned into scale * s + bias right after the S phase, and only log2(e) is left
+    // to fold into the exponent
+    const float c2 = BIAS ? LOG2E : p.scale * LOG2E;
+    const char* bias_row = nullptr;  // this lane's row of the bias
+    if (BIAS)
+        bias_row = (const char*)p.bias + (p.bias_f32 ? 4 : 2) * ((int64_t)b * p.bias_sb + (int64_t)h * p.bias_sh +
+                                                                (int64_t)(qvalid ? qrow : 0) * p.bias_sm);
     const float rescale_thr = RESCALE_LOG2 / c2;
     f32x16 zero16;
 #pragma unroll
@@ -148,6 +155,17 @@ __global__ __launch_bounds__(FWD_THREADS, D == 128 ? 2 : 3) void fwd_kernel(cons
                 if (PREFETCH && j < NLOADS) issue_copy(j, kt_next, cur ^ 1);
             }
             __builtin_amdgcn_sched_barrier(0);
+        }
+
+        if (BIAS) {
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int grp = 0; grp < 4; ++grp) {
+                    const f32x4 b4 = load_bias4<T>(bias_row, kt * FWD_KT + 32 * kb + 8 * grp + 4 * hi, Sk, p.bias_f32 != 0, p.bias_vec != 0);
+#pragma unroll
+                    for (int x = 0; x < 4; ++x) s[kb][4 * grp + x] = fmaf(s[kb][4 * grp + x], p.scale, b4[x]);
+                }
         }
 
         // ---- bitfield rule in registers (partial tiles only) ------------------------------
@@ -343,16 +361,20 @@ __global__ __launch_bounds__(FWD_THREADS, D == 128 ? 2 : 3) void fwd_kernel(cons
     }
 }
 
-template <typename T, int D>
-static int launch_fwd_t(const AttnParams& p, hipStream_t stream) {
+template <typename T, int D, bool BIAS>
+static int launch_fwd_b(const AttnParams& p, hipStream_t stream) {
     const int blocks = p.num_m * p.B * p.Hq;
     if (p.mask_mode == MASK_INDEXED)
-        hipLaunchKernelGGL((fwd_kernel<T, D, MASK_INDEXED>), dim3(blocks), dim3(FWD_THREADS), 0, stream, p);
+        hipLaunchKernelGGL((fwd_kernel<T, D, MASK_INDEXED, BIAS>), dim3(blocks), dim3(FWD_THREADS), 0, stream, p);
     else if (p.mask_mode == MASK_DENSE)
-        hipLaunchKernelGGL((fwd_kernel<T, D, MASK_DENSE>), dim3(blocks), dim3(FWD_THREADS), 0, stream, p);
+        hipLaunchKernelGGL((fwd_kernel<T, D, MASK_DENSE, BIAS>), dim3(blocks), dim3(FWD_THREADS), 0, stream, p);
     else
-        hipLaunchKernelGGL((fwd_kernel<T, D, MASK_BITFIELD>), dim3(blocks), dim3(FWD_THREADS), 0, stream, p);
+        hipLaunchKernelGGL((fwd_kernel<T, D, MASK_BITFIELD, BIAS>), dim3(blocks), dim3(FWD_THREADS), 0, stream, p);
     return (int)hipGetLastError();
+}
+template <typename T, int D>
+static int launch_fwd_t(const AttnParams& p, hipStream_t stream) {
+    return p.bias != nullptr ? launch_fwd_b<T, D, true>(p, stream) : launch_fwd_b<T, D, false>(p, stream);
 }
 
 int launch_fwd(const AttnParams& p, int dtype, hipStream_t stream) {

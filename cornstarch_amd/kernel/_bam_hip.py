@@ -14,7 +14,7 @@ LIB_PATH = os.path.join(_PKG_DIR, "libbam_hip.so")
 BAM_DTYPE_F16 = 0
 BAM_DTYPE_BF16 = 1
 BAM_MAX_SEQLEN = 131072
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 _i64 = ctypes.c_int64
 _int = ctypes.c_int
@@ -36,26 +36,39 @@ class IndexView(ctypes.Structure):
     ]
 
 
+class Bias(ctypes.Structure):
+    """``bam_bias`` of include/bam_hip.h (host struct holding a device pointer)."""
+
+    _fields_ = [
+        ("ptr", ctypes.c_void_p),
+        ("stride_b", ctypes.c_int64),
+        ("stride_h", ctypes.c_int64),
+        ("stride_m", ctypes.c_int64),
+        ("is_f32", ctypes.c_int32),
+    ]
+
+
 _view = ctypes.POINTER(IndexView)
+_bias = ctypes.POINTER(Bias)
 
 # name -> argtypes, exactly the prototypes of include/bam_hip.h
 SIGNATURES = {
     "bam_tile_flags": [_ptr, _i64, _ptr, _i64, _i64, _int, _int, _ptr],
     "bam_materialize_mask": [_ptr, _i64, _ptr, _int, _int, _ptr],
-    "bam_fwd": [_ptr] * 7 + [_i64] * 15 + [_int] * 5 + [_f32, _int, _ptr],
+    "bam_fwd": [_ptr] * 7 + [_i64] * 15 + [_int] * 5 + [_f32, _int, _bias, _ptr],
     "bam_bwd_preprocess": [_ptr] * 3 + [_i64] * 6 + [_int] * 5 + [_ptr],
-    "bam_bwd": [_ptr] * 11 + [_i64] * 24 + [_int] * 5 + [_f32, _int, _int, _ptr],
-    "bam_bwd_dkdv": [_ptr] * 10 + [_i64] * 21 + [_int] * 5 + [_f32, _int, _int, _ptr],
-    "bam_bwd_dq": [_ptr] * 9 + [_i64] * 18 + [_int] * 5 + [_f32, _int, _int, _ptr],
+    "bam_bwd": [_ptr] * 11 + [_i64] * 24 + [_int] * 5 + [_f32, _int, _int, _bias, _ptr],
+    "bam_bwd_dkdv": [_ptr] * 10 + [_i64] * 21 + [_int] * 5 + [_f32, _int, _int, _bias, _ptr],
+    "bam_bwd_dq": [_ptr] * 9 + [_i64] * 18 + [_int] * 5 + [_f32, _int, _int, _bias, _ptr],
     "bam_mask_tile_flags": [_ptr, _ptr, _i64, _i64, _int, _int, _int, _ptr],
-    "bam_fwd_masked": [_ptr] * 7 + [_i64] * 14 + [_int] * 6 + [_f32, _int, _ptr],
-    "bam_bwd_dkdv_masked": [_ptr] * 10 + [_i64] * 20 + [_int] * 6 + [_f32, _int, _int, _ptr],
-    "bam_bwd_dq_masked": [_ptr] * 9 + [_i64] * 17 + [_int] * 6 + [_f32, _int, _int, _ptr],
+    "bam_fwd_masked": [_ptr] * 7 + [_i64] * 14 + [_int] * 6 + [_f32, _int, _bias, _ptr],
+    "bam_bwd_dkdv_masked": [_ptr] * 10 + [_i64] * 20 + [_int] * 6 + [_f32, _int, _int, _bias, _ptr],
+    "bam_bwd_dq_masked": [_ptr] * 9 + [_i64] * 17 + [_int] * 6 + [_f32, _int, _int, _bias, _ptr],
     "bam_flag_row_workloads": [_ptr, _i64, _i64, _int, _int, _int, _ptr, _ptr],
     "bam_gather_bitfields": [_ptr, _i64, _int, _ptr, _int, _ptr, _i64, _ptr, _int, _ptr],
-    "bam_fwd_indexed": [_ptr] * 5 + [_view, _ptr] + [_i64] * 14 + [_int] * 4 + [_f32, _int, _ptr],
-    "bam_bwd_dkdv_indexed": [_ptr] * 8 + [_view, _ptr] + [_i64] * 20 + [_int] * 4 + [_f32, _int, _int, _ptr],
-    "bam_bwd_dq_indexed": [_ptr] * 7 + [_view, _ptr] + [_i64] * 17 + [_int] * 4 + [_f32, _int, _int, _ptr],
+    "bam_fwd_indexed": [_ptr] * 5 + [_view, _ptr] + [_i64] * 14 + [_int] * 4 + [_f32, _int, _bias, _ptr],
+    "bam_bwd_dkdv_indexed": [_ptr] * 8 + [_view, _ptr] + [_i64] * 20 + [_int] * 4 + [_f32, _int, _int, _bias, _ptr],
+    "bam_bwd_dq_indexed": [_ptr] * 7 + [_view, _ptr] + [_i64] * 17 + [_int] * 4 + [_f32, _int, _int, _bias, _ptr],
 }
 
 _lib = None

@@ -20,6 +20,8 @@ import torch.nn.functional as F
 
 from . import _bam_hip
 from .bitfield_attention import (
+    _bias_arg,
+    _BiasView,
     _dtype_code,
     _is_kernel_ready,
     _kernel_ready,
@@ -31,11 +33,6 @@ from .bitfield_attention import (
 
 BLOCK_M = 128
 BLOCK_N = 32
-
-
-def _check_bias(bias):
-    if bias is not None:
-        raise NotImplementedError("attention bias is not implemented")
 
 
 def mask_tile_flags(mask: Optional[torch.Tensor], batch: int, seqlen_q: int, seqlen_k: int, device) -> torch.Tensor:
@@ -84,8 +81,9 @@ def _flash_attn_forward(
     assert q.dtype == k.dtype == v.dtype, "All tensors must have the same type"
     assert q.dtype in [torch.float16, torch.bfloat16], "Only support fp16 and bf16"
     assert q.is_cuda and k.is_cuda and v.is_cuda
-    _check_bias(bias)
     softmax_scale = softmax_scale or 1.0 / math.sqrt(d)
+    # reference attention.py:874-895
+    bias_view = _BiasView(bias, q, batch, nheads, seqlen_q, seqlen_k) if bias is not None else None
     mask = _checked_mask(mask, batch, seqlen_q, seqlen_k)
 
     dp = _padded_head_dim(d)
@@ -102,7 +100,7 @@ def _flash_attn_forward(
             mask.data_ptr() if mask is not None else None, flags.data_ptr(),
             *_strides3(qk, kk, vk, o), flags.stride(0), flags.stride(1),
             batch, seqlen_q, seqlen_k, nheads, nheads_k, dp, float(softmax_scale), _dtype_code(q.dtype),
-            _stream_ptr(q.device),
+            _bias_arg(bias_view), _stream_ptr(q.device),
         )
     if dp != d:
         o = o[..., :d].contiguous()
@@ -135,8 +133,9 @@ def _flash_attn_backward(
     assert lse.shape == (batch, nheads, seqlen_q_rounded)
     assert q.stride(-1) == k.stride(-1) == v.stride(-1) == o.stride(-1) == 1
     assert dq.stride(-1) == dk.stride(-1) == dv.stride(-1) == 1
-    _check_bias(bias)
     softmax_scale = softmax_scale or 1.0 / math.sqrt(d)
+    # the reference asserts the unit stride here instead of copying (attention.py:1002-1019)
+    bias_view = _BiasView(bias, q, batch, nheads, seqlen_q, seqlen_k, may_copy=False) if bias is not None else None
     mask = _checked_mask(mask, batch, seqlen_q, seqlen_k)
     flags = mask_tile_flags(mask, batch, seqlen_q, seqlen_k, q.device)
 
@@ -159,7 +158,7 @@ def _flash_attn_backward(
             wk.data_ptr(), wv.data_ptr(), mask_ptr, flags.data_ptr(),
             *_strides3(qk, kk, vk, gk, wk, wv), flags.stride(0), flags.stride(1),
             batch, seqlen_q, seqlen_k, nheads, nheads_k, dp, float(softmax_scale), _dtype_code(q.dtype), 0,
-            _stream_ptr(q.device),
+            _bias_arg(bias_view), _stream_ptr(q.device),
         )
         _bam_hip.call(
             "bam_bwd_dq_masked",
@@ -167,7 +166,7 @@ def _flash_attn_backward(
             wq.data_ptr(), mask_ptr, flags.data_ptr(),
             *_strides3(qk, kk, vk, gk, wq), flags.stride(0), flags.stride(1),
             batch, seqlen_q, seqlen_k, nheads, nheads_k, dp, float(softmax_scale), _dtype_code(q.dtype), 0,
-            _stream_ptr(q.device),
+            _bias_arg(bias_view), _stream_ptr(q.device),
         )
     if not direct:
         for dst, w in zip(outs, work):
@@ -191,6 +190,8 @@ class FlashAttnFunc(torch.autograd.Function):
         mask: optional bool (batch_size, seqlen_q, seqlen_k), True = attend
         """
         q, k, v = [x if x.stride(-1) == 1 else x.contiguous() for x in [q, k, v]]
+        if bias is not None and bias.stride(-1) != 1:
+            bias = bias.contiguous()
         o, lse, ctx.softmax_scale = _flash_attn_forward(q, k, v, bias=bias, mask=mask, softmax_scale=softmax_scale)
         ctx.save_for_backward(q, k, v, o, lse, bias, mask)
         return o

@@ -138,9 +138,41 @@ class BitfieldUtils:
         return out.to(torch.int64)
 
 
-def _check_unsupported(bias):
-    if bias is not None:
-        raise NotImplementedError("attention bias is not implemented (no caller of the reference passes one)")
+class _BiasView:
+    """Additive attention bias as the kernels take it: the checks and the broadcast of the reference host
+    functions (bitfield_attention.py:952-972, 1124-1143) and the ``bam_bias`` struct built from the expanded
+    view.  ``bias`` is 4-dimensional, broadcastable to (batch, nheads, seqlen_q, seqlen_k), its last two
+    dimensions are (1, seqlen_k) ("vector", e.g. ALiBi slopes times key position) or (seqlen_q, seqlen_k)
+    ("matrix"); fp32 or the dtype of q.  Nothing is copied unless the last stride is not 1."""
+
+    def __init__(self, bias: torch.Tensor, q: torch.Tensor, batch: int, nheads: int, seqlen_q: int, seqlen_k: int,
+                 may_copy: bool = True):
+        assert bias.dtype in [q.dtype, torch.float]
+        assert bias.is_cuda
+        assert bias.dim() == 4
+        if bias.stride(-1) != 1:
+            assert may_copy, "bias must have unit stride along the keys"
+            bias = bias.contiguous()
+        if bias.shape[2:] == (1, seqlen_k):
+            self.bias_type = "vector"
+        elif bias.shape[2:] == (seqlen_q, seqlen_k):
+            self.bias_type = "matrix"
+        else:
+            raise RuntimeError("Last 2 dimensions of bias must be (1, seqlen_k) or (seqlen_q, seqlen_k)")
+        bias = bias.expand(batch, nheads, seqlen_q, seqlen_k)
+        self.tensor = bias  # keeps the memory alive while launches are in flight on the host side
+        self.struct = _bam_hip.Bias(
+            bias.data_ptr(), bias.stride(0), bias.stride(1), bias.stride(2), int(bias.dtype == torch.float)
+        )
+
+    def byref(self):
+        import ctypes
+
+        return ctypes.byref(self.struct)
+
+
+def _bias_arg(view: Optional["_BiasView"]):
+    return view.byref() if view is not None else None
 
 
 class _IndexView:
@@ -206,7 +238,7 @@ def _bitfield_attn_forward(
     assert k.shape == v.shape and k.shape[0] == batch and k.shape[3] == d
     assert nheads % nheads_k == 0
     assert bitfield_mask.dtype == torch.int64 and bitfield_mask.dim() == 2 and bitfield_mask.shape[0] == batch
-    _check_unsupported(bias)
+    bias_view = _BiasView(bias, q, batch, nheads, seqlen_q, seqlen_k) if bias is not None else None
     view = None
     if offsets_q is not None or offsets_k is not None:
         view = _IndexView(bitfield_mask, offsets_q, offsets_k)
@@ -236,7 +268,7 @@ def _bitfield_attn_forward(
                 flags.data_ptr(), *_strides3(qk, kk, vk, o),
                 bf.stride(0), flags.stride(0), flags.stride(1),
                 batch, seqlen_q, nheads, nheads_k, dp, float(softmax_scale), _dtype_code(q.dtype),
-                _stream_ptr(q.device),
+                _bias_arg(bias_view), _stream_ptr(q.device),
             )
         else:
             _bam_hip.call(
@@ -245,7 +277,7 @@ def _bitfield_attn_forward(
                 flags.data_ptr(), *_strides3(qk, kk, vk, o),
                 flags.stride(0), flags.stride(1),
                 batch, nheads, nheads_k, dp, float(softmax_scale), _dtype_code(q.dtype),
-                _stream_ptr(q.device),
+                _bias_arg(bias_view), _stream_ptr(q.device),
             )
     if dp != d:
         o = o[..., :d].contiguous()
@@ -269,9 +301,10 @@ def _launch_bwd_preprocess(o, do, delta):
         )
 
 
-def _launch_bwd_dkdv(q, k, v, do, lse, delta, dk, dv, bf, flags, softmax_scale, accumulate=True):
+def _launch_bwd_dkdv(q, k, v, do, lse, delta, dk, dv, bf, flags, softmax_scale, accumulate=True, bias=None):
     """accumulate=True: dk/dv are fp32 and added to; False: dk/dv have q's dtype and are overwritten.
-    ``bf``: the (B, S) bitfield tensor, or an ``_IndexView`` for index-tensor attention."""
+    ``bf``: the (B, S) bitfield tensor, or an ``_IndexView`` for index-tensor attention.  ``bias``: a
+    ``_BiasView`` or None."""
     B, S, Hq, D = q.shape
     with torch.cuda.device(q.device):
         if isinstance(bf, _IndexView):
@@ -281,7 +314,7 @@ def _launch_bwd_dkdv(q, k, v, do, lse, delta, dk, dv, bf, flags, softmax_scale, 
                 dk.data_ptr(), dv.data_ptr(), bf.byref(), flags.data_ptr(),
                 *_strides3(q, k, v, do, dk, dv), flags.stride(0), flags.stride(1),
                 B, Hq, k.shape[2], D, float(softmax_scale), _dtype_code(q.dtype), int(accumulate),
-                _stream_ptr(q.device),
+                _bias_arg(bias), _stream_ptr(q.device),
             )
             return
         _bam_hip.call(
@@ -290,11 +323,11 @@ def _launch_bwd_dkdv(q, k, v, do, lse, delta, dk, dv, bf, flags, softmax_scale, 
             dk.data_ptr(), dv.data_ptr(), bf.data_ptr(), flags.data_ptr(),
             *_strides3(q, k, v, do, dk, dv), bf.stride(0), flags.stride(0), flags.stride(1),
             B, S, Hq, k.shape[2], D, float(softmax_scale), _dtype_code(q.dtype), int(accumulate),
-            _stream_ptr(q.device),
+            _bias_arg(bias), _stream_ptr(q.device),
         )
 
 
-def _launch_bwd_dq(q, k, v, do, lse, delta, dq, bf, flags, softmax_scale, accumulate=True):
+def _launch_bwd_dq(q, k, v, do, lse, delta, dq, bf, flags, softmax_scale, accumulate=True, bias=None):
     B, S, Hq, D = q.shape
     with torch.cuda.device(q.device):
         if isinstance(bf, _IndexView):
@@ -304,7 +337,7 @@ def _launch_bwd_dq(q, k, v, do, lse, delta, dq, bf, flags, softmax_scale, accumu
                 dq.data_ptr(), bf.byref(), flags.data_ptr(),
                 *_strides3(q, k, v, do, dq), flags.stride(0), flags.stride(1),
                 B, Hq, k.shape[2], D, float(softmax_scale), _dtype_code(q.dtype), int(accumulate),
-                _stream_ptr(q.device),
+                _bias_arg(bias), _stream_ptr(q.device),
             )
             return
         _bam_hip.call(
@@ -313,7 +346,7 @@ def _launch_bwd_dq(q, k, v, do, lse, delta, dq, bf, flags, softmax_scale, accumu
             dq.data_ptr(), bf.data_ptr(), flags.data_ptr(),
             *_strides3(q, k, v, do, dq), bf.stride(0), flags.stride(0), flags.stride(1),
             B, S, Hq, k.shape[2], D, float(softmax_scale), _dtype_code(q.dtype), int(accumulate),
-            _stream_ptr(q.device),
+            _bias_arg(bias), _stream_ptr(q.device),
         )
 
 
@@ -321,7 +354,7 @@ def _is_kernel_ready(x: torch.Tensor, elems_per_16b: int = 8) -> bool:
     return _kernel_ready(x, elems_per_16b) is x
 
 
-def _bitfield_attn_backward_overwrite(do, q, k, v, o, bitfield_mask, compressed_mask, lse, softmax_scale):
+def _bitfield_attn_backward_overwrite(do, q, k, v, o, bitfield_mask, compressed_mask, lse, softmax_scale, bias=None):
     """Gradients in the input dtype, written (not accumulated) by the kernels: what
     ``BitfieldAttentionFunction.backward`` needs, without the reference's zero-filled fp32
     staging buffers and the final cast (bitfield_attention.py:1248-1266).  Returns None when the
@@ -340,9 +373,11 @@ def _bitfield_attn_backward_overwrite(do, q, k, v, o, bitfield_mask, compressed_
     bf = bitfield_mask if bitfield_mask.stride(1) == 1 else bitfield_mask.contiguous()
     flags = compressed_mask if compressed_mask.stride(-1) == 1 else compressed_mask.contiguous()
     delta = torch.empty_like(lse)
+    batch, seqlen_q, nheads, _ = q.shape
+    bias_view = _BiasView(bias, q, batch, nheads, seqlen_q, k.shape[1], may_copy=False) if bias is not None else None
     _launch_bwd_preprocess(o, do, delta)
-    _launch_bwd_dkdv(q, k, v, do, lse, delta, dk, dv, bf, flags, softmax_scale, accumulate=False)
-    _launch_bwd_dq(q, k, v, do, lse, delta, dq, bf, flags, softmax_scale, accumulate=False)
+    _launch_bwd_dkdv(q, k, v, do, lse, delta, dk, dv, bf, flags, softmax_scale, accumulate=False, bias=bias_view)
+    _launch_bwd_dq(q, k, v, do, lse, delta, dq, bf, flags, softmax_scale, accumulate=False, bias=bias_view)
     return dq, dk, dv
 
 
@@ -376,7 +411,8 @@ def _bitfield_attn_backward(
     assert dq.stride(-1) == dk.stride(-1) == dv.stride(-1) == 1
     assert dq.dtype == dk.dtype == dv.dtype == torch.float32
     assert q.is_cuda
-    _check_unsupported(bias)
+    # the reference asserts the unit stride here instead of copying (bitfield_attention.py:1130)
+    bias_view = _BiasView(bias, q, batch, nheads, seqlen_q, seqlen_k, may_copy=False) if bias is not None else None
     view = None
     if offsets_q is not None or offsets_k is not None:
         view = _IndexView(bitfield_mask, offsets_q, offsets_k)
@@ -401,8 +437,8 @@ def _bitfield_attn_backward(
     delta = torch.empty_like(lse)
     wq, wk, wv = work
     _launch_bwd_preprocess(ok, gk, delta)
-    _launch_bwd_dkdv(qk, kk, vk, gk, lse, delta, wk, wv, bf, flags, softmax_scale)
-    _launch_bwd_dq(qk, kk, vk, gk, lse, delta, wq, bf, flags, softmax_scale)
+    _launch_bwd_dkdv(qk, kk, vk, gk, lse, delta, wk, wv, bf, flags, softmax_scale, bias=bias_view)
+    _launch_bwd_dq(qk, kk, vk, gk, lse, delta, wq, bf, flags, softmax_scale, bias=bias_view)
     # the kernels accumulated into `work`; hand the sums back if those were copies
     for dst, mid, w in zip((dq, dk, dv), acc, work):
         if dp != d:
@@ -428,6 +464,8 @@ class BitfieldAttentionFunction(torch.autograd.Function):
         bitfield_mask: (batch_size, seqlen) int64
         """
         q, k, v = [x if x.stride(-1) == 1 else x.contiguous() for x in [q, k, v]]
+        if bias is not None and bias.stride(-1) != 1:
+            bias = bias.contiguous()
 
         compressed_mask = BitfieldUtils.materialize_compressed_mask_from_bitfield_mask(bitfield_mask)
 
@@ -441,10 +479,11 @@ class BitfieldAttentionFunction(torch.autograd.Function):
     def backward(ctx, do: torch.Tensor):
         q, k, v, o, lse, bias, bitfield_mask, compressed_mask = ctx.saved_tensors
         assert not ctx.needs_input_grad[3], "the bitfield mask is not differentiable"
+        assert not ctx.needs_input_grad[4], "FlashAttention does not support bias gradient yet"
         with torch.no_grad():
             direct = _bitfield_attn_backward_overwrite(
-                do, q, k, v, o, bitfield_mask, compressed_mask, lse, ctx.softmax_scale
-            ) if bias is None else None
+                do, q, k, v, o, bitfield_mask, compressed_mask, lse, ctx.softmax_scale, bias=bias
+            )
             if direct is not None:
                 return (*direct, None, None, None)
             dq = torch.zeros_like(q, dtype=torch.float32)

@@ -57,6 +57,24 @@ typedef struct bam_index_view {
     int32_t Sk;
 } bam_index_view;
 
+/*
+ * Additive attention bias (`bias` of `_bitfield_attn_forward` / `_bitfield_attn_backward` and of the
+ * materialized-mask `_flash_attn_forward` / `_flash_attn_backward`; reference bitfield_attention.py:952-972,
+ * 321-329, 410-434, 815-835): the scores become scale * q k^T + bias before mask and softmax; the log-sum-exp
+ * includes it; it receives no gradient.  `ptr` is a logical (B, Hq, Sq, Sk) view with unit stride along the keys
+ * and element strides for batch, head and query row; a stride of 0 broadcasts, so the reference's "vector" form
+ * (.., 1, Sk) has stride_m == 0 and its "matrix" form (.., Sq, Sk) a real one.  Elements are fp32 (is_f32 != 0)
+ * or have the dtype of q.  Pointer alignment: one element.  Every attention entry point takes a
+ * `const bam_bias*` that may be null (no bias).  The struct lives in host memory.
+ */
+typedef struct bam_bias {
+    const void* ptr;
+    int64_t stride_b;
+    int64_t stride_h;
+    int64_t stride_m;
+    int32_t is_f32;
+} bam_bias;
+
 const char* bam_last_error(void);
 
 /* ABI version of this library (bumped on any signature change). */
@@ -110,7 +128,7 @@ int bam_fwd(const void* q, const void* k, const void* v, void* o, float* lse, co
             int64_t k_stride_b, int64_t k_stride_s, int64_t k_stride_h, int64_t v_stride_b,
             int64_t v_stride_s, int64_t v_stride_h, int64_t o_stride_b, int64_t o_stride_s,
             int64_t o_stride_h, int64_t bf_stride_b, int64_t flags_stride_b, int64_t flags_stride_m, int B,
-            int S, int Hq, int Hkv, int D, float scale, int dtype, void* stream);
+            int S, int Hq, int Hkv, int D, float scale, int dtype, const bam_bias* bias, void* stream);
 
 /*
  * Forward with index tensors (`offsets_q` / `offsets_k` of `_bitfield_attn_forward`,
@@ -124,7 +142,7 @@ int bam_fwd_indexed(const void* q, const void* k, const void* v, void* o, float*
                     int64_t k_stride_b, int64_t k_stride_s, int64_t k_stride_h, int64_t v_stride_b,
                     int64_t v_stride_s, int64_t v_stride_h, int64_t o_stride_b, int64_t o_stride_s,
                     int64_t o_stride_h, int64_t flags_stride_b, int64_t flags_stride_m, int B, int Hq, int Hkv,
-                    int D, float scale, int dtype, void* stream);
+                    int D, float scale, int dtype, const bam_bias* bias, void* stream);
 
 /*
  * delta[b,h,i] = sum_d o[b,i,h,d] * do[b,i,h,d] in fp32.  Replaces
@@ -153,7 +171,7 @@ int bam_bwd(const void* q, const void* k, const void* v, const void* dout, const
             int64_t dq_stride_b, int64_t dq_stride_s, int64_t dq_stride_h, int64_t dk_stride_b,
             int64_t dk_stride_s, int64_t dk_stride_h, int64_t dv_stride_b, int64_t dv_stride_s,
             int64_t dv_stride_h, int64_t bf_stride_b, int64_t flags_stride_b, int64_t flags_stride_m, int B,
-            int S, int Hq, int Hkv, int D, float scale, int dtype, int accumulate, void* stream);
+            int S, int Hq, int Hkv, int D, float scale, int dtype, int accumulate, const bam_bias* bias, void* stream);
 
 /*
  * The two halves of bam_bwd as separate launches (same reference kernel,
@@ -170,7 +188,7 @@ int bam_bwd_dkdv(const void* q, const void* k, const void* v, const void* dout, 
                  int64_t dk_stride_b, int64_t dk_stride_s, int64_t dk_stride_h, int64_t dv_stride_b,
                  int64_t dv_stride_s, int64_t dv_stride_h, int64_t bf_stride_b, int64_t flags_stride_b,
                  int64_t flags_stride_m, int B, int S, int Hq, int Hkv, int D, float scale, int dtype,
-                 int accumulate, void* stream);
+                 int accumulate, const bam_bias* bias, void* stream);
 
 int bam_bwd_dq(const void* q, const void* k, const void* v, const void* dout, const float* lse,
                const float* delta, void* dq, const int64_t* bf, const int8_t* flags, int64_t q_stride_b,
@@ -179,7 +197,7 @@ int bam_bwd_dq(const void* q, const void* k, const void* v, const void* dout, co
                int64_t do_stride_b, int64_t do_stride_s, int64_t do_stride_h, int64_t dq_stride_b,
                int64_t dq_stride_s, int64_t dq_stride_h, int64_t bf_stride_b, int64_t flags_stride_b,
                int64_t flags_stride_m, int B, int S, int Hq, int Hkv, int D, float scale, int dtype,
-               int accumulate, void* stream);
+               int accumulate, const bam_bias* bias, void* stream);
 
 /*
  * bam_bwd_dkdv / bam_bwd_dq with index tensors (`offsets_q` / `offsets_k` of
@@ -194,7 +212,7 @@ int bam_bwd_dkdv_indexed(const void* q, const void* k, const void* v, const void
                          int64_t v_stride_h, int64_t do_stride_b, int64_t do_stride_s, int64_t do_stride_h,
                          int64_t dk_stride_b, int64_t dk_stride_s, int64_t dk_stride_h, int64_t dv_stride_b,
                          int64_t dv_stride_s, int64_t dv_stride_h, int64_t flags_stride_b, int64_t flags_stride_m,
-                         int B, int Hq, int Hkv, int D, float scale, int dtype, int accumulate, void* stream);
+                         int B, int Hq, int Hkv, int D, float scale, int dtype, int accumulate, const bam_bias* bias, void* stream);
 
 int bam_bwd_dq_indexed(const void* q, const void* k, const void* v, const void* dout, const float* lse,
                        const float* delta, void* dq, const bam_index_view* iv, const int8_t* flags,
@@ -203,7 +221,7 @@ int bam_bwd_dq_indexed(const void* q, const void* k, const void* v, const void* 
                        int64_t v_stride_h, int64_t do_stride_b, int64_t do_stride_s, int64_t do_stride_h,
                        int64_t dq_stride_b, int64_t dq_stride_s, int64_t dq_stride_h, int64_t flags_stride_b,
                        int64_t flags_stride_m, int B, int Hq, int Hkv, int D, float scale, int dtype,
-                       int accumulate, void* stream);
+                       int accumulate, const bam_bias* bias, void* stream);
 
 /*
  * Materialized-mask attention: the sibling path of the reference,
@@ -224,7 +242,7 @@ int bam_fwd_masked(const void* q, const void* k, const void* v, void* o, float* 
                    int64_t k_stride_b, int64_t k_stride_s, int64_t k_stride_h, int64_t v_stride_b,
                    int64_t v_stride_s, int64_t v_stride_h, int64_t o_stride_b, int64_t o_stride_s,
                    int64_t o_stride_h, int64_t flags_stride_b, int64_t flags_stride_m, int B, int Sq, int Sk, int Hq,
-                   int Hkv, int D, float scale, int dtype, void* stream);
+                   int Hkv, int D, float scale, int dtype, const bam_bias* bias, void* stream);
 
 int bam_bwd_dkdv_masked(const void* q, const void* k, const void* v, const void* dout, const float* lse,
                         const float* delta, void* dk, void* dv, const uint8_t* mask, const int8_t* flags,
@@ -234,7 +252,7 @@ int bam_bwd_dkdv_masked(const void* q, const void* k, const void* v, const void*
                         int64_t dk_stride_b, int64_t dk_stride_s, int64_t dk_stride_h, int64_t dv_stride_b,
                         int64_t dv_stride_s, int64_t dv_stride_h, int64_t flags_stride_b, int64_t flags_stride_m,
                         int B, int Sq, int Sk, int Hq, int Hkv, int D, float scale, int dtype, int accumulate,
-                        void* stream);
+                        const bam_bias* bias, void* stream);
 
 int bam_bwd_dq_masked(const void* q, const void* k, const void* v, const void* dout, const float* lse,
                       const float* delta, void* dq, const uint8_t* mask, const int8_t* flags, int64_t q_stride_b,
@@ -242,7 +260,7 @@ int bam_bwd_dq_masked(const void* q, const void* k, const void* v, const void* d
                       int64_t k_stride_h, int64_t v_stride_b, int64_t v_stride_s, int64_t v_stride_h,
                       int64_t do_stride_b, int64_t do_stride_s, int64_t do_stride_h, int64_t dq_stride_b,
                       int64_t dq_stride_s, int64_t dq_stride_h, int64_t flags_stride_b, int64_t flags_stride_m, int B,
-                      int Sq, int Sk, int Hq, int Hkv, int D, float scale, int dtype, int accumulate, void* stream);
+                      int Sq, int Sk, int Hq, int Hkv, int D, float scale, int dtype, int accumulate, const bam_bias* bias, void* stream);
 
 #ifdef __cplusplus
 }

@@ -34,6 +34,10 @@ What pins each function (the pins live in ``tests/test_oracle.py``):
   reference's ``flash_attn_func``) -- library SDPA with the same ``attn_mask`` and autograd through it,
   which is what the reference's test compares against (``tests/test_kernel/test_attention.py``);
   ``mask_tile_flags`` -- brute-force classification of random masks.
+* ``bias`` of the four attention functions -- library SDPA with the float ``attn_mask`` = bias, -inf
+  where the pair is not allowed (forward and autograd through it); closed forms: a bias that is
+  constant along the keys leaves o unchanged and shifts lse by that constant, and bias = log w
+  turns the softmax into the w-weighted one.
 * ``create_bitfield_attention_mask`` -- golden vectors of
   ``tests/test_models/test_multimodal_merge_outputs.py:94-110``.
 
@@ -199,15 +203,18 @@ def attention_sdpa(q, k, v, bitfield, softmax_scale=None):
     return torch.where(dead.transpose(1, 2).unsqueeze(-1), torch.zeros_like(o), o)
 
 
-def _chunk_forward(qc, kb, vb, allow, scale):
+def _chunk_forward(qc, kb, vb, allow, scale, bias=None):
     """qc (rows,Hq,D), kb/vb (S,Hkv,D), allow (rows,S) -> o (rows,Hq,D), lse (Hq,rows).
-    s = scale * q.k ; lse = log sum_allowed exp(s) ; o = sum_allowed exp(s-lse) v
-    (bitfield_attention.py:389-390,435-495); GQA h -> h // (Hq//Hkv) (:292-293)."""
+    s = scale * q.k (+ bias) ; lse = log sum_allowed exp(s) ; o = sum_allowed exp(s-lse) v
+    (bitfield_attention.py:389-390,410-434,435-495); GQA h -> h // (Hq//Hkv) (:292-293).
+    ``bias`` broadcasts against (Hq, rows, S)."""
     Hq, Hkv = qc.shape[1], kb.shape[1]
     g = Hq // Hkv
     kk = kb.repeat_interleave(g, dim=1) if g > 1 else kb
     vv = vb.repeat_interleave(g, dim=1) if g > 1 else vb
     s = torch.einsum("ihd,jhd->hij", qc, kk) * scale
+    if bias is not None:
+        s = s + bias.to(s.dtype)
     s = s.masked_fill(~allow[None], float("-inf"))
     lse = torch.logsumexp(s, dim=-1)  # -inf where nothing is allowed
     p = torch.exp(s - torch.where(torch.isinf(lse), torch.zeros_like(lse), lse)[..., None])
@@ -215,12 +222,22 @@ def _chunk_forward(qc, kb, vb, allow, scale):
     return o, lse
 
 
+def _bias_rows(bias, b, r0, r1):
+    """Rows r0..r1 of batch b of a bias broadcastable to (B, Hq, Sq, Sk) -> broadcastable to (Hq, rows, Sk)
+    (indexed by LOCAL row / key like the reference, bitfield_attention.py:321-329)."""
+    if bias is None:
+        return None
+    bb = bias[b if bias.shape[0] > 1 else 0]
+    return bb[:, r0:r1] if bb.shape[1] > 1 else bb
+
+
 def attention_forward(q, k, v, bitfield, softmax_scale=None, row_chunk=1024, dtype=torch.float32,
-                      idx_q=None, idx_k=None):
+                      idx_q=None, idx_k=None, bias=None):
     """Explicit masked softmax attention -> (o (B,S,Hq,D), lse (B,Hq,S)) in ``dtype``.
     With index tensors q holds the rows at global positions ``idx_q`` and k/v the keys at
     ``idx_k`` (any order); ``bitfield`` stays indexed by global position
-    (bitfield_attention.py:71-87)."""
+    (bitfield_attention.py:71-87).  ``bias``: 4-d, broadcastable to (B, Hq, S, S), added to the
+    scaled scores (bitfield_attention.py:410-434)."""
     B, S, Hq, D = q.shape
     scale = softmax_scale or 1.0 / math.sqrt(D)
     q, k, v = q.to(dtype), k.to(dtype), v.to(dtype)
@@ -230,14 +247,14 @@ def attention_forward(q, k, v, bitfield, softmax_scale=None, row_chunk=1024, dty
         for r0 in range(0, S, row_chunk):
             r1 = min(r0 + row_chunk, S)
             allow = allow_rows(bitfield[b], r0, r1, idx_q, idx_k)
-            oc, lc = _chunk_forward(q[b, r0:r1], k[b], v[b], allow, scale)
+            oc, lc = _chunk_forward(q[b, r0:r1], k[b], v[b], allow, scale, _bias_rows(bias, b, r0, r1))
             o[b, r0:r1] = oc
             lse[b, :, r0:r1] = lc
     return o, lse
 
 
 def attention_backward(q, k, v, bitfield, do, softmax_scale=None, row_chunk=1024, dtype=torch.float32,
-                       idx_q=None, idx_k=None):
+                       idx_q=None, idx_k=None, bias=None):
     """dq, dk, dv of sum(o * do) by autograd through the explicit forward, one row
     chunk at a time (bounded memory).  Matches the reference's gradient contract
     (bitfield_attention.py:840-886): dk/dv are summed over the q-heads of a group."""
@@ -254,7 +271,7 @@ def attention_backward(q, k, v, bitfield, do, softmax_scale=None, row_chunk=1024
             qc = q[b, r0:r1].detach().requires_grad_(True)
             kb = k[b].detach().requires_grad_(True)
             vb = v[b].detach().requires_grad_(True)
-            oc, _ = _chunk_forward(qc, kb, vb, allow, scale)
+            oc, _ = _chunk_forward(qc, kb, vb, allow, scale, _bias_rows(bias, b, r0, r1))
             gq, gk, gv = torch.autograd.grad(oc, (qc, kb, vb), do[b, r0:r1])
             dq[b, r0:r1] = gq
             dk[b] += gk
@@ -262,7 +279,7 @@ def attention_backward(q, k, v, bitfield, do, softmax_scale=None, row_chunk=1024
     return dq, dk, dv
 
 
-def masked_attention_forward(q, k, v, mask, softmax_scale=None, dtype=torch.float32):
+def masked_attention_forward(q, k, v, mask, softmax_scale=None, dtype=torch.float32, bias=None):
     """Attention with a materialized bool mask (B, Sq, Sk) (None: attend everywhere), the contract of
     the reference's ``flash_attn_func`` (cornstarch/kernel/attention.py:184-232: pairs whose mask
     byte is False get -inf before the softmax) -> (o (B,Sq,Hq,D), lse (B,Hq,Sq))."""
@@ -274,15 +291,15 @@ def masked_attention_forward(q, k, v, mask, softmax_scale=None, dtype=torch.floa
     lse = torch.empty((B, Hq, Sq), dtype=dtype, device=q.device)
     for b in range(B):
         allow = mask[b] if mask is not None else torch.ones((Sq, Sk), dtype=torch.bool, device=q.device)
-        o[b], lse[b] = _chunk_forward(q[b], k[b], v[b], allow, scale)
+        o[b], lse[b] = _chunk_forward(q[b], k[b], v[b], allow, scale, _bias_rows(bias, b, 0, Sq))
     return o, lse
 
 
-def masked_attention_backward(q, k, v, mask, do, softmax_scale=None, dtype=torch.float32):
+def masked_attention_backward(q, k, v, mask, do, softmax_scale=None, dtype=torch.float32, bias=None):
     """dq, dk, dv of sum(o * do) for ``masked_attention_forward`` by autograd."""
     q, k, v, do = (t.to(dtype) for t in (q, k, v, do))
     qr, kr, vr = (t.detach().requires_grad_(True) for t in (q, k, v))
-    o, _ = masked_attention_forward(qr, kr, vr, mask, softmax_scale, dtype)
+    o, _ = masked_attention_forward(qr, kr, vr, mask, softmax_scale, dtype, bias)
     return torch.autograd.grad(o, (qr, kr, vr), do)
 
 

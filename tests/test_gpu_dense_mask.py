@@ -100,5 +100,5 @@ def test_private_entry_points_and_hf_adapter():
         assert rel_l2(got.float().cpu(), w) <= GRAD_REL_L2
     out, none = interface.cornstarch_attention_forward(None, q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), mask)
     assert none is None and torch.equal(out, o)
-    with pytest.raises(NotImplementedError):
-        A.flash_attn_func(q, k, v, bias=torch.zeros(1, 4, 1, 144, device=d))
+    with pytest.raises(RuntimeError):  # reference attention.py:886-890
+        A.flash_attn_func(q, k, v, bias=torch.zeros(1, 4, 3, 144, device=d))

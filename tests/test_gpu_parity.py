@@ -295,8 +295,9 @@ def test_backward_accumulates_into_caller_buffers():
     BA._bitfield_attn_backward(do, q, k, v, o, bfg, flags, lse, *ones)
     for a, b in zip(z, ones):
         assert torch.allclose(a + 1, b, atol=1e-6)
-    with pytest.raises(NotImplementedError):
-        BA._bitfield_attn_forward(q, k, v, bfg, flags, bias=torch.zeros(1, 2, 1, 256, device=d))
+    # a bias of the wrong shape is the reference's RuntimeError (bitfield_attention.py:964-968)
+    with pytest.raises(RuntimeError):
+        BA._bitfield_attn_forward(q, k, v, bfg, flags, bias=torch.zeros(1, 2, 2, 256, device=d))
     # identity index tensors change nothing
     ar = torch.arange(256, device=d)
     o2, lse2, _ = BA._bitfield_attn_forward(q, k, v, bfg, flags, offsets_q=ar, offsets_k=ar)

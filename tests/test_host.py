@@ -47,15 +47,22 @@ def test_abi_rejects_bad_arguments_without_touching_the_gpu():
     # null pointers / unsupported head dim are refused before any HIP call
     rc = lib.bam_tile_flags(None, 0, None, 0, 0, 1, 128, None)
     assert rc == -1 and b"null" in lib.bam_last_error()
-    args = [ctypes.c_void_p(16)] * 7 + [8] * 15 + [1, 128, 4, 4, 48] + [0.125, 1, None]
+    args = [ctypes.c_void_p(16)] * 7 + [8] * 15 + [1, 128, 4, 4, 48] + [0.125, 1, None, None]
     rc = lib.bam_fwd(*args)
     assert rc == -2 and b"head dimension 48" in lib.bam_last_error()
-    args = [ctypes.c_void_p(16)] * 7 + [8] * 15 + [1, 128, 6, 4, 64] + [0.125, 1, None]
+    args = [ctypes.c_void_p(16)] * 7 + [8] * 15 + [1, 128, 6, 4, 64] + [0.125, 1, None, None]
     assert lib.bam_fwd(*args) == -1 and b"multiple of Hkv" in lib.bam_last_error()
-    args = [ctypes.c_void_p(8)] + [ctypes.c_void_p(16)] * 6 + [8] * 15 + [1, 128, 4, 4, 64] + [0.125, 1, None]
+    args = [ctypes.c_void_p(8)] + [ctypes.c_void_p(16)] * 6 + [8] * 15 + [1, 128, 4, 4, 64] + [0.125, 1, None, None]
     assert lib.bam_fwd(*args) == -1 and b"16-byte aligned" in lib.bam_last_error()
-    args = [ctypes.c_void_p(16)] * 7 + [8] * 15 + [1, 128, 4, 4, 64] + [-1.0, 1, None]
+    args = [ctypes.c_void_p(16)] * 7 + [8] * 15 + [1, 128, 4, 4, 64] + [-1.0, 1, None, None]
     assert lib.bam_fwd(*args) == -1 and b"scale" in lib.bam_last_error()
+    # a bias descriptor without a pointer, or with a pointer that is not a multiple of its element size
+    bias = _bam_hip.Bias(None, 0, 0, 0, 1)
+    args = [ctypes.c_void_p(16)] * 7 + [8] * 15 + [1, 128, 4, 4, 64] + [0.125, 1, ctypes.byref(bias), None]
+    assert lib.bam_fwd(*args) == -1 and b"bias" in lib.bam_last_error()
+    bias = _bam_hip.Bias(18, 0, 0, 0, 1)
+    args = [ctypes.c_void_p(16)] * 7 + [8] * 15 + [1, 128, 4, 4, 64] + [0.125, 1, ctypes.byref(bias), None]
+    assert lib.bam_fwd(*args) == -1 and b"bias" in lib.bam_last_error()
     with pytest.raises(_bam_hip.BamError):
         _bam_hip.call("bam_materialize_mask", None, 0, None, 1, 8, None)
 

@@ -333,3 +333,58 @@ def test_dense_mask_tile_flags_against_loops():
                 want = 0 if not t.any() else 2 if t.all() else 1
                 assert got[b, m, n] == want
     assert got[0, 0, 0] == 2 and got[0, 1, 1] == 0 and got[0, 2, 5] == 2
+
+
+# ------------------------------------------------------------------ additive bias
+@pytest.mark.parametrize("kind", ["vector", "matrix", "matrix_per_batch"])
+def test_bias_against_library_sdpa_with_float_mask(kind):
+    # SDPA adds a float attn_mask to the scaled scores: bias where the pair is allowed, -inf elsewhere
+    B, S, Hq, Hkv, D = 2, 150, 4, 2, 16
+    g = torch.Generator().manual_seed(11)
+    q = torch.randn(B, S, Hq, D, generator=g, dtype=torch.float64) * 0.5
+    k = torch.randn(B, S, Hkv, D, generator=g, dtype=torch.float64) * 0.5
+    v = torch.randn(B, S, Hkv, D, generator=g, dtype=torch.float64) * 0.5
+    do = torch.randn(B, S, Hq, D, generator=g, dtype=torch.float64)
+    shape = {"vector": (1, Hq, 1, S), "matrix": (1, Hq, S, S), "matrix_per_batch": (B, 1, S, S)}[kind]
+    bias = torch.randn(shape, generator=g, dtype=torch.float64)
+    bf, allow = reference_test_bitfield(B, S)
+    fmask = torch.where(allow.unsqueeze(1), bias.expand(B, Hq, S, S), torch.full((), float("-inf"), dtype=torch.float64))
+    qr, kr, vr = (t.clone().requires_grad_(True) for t in (q, k, v))
+    ref = F.scaled_dot_product_attention(
+        qr.transpose(1, 2), kr.transpose(1, 2), vr.transpose(1, 2), attn_mask=fmask, enable_gqa=True
+    ).transpose(1, 2)
+    o, lse = O.attention_forward(q, k, v, bf, dtype=torch.float64, bias=bias, row_chunk=64)
+    assert torch.allclose(o, ref, atol=1e-10, rtol=0)
+    kk = k.repeat_interleave(Hq // Hkv, dim=2)
+    s = torch.einsum("bihd,bjhd->bhij", q, kk) / math.sqrt(D) + fmask
+    assert torch.allclose(lse, torch.logsumexp(s, dim=-1), atol=1e-10, rtol=0)
+    want = torch.autograd.grad(ref, (qr, kr, vr), do)
+    got = O.attention_backward(q, k, v, bf, do, dtype=torch.float64, bias=bias, row_chunk=64)
+    for a, b_ in zip(got, want):
+        assert torch.allclose(a, b_, atol=1e-10, rtol=0)
+    # the materialized-mask functions take the same bias
+    o2, lse2 = O.masked_attention_forward(q, k, v, allow, dtype=torch.float64, bias=bias)
+    assert torch.allclose(o2, ref, atol=1e-10, rtol=0) and torch.allclose(lse2, lse, atol=1e-10, rtol=0)
+    got2 = O.masked_attention_backward(q, k, v, allow, do, dtype=torch.float64, bias=bias)
+    for a, b_ in zip(got2, want):
+        assert torch.allclose(a, b_, atol=1e-10, rtol=0)
+
+
+def test_bias_closed_forms():
+    B, S, H, D = 1, 96, 2, 8
+    g = torch.Generator().manual_seed(12)
+    q, k, v = (torch.randn(B, S, H, D, generator=g, dtype=torch.float64) for _ in range(3))
+    bf, _ = reference_test_bitfield(B, S)
+    o0, lse0 = O.attention_forward(q, k, v, bf, dtype=torch.float64)
+    # constant along the keys: softmax unchanged, lse shifted by the constant
+    c = torch.randn(B, H, S, 1, generator=g, dtype=torch.float64)
+    o1, lse1 = O.attention_forward(q, k, v, bf, dtype=torch.float64, bias=c.expand(B, H, S, S))
+    assert torch.allclose(o1, o0, atol=1e-12, rtol=0)
+    assert torch.allclose(lse1, lse0 + c[..., 0], atol=1e-12, rtol=0)
+    # bias = log w on zero queries: o = sum_j w_j v_j / sum_j w_j over the allowed keys
+    w = torch.rand(1, H, 1, S, generator=g, dtype=torch.float64) + 0.1
+    o2, _ = O.attention_forward(torch.zeros_like(q), k, v, bf, dtype=torch.float64, bias=w.log())
+    allow = O.materialize_mask(bf)[0].to(torch.float64)  # (S, S)
+    ww = allow[None] * w[0, :, 0][:, None, :]  # (H, S, S)
+    want = torch.einsum("hij,jhd->ihd", ww / ww.sum(-1, keepdim=True), v[0])
+    assert torch.allclose(o2[0], want, atol=1e-12, rtol=0)
