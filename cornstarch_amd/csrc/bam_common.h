@@ -86,6 +86,11 @@ struct BF16 {
     static __device__ __forceinline__ float to_float(unsigned short raw) {
         return __builtin_bit_cast(float, ((unsigned)raw) << 16);
     }
+    // acc + the two elements of a packed pair
+    static __device__ __forceinline__ float add_pair(unsigned packed, float acc) {
+        typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, packed), __builtin_bit_cast(bf16x2, 0x3F803F80u), acc, false);
+    }
 };
 
 struct F16 {
@@ -102,6 +107,10 @@ struct F16 {
     }
     static __device__ __forceinline__ float to_float(unsigned short raw) {
         return (float)__builtin_bit_cast(_Float16, raw);
+    }
+    static __device__ __forceinline__ float add_pair(unsigned packed, float acc) {
+        typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+        return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, packed), __builtin_bit_cast(f16x2, 0x3C003C00u), acc, false);
     }
 };
 

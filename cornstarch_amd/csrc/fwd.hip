@@ -250,7 +250,7 @@ __global__ __launch_bounds__(FWD_THREADS, D == 128 ? 2 : 3) void fwd_kernel(cons
         // ---- online softmax (per-lane scalars) ----------------------------------------------
         float mloc = fmaxf(s[0][0], s[1][0]);
 #pragma unroll
-        for (int i = 1; i < 16; ++i) mloc = fmaxf(mloc, fmaxf(s[0][i], s[1][i]));
+        for (int i = 1; i < 16; ++i) mloc = fmaxf(fmaxf(mloc, s[0][i]), s[1][i]);
         mloc = half_swap_max(mloc);
         if (__any(mloc > m_i + rescale_thr)) {  // wave-uniform; rare after the first tiles
             const float mnew = fmaxf(m_i, mloc);
@@ -264,23 +264,27 @@ __global__ __launch_bounds__(FWD_THREADS, D == 128 ? 2 : 3) void fwd_kernel(cons
 #pragma unroll
                 for (int i = 0; i < 16; ++i) o[db][i] *= alpha;
         }
-        float psum0 = 0.f, psum1 = 0.f;
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-            const float e0 = __builtin_amdgcn_exp2f(fmaf(s[0][i], c2, nb));
-            const float e1 = __builtin_amdgcn_exp2f(fmaf(s[1][i], c2, nb));
-            s[0][i] = e0;
-            s[1][i] = e1;
-            psum0 += e0;
-            psum1 += e1;
+            s[0][i] = __builtin_amdgcn_exp2f(fmaf(s[0][i], c2, nb));
+            s[1][i] = __builtin_amdgcn_exp2f(fmaf(s[1][i], c2, nb));
         }
-        l_i += psum0 + psum1;
-
         u32x4 pb[2][2];
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
             for (int t = 0; t < 2; ++t) pb[kb][t] = pack8<T>(s[kb], 8 * t);
+        // row sum of the probabilities as the P V product sees them (rounded to T), two per instruction
+        {
+            float ps[2][2] = {{0.f, 0.f}, {0.f, 0.f}};
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+#pragma unroll
+                    for (int x = 0; x < 4; ++x) ps[kb][t] = T::add_pair(pb[kb][t][x], ps[kb][t]);
+            l_i += (ps[0][0] + ps[0][1]) + (ps[1][0] + ps[1][1]);
+        }
 
         // ---- O^T += V^T P^T -------------------------------------------------------------------
         {
