@@ -13,7 +13,7 @@ namespace bam {
 // tile lies inside the sequence) the class follows from one evaluation of the bit test plus the
 // position of the tile relative to the diagonal; long runs of equal bitfields are the common case.
 constexpr int FLAG_WAVES = 4;
-constexpr int FLAG_TILES_PER_WAVE = 8;
+constexpr int FLAG_TILES_PER_WAVE = 2;  // few tiles per wave: the grid, not the wave, covers the row of tiles
 constexpr int FLAG_COLS_PER_BLOCK = FLAG_WAVES * FLAG_TILES_PER_WAVE;
 
 __global__ __launch_bounds__(FLAG_WAVES * 64) void tile_flags_kernel(const int64_t* __restrict__ bf,
@@ -34,11 +34,19 @@ __global__ __launch_bounds__(FLAG_WAVES * 64) void tile_flags_kernel(const int64
     const int half = lane >> 5;
     const int64_t q0 = q_bits[0];
     const bool rows_uniform = rows_in_range == BLOCK_M && __all(q_bits[lane] == q0 && q_bits[lane + 64] == q0);
+    // the key bitfields of all tiles of this wave, requested together (one memory latency instead of one per tile)
+    int64_t kfs[FLAG_TILES_PER_WAVE];
+#pragma unroll
+    for (int t = 0; t < FLAG_TILES_PER_WAVE; ++t) {
+        const int j = (blockIdx.x * FLAG_COLS_PER_BLOCK + wave * FLAG_TILES_PER_WAVE + t) * BLOCK_N + (lane & 31);
+        kfs[t] = (j < S) ? row[j] : 0;
+    }
+#pragma unroll
     for (int t = 0; t < FLAG_TILES_PER_WAVE; ++t) {
         const int n = blockIdx.x * FLAG_COLS_PER_BLOCK + wave * FLAG_TILES_PER_WAVE + t;
         if (n >= num_n) break;  // wave-uniform
         const int j = n * BLOCK_N + (lane & 31);
-        const int64_t kf = (j < S) ? row[j] : 0;
+        const int64_t kf = kfs[t];
         if (rows_uniform && (n + 1) * BLOCK_N <= S) {
             const unsigned klo = __builtin_amdgcn_readfirstlane((unsigned)kf);
             const unsigned khi = __builtin_amdgcn_readfirstlane((unsigned)((uint64_t)kf >> 32));
