@@ -11,6 +11,7 @@ Cases (all fp16 inputs so that the file stores them exactly):
   gqa_pad   : B1 S96 Hq4 Hkv2 D32, irregular segments, 7 padding tokens (bitfield 0), modality bits above 31
   zigzag    : B1 S160 Hq2 Hkv1 D32 split zigzag over two ranks (index tensors), rank 1 stored
   dense     : B1 Sq70 Sk45 H2 D32, materialized bool mask with a dead row
+  bias      : B1 S80 Hq2 Hkv1 D32, bitfield of the reference's test, fp32 matrix bias (1, 2, 80, 80)
 """
 
 import os
@@ -78,6 +79,13 @@ def build():
     o, lse = O.masked_attention_forward(q, k, v, mask)
     pack(out, "dense", q, k, v, do, o, lse, O.masked_attention_backward(q, k, v, mask, do), mask=mask,
          flags=O.mask_tile_flags(mask))
+    # bias
+    bf, _ = reference_test_bitfield(1, 80)
+    q, k, v, do = tensors(1, 80, 80, 2, 1, 32, seed=15)
+    bias = torch.randn(1, 2, 80, 80, generator=torch.Generator().manual_seed(16))
+    o, lse = O.attention_forward(q, k, v, bf, bias=bias)
+    pack(out, "bias", q, k, v, do, o, lse, O.attention_backward(q, k, v, bf, do, bias=bias), bf=bf, bias=bias,
+         flags=O.tile_flags(bf))
     return out
 
 

@@ -96,3 +96,21 @@ def test_dense_mask_attention_matches_golden():
     dq, dk, dv = torch.autograd.grad(o, (q, k, v), g["do"].to(d))
     _, lse, _ = A._flash_attn_forward(q.detach(), k.detach(), v.detach(), mask=mask)
     _compare(g, o.detach(), lse, dq, dk, dv)
+
+
+@pytest.mark.gpu
+def test_attention_with_bias_matches_golden():
+    from cornstarch_amd.kernel import bitfield_attention as BA
+
+    d = torch.device("cuda:0")
+    g = load("bias")
+    bf, bias = g["bf"].to(d), g["bias"].to(d)
+    BA.BitfieldUtils.clear_cache()
+    flags = BA.BitfieldUtils.materialize_compressed_mask_from_bitfield_mask(bf)
+    assert torch.equal(flags.cpu(), g["flags"])
+    q, k, v = (g[n].to(d).requires_grad_(True) for n in ("q", "k", "v"))
+    o = BA.bitfield_attn_func(q, k, v, bf, bias)
+    dq, dk, dv = torch.autograd.grad(o, (q, k, v), g["do"].to(d))
+    _, lse, _ = BA._bitfield_attn_forward(q.detach(), k.detach(), v.detach(), bf, flags, bias=bias)
+    _compare(g, o.detach(), lse, dq, dk, dv)
+    BA.BitfieldUtils.clear_cache()
