@@ -304,6 +304,46 @@ def test_backward_accumulates_into_caller_buffers():
     assert torch.equal(o2, o) and torch.equal(lse2, lse)
 
 
+@pytest.mark.parametrize("accumulate", [1, 0], ids=["fp32_accumulate", "typed_overwrite"])
+def test_combined_backward_entry_point(accumulate):
+    # bam_bwd = dK/dV and dQ in one call; the host functions use the two separate entry points, so this one is
+    # called here directly, with and without a bias descriptor, and compared with them bit for bit
+    import ctypes
+
+    from cornstarch_amd.kernel import _bam_hip
+
+    d = dev()
+    B, S, Hq, Hkv, D = 2, 200, 4, 2, 64
+    bf = random_bitfield(B, S, seed=61).to(d)
+    q, k, v, do = (t.to(d) for t in make_inputs(B, S, Hq, Hkv, D, torch.bfloat16, seed=62))
+    flags = flags_of(bf)
+    bias = torch.randn(1, Hq, 1, S, device=d)
+    for bias_t in (None, bias):
+        o, lse, sc = BA._bitfield_attn_forward(q, k, v, bf, flags, bias=bias_t)
+        delta = torch.empty_like(lse)
+        BA._launch_bwd_preprocess(o, do, delta)
+        gdt = torch.float32 if accumulate else q.dtype
+        want = [torch.zeros(t.shape, dtype=gdt, device=d) for t in (q, k, v)]
+        bview = BA._BiasView(bias_t, q, B, Hq, S, S) if bias_t is not None else None
+        BA._launch_bwd_dkdv(q, k, v, do, lse, delta, want[1], want[2], bf, flags, sc, accumulate=bool(accumulate), bias=bview)
+        BA._launch_bwd_dq(q, k, v, do, lse, delta, want[0], bf, flags, sc, accumulate=bool(accumulate), bias=bview)
+        got = [torch.zeros(t.shape, dtype=gdt, device=d) for t in (q, k, v)]
+        _bam_hip.call(
+            "bam_bwd", q.data_ptr(), k.data_ptr(), v.data_ptr(), do.data_ptr(), lse.data_ptr(), delta.data_ptr(),
+            got[0].data_ptr(), got[1].data_ptr(), got[2].data_ptr(), bf.data_ptr(), flags.data_ptr(),
+            *BA._strides3(q, k, v, do, *got), bf.stride(0), flags.stride(0), flags.stride(1),
+            B, S, Hq, Hkv, D, float(sc), BA._dtype_code(q.dtype), accumulate,
+            bview.byref() if bview is not None else None, BA._stream_ptr(d),
+        )
+        torch.cuda.synchronize()
+        for a, b in zip(got, want):
+            assert torch.equal(a, b)
+        wq, wk, wv = O.attention_backward(q.cpu(), k.cpu(), v.cpu(), bf.cpu(), do.cpu(),
+                                          bias=bias_t.cpu() if bias_t is not None else None)
+        for a, w in zip(got, (wq, wk, wv)):
+            assert rel_l2(a.float().cpu(), w) <= GRAD_REL_L2
+
+
 # -------------------------------------------------- the five benchmark configurations
 def _oracle_on_device(q, k, v, do, bf, row_chunk):
     o, lse = O.attention_forward(q, k, v, bf, row_chunk=row_chunk)
