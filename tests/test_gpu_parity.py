@@ -397,3 +397,38 @@ def test_full_size_configs_against_fp32_library_math(name, row_chunk):
     assert worst_lse <= 1e-2, worst_lse
     for key in num:
         assert math.sqrt(num[key] / den[key]) <= GRAD_REL_L2, (key, math.sqrt(num[key] / den[key]))
+
+
+def test_maximum_sequence_length_and_one_beyond():
+    # S = 131072 is the longest sequence the tile lists hold; the oracle runs as fp32 library math on the device
+    from cornstarch_amd.kernel import _bam_hip
+
+    S, Hq, Hkv, D = _bam_hip.BAM_MAX_SEQLEN, 2, 1, 32
+    d = dev()
+    g = torch.Generator().manual_seed(77)
+    q = (torch.randn(1, S, Hq, D, generator=g) * 0.5).to(torch.bfloat16).to(d)
+    k = (torch.randn(1, S, Hkv, D, generator=g) * 0.5).to(torch.bfloat16).to(d)
+    v = (torch.randn(1, S, Hkv, D, generator=g) * 0.5).to(torch.bfloat16).to(d)
+    do = torch.randn(1, S, Hq, D, generator=g).to(torch.bfloat16).to(d)
+    text = (1 << 62) | 1 | 2 | 4
+    bf = torch.full((1, S), text, dtype=torch.int64)
+    bf[0, 1000:5000] = 2        # two modality segments, the second one ends with the sequence
+    bf[0, S - 3000:] = 4
+    bf = bf.to(d)
+    flags = flags_of(bf)
+    assert torch.equal(flags.cpu(), O.tile_flags(bf.cpu()))
+    qg, kg, vg = (t.clone().requires_grad_(True) for t in (q, k, v))
+    o = BA.bitfield_attn_func(qg, kg, vg, bf)
+    dq, dk, dv = torch.autograd.grad(o, (qg, kg, vg), do)
+    o_r, lse_r, gq, gk, gv = _oracle_on_device(q, k, v, do, bf, 512)
+    assert (o.detach().float() - o_r).abs().max().item() <= O_MAX_ABS
+    for got, want in ((dq, gq), (dk, gk), (dv, gv)):
+        assert rel_l2(got.float(), want) <= GRAD_REL_L2
+    BA.BitfieldUtils.clear_cache()
+    # one token more is refused with a clear error, before anything is launched
+    S1 = S + 1
+    q1 = torch.zeros(1, S1, 1, 32, dtype=torch.bfloat16, device=d)
+    bf1 = torch.full((1, S1), text, dtype=torch.int64, device=d)
+    fl1 = torch.full((1, -(-S1 // 128), -(-S1 // 32)), 2, dtype=torch.int8, device=d)
+    with pytest.raises(_bam_hip.BamError, match="BAM_MAX_SEQLEN"):
+        BA._bitfield_attn_forward(q1, q1, q1, bf1, fl1)
