@@ -168,10 +168,11 @@ __device__ __forceinline__ float load_bias1(const void* base, int64_t index, boo
 // ---------------------------------------------------------------------------------
 // LDS tile layout.  A tile is ROWS x D elements of 2 bytes, stored as 16-byte chunks;
 // chunk c of row r lives at chunk slot  r * (D/8) + (c ^ swz(r)).  The XOR pattern is a
-// one-bit rotation of the 256-byte line number, which makes both access shapes used by
-// the kernels conflict free:
-//   * natural read  : 16 lanes read the same chunk column of 16 consecutive rows;
-//   * transposed read (ds_read_b64_tr_b16): 16 lanes read a 4-row x 32-byte block.
+// one-bit rotation of the 256-byte line number.  Access shapes used by the kernels:
+//   * natural read  : 16 lanes read the same chunk column of 16 consecutive rows (conflict free);
+//   * transposed read (ds_read_b64_tr_b16): 16 lanes read a 4-row x 32-byte block (conflict free
+//     within the 16 lanes; the two blocks of a half wave overlap in two bank groups, which costs
+//     two cycles per instruction, hidden inside the four cycles a wave-wide LDS instruction takes).
 template <int D>
 __device__ __forceinline__ int swz(int row) {
     constexpr int NCH = D / 8;                                       // chunks per row: 4, 8, 16
