@@ -102,3 +102,27 @@ def test_private_entry_points_and_hf_adapter():
     assert none is None and torch.equal(out, o)
     with pytest.raises(RuntimeError):  # reference attention.py:886-890
         A.flash_attn_func(q, k, v, bias=torch.zeros(1, 4, 3, 144, device=d))
+
+
+def test_full_size_mask_materialized_from_bitfields_gives_the_bitfield_result_bit_for_bit():
+    # C2 (S = 8192, GQA 32/8, D = 128): the same kernels with the allow decision read from the materialized mask
+    # instead of derived from the bitfields must produce identical bits, forward and backward
+    from cornstarch_amd import workloads as W
+    from cornstarch_amd.kernel import bitfield_attention as BA
+
+    d = dev()
+    q, k, v, do = (t.to(d) for t in W.make_tensors("C2"))
+    bf = W.make_bitfields("C2").to(d)
+    mask = BA.materialize_bitfield_mask(bf)
+    assert mask.dtype == torch.bool and mask.shape == (1, 8192, 8192)
+    BA.BitfieldUtils.clear_cache()
+    flags_b = BA.BitfieldUtils.materialize_compressed_mask_from_bitfield_mask(bf)
+    assert torch.equal(A.mask_tile_flags(mask, 1, 8192, 8192, d), flags_b)
+    outs = []
+    for fn in (lambda a, b, c: BA.bitfield_attn_func(a, b, c, bf), lambda a, b, c: A.flash_attn_func(a, b, c, mask=mask)):
+        qg, kg, vg = (t.clone().requires_grad_(True) for t in (q, k, v))
+        o = fn(qg, kg, vg)
+        outs.append((o.detach(), *torch.autograd.grad(o, (qg, kg, vg), do)))
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)
+    BA.BitfieldUtils.clear_cache()
