@@ -140,7 +140,10 @@ __global__ __launch_bounds__(FWD_THREADS, D == 128 ? 2 : 3) void fwd_kernel(cons
         // ---- S^T = K Q^T : 64 keys x 32 queries per wave ----------------------------------
         // two independent accumulator chains (key blocks 0 and 1) alternate; operand reads run AHEAD
         // MFMAs in front of their use; the first MFMA of a chain takes C = 0
+        // (the MFMA phases run at raised wave priority: when the SIMD's other wave is in its softmax phase, this
+        // wave's next MFMA is picked first and the MFMA pipe does not idle behind a queue of VALU instructions)
         f32x16 s[2];
+        __builtin_amdgcn_s_setprio(1);
         {
             constexpr int NOP = 2 * KK, AHEAD = 4;
             u32x4 ka[NOP];
@@ -156,6 +159,7 @@ __global__ __launch_bounds__(FWD_THREADS, D == 128 ? 2 : 3) void fwd_kernel(cons
             }
             __builtin_amdgcn_sched_barrier(0);
         }
+        __builtin_amdgcn_s_setprio(0);
 
         if (BIAS) {
 #pragma unroll
@@ -287,6 +291,7 @@ __global__ __launch_bounds__(FWD_THREADS, D == 128 ? 2 : 3) void fwd_kernel(cons
         }
 
         // ---- O^T += V^T P^T -------------------------------------------------------------------
+        __builtin_amdgcn_s_setprio(1);
         {
             u32x4 va[2][2][DB];
 #pragma unroll
@@ -304,6 +309,7 @@ __global__ __launch_bounds__(FWD_THREADS, D == 128 ? 2 : 3) void fwd_kernel(cons
                     for (int db = 0; db < DB; ++db) o[db] = T::mfma(va[kb][t][db], pb[kb][t], o[db]);
             sched_pipeline_mfma_lds<4 * DB, (DB >= 2 ? 3 : 2), 2>();
         }
+        __builtin_amdgcn_s_setprio(0);
     };
 
     __syncthreads();
