@@ -432,3 +432,24 @@ def test_maximum_sequence_length_and_one_beyond():
     fl1 = torch.full((1, -(-S1 // 128), -(-S1 // 32)), 2, dtype=torch.int8, device=d)
     with pytest.raises(_bam_hip.BamError, match="BAM_MAX_SEQLEN"):
         BA._bitfield_attn_forward(q1, q1, q1, bf1, fl1)
+
+
+@pytest.mark.parametrize("std,D,dtype", [(2.0, 128, torch.bfloat16), (3.0, 64, torch.float16), (4.0, 128, torch.bfloat16)])
+def test_large_score_magnitudes(std, D, dtype):
+    # log-sum-exp up to ~80: the deferred rescale of the online softmax (probabilities may exceed 1 by up to
+    # 2^8 before the running maximum moves) must stay finite and accurate, also in fp16
+    g = torch.Generator().manual_seed(5)
+    B, S, Hq, Hkv = 1, 700, 4, 2
+    q = (torch.randn(B, S, Hq, D, generator=g) * std).to(dtype)
+    k = (torch.randn(B, S, Hkv, D, generator=g) * std).to(dtype)
+    v = torch.randn(B, S, Hkv, D, generator=g).to(dtype)
+    do = torch.randn(B, S, Hq, D, generator=g).to(dtype)
+    bf = random_bitfield(B, S, seed=3)
+    o, lse, dq, dk, dv = run_hip(q, k, v, bf, do)
+    o_ref, lse_ref = O.attention_forward(q, k, v, bf)
+    assert lse_ref.abs().max().item() > 15
+    assert torch.isfinite(o).all()
+    assert (o.float() - o_ref).abs().max().item() <= O_MAX_ABS
+    assert (lse - lse_ref).abs().max().item() <= 3e-2
+    for got, want in zip((dq, dk, dv), O.attention_backward(q, k, v, bf, do)):
+        assert rel_l2(got.float(), want) <= GRAD_REL_L2
