@@ -6,8 +6,11 @@ resident in HBM: tile flags -> forward -> delta -> dK/dV -> dQ (gradients writte
 input dtype), i.e. everything ``bitfield_attn_func(...).backward(dO)`` launches.  The figure of merit is effective
 TFLOP/s over UNMASKED (query, key) pairs: fwd 4*D*Hq*pairs, bwd 10*D*Hq*pairs.
 
-Prints one JSON line (see --help for the knobs).  The CPU baseline leg times the oracle's
-materialized-mask SDPA in fp32 on the host cores on a bounded sample (one KV group).
+Prints one JSON line (see --help for the knobs).  Next to the kernel-level step it reports the same work
+driven through the public entry point (``bitfield_attn_func`` + ``torch.autograd.grad``, "api_ms_per_step"),
+mean and median, the MFMA FLOPs the kernels issue according to their tile lists, a short record for the other
+three GPU workloads, and the CPU baseline: the oracle's materialized-mask SDPA in fp32 on the host cores on a
+bounded sample.
 """
 
 from __future__ import annotations
@@ -16,6 +19,7 @@ import argparse
 import json
 import math
 import os
+import statistics
 import sys
 import time
 
@@ -32,6 +36,9 @@ def parse():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="C2", choices=["C2", "C3", "C4", "C5"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-other-workloads", action="store_true",
+                    help="skip the short C3 / C4 / C5 records that accompany the default (C2) run")
+    ap.add_argument("--other-steps", type=int, default=5)
     ap.add_argument("--copy-calibration", action="store_true",
                     help="after the timed region, run a plain 1 GiB device copy (reads 1 GiB, writes 1 GiB) so that "
                          "a rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run of this command also holds a kernel of known traffic")
@@ -49,7 +56,8 @@ def cpu_baseline(name):
 
     w = W.WORKLOADS[name]
     G = w.Hq // w.Hkv
-    torch.set_num_threads(min(os.cpu_count() or 1, 16))
+    # every core this process may use: the scheduler's share where the environment states one, else all of them
+    torch.set_num_threads(int(os.environ.get("OMP_NUM_THREADS") or 0) or os.cpu_count() or 1)
     bf = W.make_bitfields(name)
 
     def timed(heads, reps):
@@ -91,27 +99,38 @@ def measured_traffic(workload, kernel):
     return None
 
 
-def main():
-    args = parse()
-    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
-        sys.exit(2)
+def issued_flops(flags, w):
+    """MFMA FLOPs the three attention kernels issue, from the tile lists they build out of the flags:
+    the forward and dQ kernels compute every 128-row x 64-key tile with a non-zero flag (4 resp. 6 D-deep
+    products per pair), dK/dV every 128-row x 32-key flag tile (8).  Partial tiles count in full."""
+    import torch
+    import torch.nn.functional as F
 
+    nz = flags > 0
+    if nz.shape[-1] % 2:
+        nz = F.pad(nz, (0, 1))
+    tiles64 = int((nz[..., 0::2] | nz[..., 1::2]).sum())
+    tiles32 = int(nz.sum())
+    per_pair = w.D * w.Hq
+    return {
+        "fwd": 4 * per_pair * tiles64 * 128 * 64,
+        "dkdv": 8 * per_pair * tiles32 * 128 * 32,
+        "dq": 6 * per_pair * tiles64 * 128 * 64,
+    }
+
+
+def run_workload(name, steps, warmup, dev):
+    """Times `steps` steps of workload `name` (after `warmup` untimed ones), kernel level and through the public
+    entry point.  Returns a dict of measurements."""
     import torch
 
     from cornstarch_amd import workloads as W
     from cornstarch_amd.kernel import bitfield_attention as BA
     from oracle import bam_oracle as O  # checker / baseline only
 
-    assert torch.cuda.is_available(), "bench.py needs the GPU"
-    dev = torch.device("cuda:0")
-    torch.cuda.set_device(dev)
-    name = args.workload
     w = W.WORKLOADS[name]
-
     q, k, v, do = (t.to(dev) for t in W.make_tensors(name))
-    bf_cpu = W.make_bitfields(name)
-    bf = bf_cpu.to(dev)
+    bf = W.make_bitfields(name).to(dev)
     pairs = O.unmasked_pairs(bf)  # exact, on the GPU through torch ops (setup, untimed)
     f_fwd = 4 * w.D * w.Hq * pairs
     f_bwd = 10 * w.D * w.Hq * pairs
@@ -142,17 +161,75 @@ def main():
         mark(6)
         return o, (dq, dk, dv)
 
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         step()
     torch.cuda.synchronize()
 
-    events = [[torch.cuda.Event(enable_timing=True) for _ in range(n_ev)] for _ in range(args.steps)]
+    events = [[torch.cuda.Event(enable_timing=True) for _ in range(n_ev)] for _ in range(steps)]
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for i in range(args.steps):
+    for i in range(steps):
         step(events[i])
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
+
+    ms_per_step = wall * 1e3 / steps
+    per_step = [ev[0].elapsed_time(ev[-1]) for ev in events]
+    stage_ms, stage_med = {}, {}
+    for si, s in enumerate(stages):
+        xs = [ev[si].elapsed_time(ev[si + 1]) for ev in events]
+        stage_ms[s] = sum(xs) / steps
+        stage_med[s] = statistics.median(xs)
+
+    # the same work through the entry point callers use: autograd Function, flag cache cleared every step
+    qg, kg, vg = (t.detach().requires_grad_(True) for t in (q, k, v))
+
+    def api_step():
+        BA.BitfieldUtils.clear_cache()
+        o = BA.bitfield_attn_func(qg, kg, vg, bf)
+        return torch.autograd.grad(o, (qg, kg, vg), do)
+
+    for _ in range(min(warmup, 3)):
+        api_step()
+    torch.cuda.synchronize()
+    api_ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    t0 = time.perf_counter()
+    for a, b in api_ev:
+        a.record()
+        api_step()
+        b.record()
+    torch.cuda.synchronize()
+    api_wall = time.perf_counter() - t0
+    api_times = [a.elapsed_time(b) for a, b in api_ev]
+
+    BA.BitfieldUtils.clear_cache()
+    flags = BA.BitfieldUtils.materialize_compressed_mask_from_bitfield_mask(bf)
+    issued = issued_flops(flags, w)
+    BA.BitfieldUtils.clear_cache()
+    return {
+        "w": w, "pairs": pairs, "f_fwd": f_fwd, "f_bwd": f_bwd,
+        "ms_per_step": ms_per_step, "median_ms_per_step": statistics.median(per_step),
+        "stage_ms": stage_ms, "stage_median_ms": stage_med,
+        "api_ms_per_step": api_wall * 1e3 / steps, "api_median_ms_per_step": statistics.median(api_times),
+        "issued": issued,
+    }
+
+
+def main():
+    args = parse()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    assert torch.cuda.is_available(), "bench.py needs the GPU"
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    name = args.workload
+    r = run_workload(name, args.steps, args.warmup, dev)
+    w, pairs, f_fwd, f_bwd = r["w"], r["pairs"], r["f_fwd"], r["f_bwd"]
+    stage_ms, ms_per_step = r["stage_ms"], r["ms_per_step"]
 
     if args.copy_calibration:
         src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
@@ -162,10 +239,6 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    ms_per_step = wall * 1e3 / args.steps
-    stage_ms = {}
-    for si, s in enumerate(stages):
-        stage_ms[s] = sum(ev[si].elapsed_time(ev[si + 1]) for ev in events) / args.steps
     fwd_ms = stage_ms["flags"] + stage_ms["fwd"]
     bwd_ms = stage_ms["alloc"] + stage_ms["delta"] + stage_ms["dkdv"] + stage_ms["dq"]
 
@@ -199,11 +272,23 @@ def main():
             "flops_fwd": f_fwd,
             "flops_bwd": f_bwd,
         },
+        "median_ms_per_step": round(r["median_ms_per_step"], 4),
+        "api_ms_per_step": round(r["api_ms_per_step"], 4),
+        "api_median_ms_per_step": round(r["api_median_ms_per_step"], 4),
         "fwd_ms": round(fwd_ms, 4),
         "bwd_ms": round(bwd_ms, 4),
         "fwd_tflops": round(f_fwd / (fwd_ms * 1e-3) / 1e12, 3),
         "mfma_util_unmasked": round(value / PEAK_BF16_DENSE_TFLOPS, 4),
         "stage_ms": {s: round(x, 4) for s, x in stage_ms.items()},
+        "stage_median_ms": {s: round(x, 4) for s, x in r["stage_median_ms"].items()},
+        # MFMA FLOPs issued according to the tile lists, and their ratio to the algorithmic (unmasked-pair) FLOPs of
+        # the GEMMs each kernel runs (forward 2, dK/dV 4, dQ 3: dQ recomputes S and dP)
+        "issued_mfma_flops": r["issued"],
+        "issued_over_unmasked": {
+            "fwd": round(r["issued"]["fwd"] / f_fwd, 4),
+            "dkdv": round(r["issued"]["dkdv"] / (8 * w.D * w.Hq * pairs), 4),
+            "dq": round(r["issued"]["dq"] / (6 * w.D * w.Hq * pairs), 4),
+        },
         "roofline": {
             "kernel": kname[dom],
             "bound": "mfma",
@@ -212,9 +297,28 @@ def main():
             "unit": "TFLOP/s",
             "frac": round(achieved / PEAK_BF16_DENSE_TFLOPS, 4),
             "traffic": traffic,
+            "traffic_source": "profiles/hbm_traffic.txt (rocprofv3 --pmc run of this command on another box)"
+            if traffic is not None else None,
             "avg_launch_ms": round(stage_ms[dom], 4),
+            "issued_tflops": round(r["issued"][dom] / (stage_ms[dom] * 1e-3) / 1e12, 3),
         },
     }
+    if name == "C2" and not args.no_other_workloads:
+        others = {}
+        for other in ("C3", "C4", "C5"):
+            torch.cuda.empty_cache()
+            ro = run_workload(other, args.other_steps, 2, dev)
+            tot = ro["f_fwd"] + ro["f_bwd"]
+            others[other] = {
+                "ms_per_step": round(ro["ms_per_step"], 4),
+                "api_ms_per_step": round(ro["api_ms_per_step"], 4),
+                "tflops": round(tot / (ro["ms_per_step"] * 1e-3) / 1e12, 3),
+                "steps": args.other_steps,
+                "unmasked_pairs": ro["pairs"],
+                "stage_ms": {s: round(x, 4) for s, x in ro["stage_ms"].items()},
+                "issued_over_unmasked": round(sum(ro["issued"].values()) / (18 * ro["w"].D * ro["w"].Hq * ro["pairs"]), 4),
+            }
+        result["other_workloads"] = others
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(name)
     print(json.dumps(result))

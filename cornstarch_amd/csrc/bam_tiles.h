@@ -13,7 +13,9 @@ __device__ __forceinline__ unsigned lds_addr(const void* p) {
 
 // One direct global -> LDS copy instruction.  Lane l fetches `bytes` (16 or 4) from
 // sbase + voff and the hardware writes them to LDS byte address lds_base + l * bytes;
-// sbase and lds_base must be wave-uniform.  Issued as inline asm on purpose: the compiler
+// sbase and lds_base must be wave-uniform.  The LDS base travels in M0: it is handed to the asm
+// statement as an input operand bound to that register, so the compiler writes M0 itself and knows
+// it is occupied; the s_nop is the wait state the hardware wants between an M0 write and its use.  Issued as inline asm on purpose: the compiler
 // then neither tracks the copy in vmcnt nor makes later LDS reads wait for it, which is what
 // lets a tile load stay in flight across a whole loop iteration.  The price is that the
 // caller owns the synchronization: wait_async() (or wait_async_but<N>()) + a workgroup
@@ -23,14 +25,14 @@ __device__ __forceinline__ unsigned lds_addr(const void* p) {
 // keeps each where the schedule wants it.
 template <int SITE = 0>
 __device__ __forceinline__ void dma_b128(const void* sbase, unsigned voff, unsigned lds_base) {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 ; site %3" ::"v"(voff), "s"(sbase),
-                 "s"(lds_base), "n"(SITE)
+    asm volatile("s_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 ; site %3" ::"v"(voff), "s"(sbase), "{m0}"(lds_base),
+                 "n"(SITE)
                  : "memory");
 }
 template <int SITE = 0>
 __device__ __forceinline__ void dma_b32(const void* sbase, unsigned voff, unsigned lds_base) {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1 ; site %3" ::"v"(voff), "s"(sbase),
-                 "s"(lds_base), "n"(SITE)
+    asm volatile("s_nop 0\n\tglobal_load_lds_dword %0, %1 ; site %3" ::"v"(voff), "s"(sbase), "{m0}"(lds_base),
+                 "n"(SITE)
                  : "memory");
 }
 

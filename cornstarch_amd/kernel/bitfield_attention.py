@@ -78,28 +78,38 @@ class BitfieldUtils:
         1: some pairs are allowed, the mask is evaluated
         2: every in-range pair is allowed, the mask is not evaluated
     Same API as the reference (bitfield_attention.py:159-212).  The reference returns
-    whatever the cache holds until ``clear_cache()``; here the cache is also keyed on the
-    identity of the bitfield tensor, so a different mask can never pick up stale flags.
+    whatever the cache holds until ``clear_cache()``; here a hit additionally requires the
+    argument to be the very memory the flags were computed from, unchanged: the cache holds a
+    reference to that tensor (so its address cannot be handed to another tensor while the
+    entry lives) and compares address, shape, strides and version counter.
     """
 
     compressed_mask_cache: Optional[torch.Tensor] = None
     _cache_key = None
+    _cache_owner: Optional[torch.Tensor] = None  # the bitfield tensor the cached flags belong to
 
     @classmethod
     def clear_cache(cls):
         cls.compressed_mask_cache = None
         cls._cache_key = None
+        cls._cache_owner = None
 
-    @classmethod
-    def materialize_compressed_mask_from_bitfield_mask(cls, bitfield_mask: torch.Tensor) -> torch.Tensor:
-        key = (
+    @staticmethod
+    def _key_of(bitfield_mask: torch.Tensor):
+        return (
             bitfield_mask.data_ptr(),
             tuple(bitfield_mask.shape),
             tuple(bitfield_mask.stride()),
             bitfield_mask._version,
             bitfield_mask.device,
         )
+
+    @classmethod
+    def materialize_compressed_mask_from_bitfield_mask(cls, bitfield_mask: torch.Tensor) -> torch.Tensor:
+        key = cls._key_of(bitfield_mask)
         if cls.compressed_mask_cache is not None and cls._cache_key == key:
+            # _cache_owner is alive, so this address still belongs to the tensor (or a view of the
+            # tensor) the flags were computed from, and its version says it has not been written since
             return cls.compressed_mask_cache
 
         assert bitfield_mask.is_cuda, "bitfield attention runs on the GPU only"
@@ -118,6 +128,7 @@ class BitfieldUtils:
             )
         cls.compressed_mask_cache = out
         cls._cache_key = key
+        cls._cache_owner = bitfield_mask
         return out
 
     @classmethod

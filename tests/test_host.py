@@ -132,6 +132,10 @@ def test_adapter_requires_int64_mask():
     want = torch.softmax(
         (q1 @ kv.repeat_interleave(2, 1).transpose(-1, -2)) / 32**0.5, -1) @ kv.repeat_interleave(2, 1)
     assert torch.allclose(out, want.transpose(1, 2), atol=1e-5)
+    # a window or a logit cap would change the decode logits: refused, not dropped
+    for kw in ({"sliding_window": 4}, {"softcap": 30.0}):
+        with pytest.raises(NotImplementedError):
+            interface.bitfield_attention_forward(m, q1, kv, kv, None, **kw)
 
 
 # histogram / pair counts of the synthetic workloads quoted by the baseline document

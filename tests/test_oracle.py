@@ -193,6 +193,14 @@ def test_backward_against_autograd_through_sdpa(S, Hq, Hkv, D):
     cq, ck, cv = C.attn_bwd(*(x.float().numpy() for x in (q, k, v, do)), lse.float().numpy(), dlt, bf.numpy())
     for got, want in ((cq, wq), (ck, wk), (cv, wv)):
         assert rel_l2(torch.from_numpy(got), want) < 1e-5
+    # delta has a second face the oracle does not compute it from: rowsum(o * do) = rowsum(P * (dO V^T)),
+    # with P and dO V^T built here from an explicit masked softmax
+    g = Hq // Hkv
+    kx, vx = k.repeat_interleave(g, dim=2), v.repeat_interleave(g, dim=2)
+    sc = torch.einsum("bihd,bjhd->bhij", q, kx) / math.sqrt(D)
+    P = torch.softmax(sc.masked_fill(~full.unsqueeze(1), float("-inf")), dim=-1)
+    dP = torch.einsum("bihd,bjhd->bhij", do, vx)
+    assert torch.allclose(O.delta(o, do).double(), (P * dP).sum(-1), atol=1e-5)
 
 
 def test_rows_without_any_allowed_key_give_zero_output_and_minus_inf_lse():
