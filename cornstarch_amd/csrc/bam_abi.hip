@@ -51,6 +51,7 @@ int check_problem(int B, int Sq, int Sk, int Hq, int Hkv, int D, int dtype) {
         return fail(BAM_ERR_UNSUPPORTED, "head dimension %d is not supported (32, 64 or 128)", D);
     if (dtype != BAM_DTYPE_F16 && dtype != BAM_DTYPE_BF16)
         return fail(BAM_ERR_INVALID_ARGUMENT, "dtype %d is neither BAM_DTYPE_F16 nor BAM_DTYPE_BF16", dtype);
+    static_assert(BAM_MAX_SEQLEN == bam::MAX_SEQLEN, "header and kernels disagree on the longest sequence");
     if (Sq > BAM_MAX_SEQLEN || Sk > BAM_MAX_SEQLEN)
         return fail(BAM_ERR_UNSUPPORTED, "S = %d exceeds BAM_MAX_SEQLEN = %d", Sq > Sk ? Sq : Sk, BAM_MAX_SEQLEN);
     if ((int64_t)((Sq + 127) / 128) * B * Hq > 0x7FFFFFFFll || (int64_t)((Sk + 127) / 128) * B * Hkv > 0x7FFFFFFFll)
@@ -117,6 +118,22 @@ int fill_bias(bam::AttnParams& p, const char* who, const bam_bias* bias, int Sk)
     return BAM_OK;
 }
 
+// plan may be null.  It must have been built for this very (B, S).
+int fill_plan(bam::AttnParams& p, const char* who, const bam_plan* plan, int B, int S) {
+    if (plan == nullptr) return BAM_OK;  // p.fine stays null
+    if (plan->fine == nullptr || plan->order == nullptr) return fail(BAM_ERR_INVALID_ARGUMENT, "%s: plan: null array", who);
+    if (plan->B != B || plan->S != S)
+        return fail(BAM_ERR_INVALID_ARGUMENT, "%s: plan was built for B = %d, S = %d, not B = %d, S = %d", who, plan->B,
+                    plan->S, B, S);
+    if (reinterpret_cast<uintptr_t>(plan->order) & 3u) return fail(BAM_ERR_INVALID_ARGUMENT, "%s: plan: misaligned order", who);
+    p.fine = plan->fine;
+    p.fine_sb = plan->fine_stride_b;
+    p.fine_ss = plan->fine_stride_s;
+    p.order = plan->order;
+    p.order_sb = plan->order_stride_b;
+    return BAM_OK;
+}
+
 void fill_sizes(bam::AttnParams& p, const MaskSource& m, int B, int Hq, int Hkv, int D, float scale) {
     p.bfq = m.bfq;
     p.bfk = m.bfk;
@@ -141,11 +158,11 @@ void fill_sizes(bam::AttnParams& p, const MaskSource& m, int B, int Hq, int Hkv,
 
 int fwd_impl(const char* who, const void* q, const void* k, const void* v, void* o, float* lse, const MaskSource& m,
              const int8_t* flags, const int64_t* st, int64_t flags_stride_b, int64_t flags_stride_m, int B, int Hq,
-             int Hkv, int D, float scale, int dtype, const bam_bias* bias, void* stream);
+             int Hkv, int D, float scale, int dtype, const bam_bias* bias, const bam_plan* plan, void* stream);
 int bwd_params(bam::AttnParams& p, const char* who, const void* q, const void* k, const void* v, const void* dout,
                const float* lse, const float* delta, void* dq, void* dk, void* dv, const MaskSource& m,
                const int8_t* flags, const int64_t* st, int B, int Hq, int Hkv, int D, float scale, int dtype,
-               int accumulate, bool need_dq, bool need_dkdv, const bam_bias* bias);
+               int accumulate, bool need_dq, bool need_dkdv, const bam_bias* bias, const bam_plan* plan);
 
 }  // namespace
 
@@ -159,7 +176,7 @@ namespace {
 
 int fwd_impl(const char* who, const void* q, const void* k, const void* v, void* o, float* lse, const MaskSource& m,
              const int8_t* flags, const int64_t* st, int64_t flags_stride_b, int64_t flags_stride_m, int B, int Hq,
-             int Hkv, int D, float scale, int dtype, const bam_bias* bias, void* stream) {
+             int Hkv, int D, float scale, int dtype, const bam_bias* bias, const bam_plan* plan, void* stream) {
     BAM_TRY(check_problem(B, m.Sq, m.Sk, Hq, Hkv, D, dtype));
     BAM_TRY(check_half_tensor("q", q, st[0], st[1], st[2]));
     BAM_TRY(check_half_tensor("k", k, st[3], st[4], st[5]));
@@ -179,6 +196,7 @@ int fwd_impl(const char* who, const void* q, const void* k, const void* v, void*
     p.flags_sm = flags_stride_m;
     fill_sizes(p, m, B, Hq, Hkv, D, scale);
     BAM_TRY(fill_bias(p, who, bias, m.Sk));
+    BAM_TRY(fill_plan(p, who, plan, B, m.Sq));
     return launched(bam::launch_fwd(p, dtype, (hipStream_t)stream), who);
 }
 
@@ -186,7 +204,7 @@ int fwd_impl(const char* who, const void* q, const void* k, const void* v, void*
 int bwd_params(bam::AttnParams& p, const char* who, const void* q, const void* k, const void* v, const void* dout,
                const float* lse, const float* delta, void* dq, void* dk, void* dv, const MaskSource& m,
                const int8_t* flags, const int64_t* st, int B, int Hq, int Hkv, int D, float scale, int dtype,
-               int accumulate, bool need_dq, bool need_dkdv, const bam_bias* bias) {
+               int accumulate, bool need_dq, bool need_dkdv, const bam_bias* bias, const bam_plan* plan) {
     BAM_TRY(check_problem(B, m.Sq, m.Sk, Hq, Hkv, D, dtype));
     BAM_TRY(check_half_tensor("q", q, st[0], st[1], st[2]));
     BAM_TRY(check_half_tensor("k", k, st[3], st[4], st[5]));
@@ -223,6 +241,7 @@ int bwd_params(bam::AttnParams& p, const char* who, const void* q, const void* k
     p.flags_sb = st[21];
     p.flags_sm = st[22];
     fill_sizes(p, m, B, Hq, Hkv, D, scale);
+    BAM_TRY(fill_plan(p, who, plan, B, m.Sq));
     return fill_bias(p, who, bias, m.Sk);
 }
 
@@ -232,7 +251,7 @@ extern "C" {
 
 const char* bam_last_error(void) { return g_error; }
 
-int bam_abi_version(void) { return 5; }
+int bam_abi_version(void) { return 6; }
 
 int bam_tile_flags(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int64_t flags_stride_b,
                    int64_t flags_stride_m, int B, int S, void* stream) {
@@ -243,6 +262,61 @@ int bam_tile_flags(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int64_
     return launched(bam::launch_tile_flags(bf, bf_stride_b, flags, flags_stride_b, flags_stride_m, B, S,
                                            (hipStream_t)stream),
                     "bam_tile_flags");
+}
+
+namespace {
+// workspace layout: fine | order | sort keys, each part 256-byte aligned
+struct PlanLayout {
+    int64_t fine_ss, fine_sb, order_sb, fine_off, order_off, keys_off, bytes;
+};
+PlanLayout plan_layout(int B, int S) {
+    const int64_t num_m = (S + 127) / 128, num_n = (S + 31) / 32, slots = 4 * num_m;
+    auto up = [](int64_t x, int64_t a) { return (x + a - 1) / a * a; };
+    PlanLayout l;
+    l.fine_ss = up(num_n, 16);
+    l.fine_sb = slots * l.fine_ss;
+    l.order_sb = slots;
+    l.fine_off = 0;
+    l.order_off = up(B * l.fine_sb, 256);
+    l.keys_off = l.order_off + up(B * slots * 4, 256);
+    l.bytes = l.keys_off + up(B * slots * 16, 256);
+    return l;
+}
+}  // namespace
+
+int64_t bam_plan_workspace_bytes(int B, int S) {
+    if (B <= 0 || S <= 0 || (S + 31) / 32 > bam::MAX_PLAN_SLICES) return 0;
+    return plan_layout(B, S).bytes;
+}
+
+int bam_tile_plan(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int64_t flags_stride_b,
+                  int64_t flags_stride_m, void* workspace, int64_t workspace_bytes, int B, int S, bam_plan* plan,
+                  void* stream) {
+    if (bf == nullptr || flags == nullptr || workspace == nullptr || plan == nullptr)
+        return fail(BAM_ERR_INVALID_ARGUMENT, "bam_tile_plan: null pointer");
+    if (B <= 0 || S <= 0) return fail(BAM_ERR_INVALID_ARGUMENT, "bam_tile_plan: B and S must be positive");
+    if (B > 65535 || (S + 127) / 128 > 65535)
+        return fail(BAM_ERR_UNSUPPORTED, "bam_tile_plan: grid too large (B = %d, S = %d)", B, S);
+    const int64_t need = bam_plan_workspace_bytes(B, S);
+    if (need == 0) return fail(BAM_ERR_UNSUPPORTED, "bam_tile_plan: no plan is built for S = %d (use bam_tile_flags)", S);
+    if (workspace_bytes < need)
+        return fail(BAM_ERR_INVALID_ARGUMENT, "bam_tile_plan: workspace of %lld bytes, %lld needed", (long long)workspace_bytes,
+                    (long long)need);
+    if (reinterpret_cast<uintptr_t>(workspace) & 255u)
+        return fail(BAM_ERR_INVALID_ARGUMENT, "bam_tile_plan: workspace is not 256-byte aligned");
+    const PlanLayout l = plan_layout(B, S);
+    char* w = (char*)workspace;
+    plan->fine = (const uint8_t*)(w + l.fine_off);
+    plan->fine_stride_b = l.fine_sb;
+    plan->fine_stride_s = l.fine_ss;
+    plan->order = (const int32_t*)(w + l.order_off);
+    plan->order_stride_b = l.order_sb;
+    plan->B = B;
+    plan->S = S;
+    return launched(bam::launch_tile_plan(bf, bf_stride_b, flags, flags_stride_b, flags_stride_m, (uint8_t*)(w + l.fine_off),
+                                          l.fine_sb, l.fine_ss, (int*)(w + l.order_off), l.order_sb,
+                                          (unsigned long long*)(w + l.keys_off), B, S, (hipStream_t)stream),
+                    "bam_tile_plan");
 }
 
 int bam_materialize_mask(const int64_t* bf, int64_t bf_stride_b, uint8_t* out, int B, int S, void* stream) {
@@ -284,10 +358,11 @@ int bam_fwd(const void* q, const void* k, const void* v, void* o, float* lse, co
             int64_t k_stride_b, int64_t k_stride_s, int64_t k_stride_h, int64_t v_stride_b,
             int64_t v_stride_s, int64_t v_stride_h, int64_t o_stride_b, int64_t o_stride_s,
             int64_t o_stride_h, int64_t bf_stride_b, int64_t flags_stride_b, int64_t flags_stride_m, int B,
-            int S, int Hq, int Hkv, int D, float scale, int dtype, const bam_bias* bias, void* stream) {
+            int S, int Hq, int Hkv, int D, float scale, int dtype, const bam_bias* bias, const bam_plan* plan,
+            void* stream) {
     const int64_t st[12] = BAM_FWD_STRIDES;
     return fwd_impl("bam_fwd", q, k, v, o, lse, plain_source(bf, bf_stride_b, S), flags, st, flags_stride_b,
-                    flags_stride_m, B, Hq, Hkv, D, scale, dtype, bias, stream);
+                    flags_stride_m, B, Hq, Hkv, D, scale, dtype, bias, plan, stream);
 }
 
 int bam_fwd_indexed(const void* q, const void* k, const void* v, void* o, float* lse, const bam_index_view* iv,
@@ -300,7 +375,7 @@ int bam_fwd_indexed(const void* q, const void* k, const void* v, void* o, float*
     BAM_TRY(indexed_source(iv, m));
     const int64_t st[12] = BAM_FWD_STRIDES;
     return fwd_impl("bam_fwd_indexed", q, k, v, o, lse, m, flags, st, flags_stride_b, flags_stride_m, B, Hq, Hkv, D,
-                    scale, dtype, bias, stream);
+                    scale, dtype, bias, nullptr, stream);
 }
 
 int bam_bwd_preprocess(const void* o, const void* dout, float* delta, int64_t o_stride_b, int64_t o_stride_s,
@@ -331,11 +406,12 @@ int bam_bwd(const void* q, const void* k, const void* v, const void* dout, const
             int64_t dq_stride_b, int64_t dq_stride_s, int64_t dq_stride_h, int64_t dk_stride_b,
             int64_t dk_stride_s, int64_t dk_stride_h, int64_t dv_stride_b, int64_t dv_stride_s,
             int64_t dv_stride_h, int64_t bf_stride_b, int64_t flags_stride_b, int64_t flags_stride_m, int B,
-            int S, int Hq, int Hkv, int D, float scale, int dtype, int accumulate, const bam_bias* bias, void* stream) {
+            int S, int Hq, int Hkv, int D, float scale, int dtype, int accumulate, const bam_bias* bias,
+            const bam_plan* plan, void* stream) {
     const int64_t st[23] = BAM_BWD_STRIDES;
     bam::AttnParams p = {};
     BAM_TRY(bwd_params(p, "bam_bwd", q, k, v, dout, lse, delta, dq, dk, dv, plain_source(bf, bf_stride_b, S), flags, st, B,
-                       Hq, Hkv, D, scale, dtype, accumulate, true, true, bias));
+                       Hq, Hkv, D, scale, dtype, accumulate, true, true, bias, plan));
     BAM_TRY(launched(bam::launch_bwd_dkdv(p, dtype, (hipStream_t)stream), "bam_bwd (dk/dv)"));
     return launched(bam::launch_bwd_dq(p, dtype, (hipStream_t)stream), "bam_bwd (dq)");
 }
@@ -348,13 +424,13 @@ int bam_bwd_dkdv(const void* q, const void* k, const void* v, const void* dout, 
                  int64_t dk_stride_b, int64_t dk_stride_s, int64_t dk_stride_h, int64_t dv_stride_b,
                  int64_t dv_stride_s, int64_t dv_stride_h, int64_t bf_stride_b, int64_t flags_stride_b,
                  int64_t flags_stride_m, int B, int S, int Hq, int Hkv, int D, float scale, int dtype,
-                 int accumulate, const bam_bias* bias, void* stream) {
+                 int accumulate, const bam_bias* bias, const bam_plan* plan, void* stream) {
     void* dq = nullptr;
     const int64_t dq_stride_b = 0, dq_stride_s = 0, dq_stride_h = 0;
     const int64_t st[23] = BAM_BWD_STRIDES;
     bam::AttnParams p = {};
     BAM_TRY(bwd_params(p, "bam_bwd_dkdv", q, k, v, dout, lse, delta, dq, dk, dv, plain_source(bf, bf_stride_b, S), flags,
-                       st, B, Hq, Hkv, D, scale, dtype, accumulate, false, true, bias));
+                       st, B, Hq, Hkv, D, scale, dtype, accumulate, false, true, bias, plan));
     return launched(bam::launch_bwd_dkdv(p, dtype, (hipStream_t)stream), "bam_bwd_dkdv");
 }
 
@@ -365,13 +441,13 @@ int bam_bwd_dq(const void* q, const void* k, const void* v, const void* dout, co
                int64_t do_stride_b, int64_t do_stride_s, int64_t do_stride_h, int64_t dq_stride_b,
                int64_t dq_stride_s, int64_t dq_stride_h, int64_t bf_stride_b, int64_t flags_stride_b,
                int64_t flags_stride_m, int B, int S, int Hq, int Hkv, int D, float scale, int dtype,
-               int accumulate, const bam_bias* bias, void* stream) {
+               int accumulate, const bam_bias* bias, const bam_plan* plan, void* stream) {
     void *dk = nullptr, *dv = nullptr;
     const int64_t dk_stride_b = 0, dk_stride_s = 0, dk_stride_h = 0, dv_stride_b = 0, dv_stride_s = 0, dv_stride_h = 0;
     const int64_t st[23] = BAM_BWD_STRIDES;
     bam::AttnParams p = {};
     BAM_TRY(bwd_params(p, "bam_bwd_dq", q, k, v, dout, lse, delta, dq, dk, dv, plain_source(bf, bf_stride_b, S), flags, st,
-                       B, Hq, Hkv, D, scale, dtype, accumulate, true, false, bias));
+                       B, Hq, Hkv, D, scale, dtype, accumulate, true, false, bias, plan));
     return launched(bam::launch_bwd_dq(p, dtype, (hipStream_t)stream), "bam_bwd_dq");
 }
 
@@ -390,7 +466,7 @@ int bam_bwd_dkdv_indexed(const void* q, const void* k, const void* v, const void
     const int64_t st[23] = BAM_BWD_STRIDES;
     bam::AttnParams p = {};
     BAM_TRY(bwd_params(p, "bam_bwd_dkdv_indexed", q, k, v, dout, lse, delta, dq, dk, dv, m, flags, st, B, Hq, Hkv, D, scale,
-                       dtype, accumulate, false, true, bias));
+                       dtype, accumulate, false, true, bias, nullptr));
     return launched(bam::launch_bwd_dkdv(p, dtype, (hipStream_t)stream), "bam_bwd_dkdv_indexed");
 }
 
@@ -409,7 +485,7 @@ int bam_bwd_dq_indexed(const void* q, const void* k, const void* v, const void* 
     const int64_t st[23] = BAM_BWD_STRIDES;
     bam::AttnParams p = {};
     BAM_TRY(bwd_params(p, "bam_bwd_dq_indexed", q, k, v, dout, lse, delta, dq, dk, dv, m, flags, st, B, Hq, Hkv, D, scale,
-                       dtype, accumulate, true, false, bias));
+                       dtype, accumulate, true, false, bias, nullptr));
     return launched(bam::launch_bwd_dq(p, dtype, (hipStream_t)stream), "bam_bwd_dq_indexed");
 }
 
@@ -432,7 +508,7 @@ int bam_fwd_masked(const void* q, const void* k, const void* v, void* o, float* 
     BAM_TRY(check_mask("bam_fwd_masked", mask));
     const int64_t st[12] = BAM_FWD_STRIDES;
     return fwd_impl("bam_fwd_masked", q, k, v, o, lse, dense_source(mask, Sq, Sk), flags, st, flags_stride_b,
-                    flags_stride_m, B, Hq, Hkv, D, scale, dtype, bias, stream);
+                    flags_stride_m, B, Hq, Hkv, D, scale, dtype, bias, nullptr, stream);
 }
 
 int bam_bwd_dkdv_masked(const void* q, const void* k, const void* v, const void* dout, const float* lse,
@@ -450,7 +526,7 @@ int bam_bwd_dkdv_masked(const void* q, const void* k, const void* v, const void*
     const int64_t st[23] = BAM_BWD_STRIDES;
     bam::AttnParams p = {};
     BAM_TRY(bwd_params(p, "bam_bwd_dkdv_masked", q, k, v, dout, lse, delta, dq, dk, dv, dense_source(mask, Sq, Sk), flags,
-                       st, B, Hq, Hkv, D, scale, dtype, accumulate, false, true, bias));
+                       st, B, Hq, Hkv, D, scale, dtype, accumulate, false, true, bias, nullptr));
     return launched(bam::launch_bwd_dkdv(p, dtype, (hipStream_t)stream), "bam_bwd_dkdv_masked");
 }
 
@@ -467,7 +543,7 @@ int bam_bwd_dq_masked(const void* q, const void* k, const void* v, const void* d
     const int64_t st[23] = BAM_BWD_STRIDES;
     bam::AttnParams p = {};
     BAM_TRY(bwd_params(p, "bam_bwd_dq_masked", q, k, v, dout, lse, delta, dq, dk, dv, dense_source(mask, Sq, Sk), flags, st,
-                       B, Hq, Hkv, D, scale, dtype, accumulate, true, false, bias));
+                       B, Hq, Hkv, D, scale, dtype, accumulate, true, false, bias, nullptr));
     return launched(bam::launch_bwd_dq(p, dtype, (hipStream_t)stream), "bam_bwd_dq_masked");
 }
 

@@ -10,8 +10,13 @@ constexpr int MASK_BITFIELD = 0;  // bitfield rule, position = row / column numb
 constexpr int MASK_INDEXED = 1;   // bitfield rule on gathered bitfields and explicit global positions
 constexpr int MASK_DENSE = 2;     // a materialized bool mask (B, Sq, Sk), one byte per pair (or none: all pairs allowed)
 
-// Number of 64-key (forward, dQ) or 128-row (dK/dV) tiles a workgroup can list in LDS.
-constexpr int MAX_LIST = 2048;
+// Longest sequence the attention kernels accept: a workgroup lists its 64-key tiles (forward, dQ) or its 32-row
+// slices (dK/dV) in LDS.
+constexpr int MAX_SEQLEN = 131072;
+constexpr int MAX_LIST = MAX_SEQLEN / 64;         // 64-key tiles of a row
+constexpr int MAX_SLICE_LIST = MAX_SEQLEN / 32;   // 32-row slices of a column
+// A plan (fine classes + slice order) is only built for sequences up to this many 32-row slices.
+constexpr int MAX_PLAN_SLICES = 4096;
 
 struct Tensor4 {  // logical (B, S, H, D), unit stride along D, strides in elements
     const void* ptr;
@@ -44,6 +49,13 @@ struct AttnParams {
     int bias_vec;              // every group of four keys starting at a multiple of four is one aligned, in-range access
     const int8_t* flags;       // (B, num_m, num_n)
     int64_t flags_sb, flags_sm;
+    // Optional plan (plain bitfield attention only; null = none).  fine: class 0 / 1 / 2 of every 32-row x 32-key
+    // tile, (B, 4 * num_m, fine_ss) bytes; order: the 32-row slices of each sequence sorted so that four
+    // neighbours need about the same keys, heaviest first, (B, 4 * num_m) ints, -1 = no slice.
+    const uint8_t* fine;
+    int64_t fine_sb, fine_ss;
+    const int* order;
+    int64_t order_sb;
     int B, Sq, Sk, Hq, Hkv, D;
     int Sq_rounded, num_m, num_n, num_kt;  // ceil(Sq/128)*128, ceil(Sq/128), ceil(Sk/32), ceil(Sk/128)
     float scale;
@@ -51,6 +63,11 @@ struct AttnParams {
 
 int launch_tile_flags(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int64_t flags_stride_b,
                       int64_t flags_stride_m, int B, int S, hipStream_t stream);
+// Flags plus plan: fine (B, 4 * num_m, fine_ss) bytes, order (B, 4 * num_m) ints, keys: scratch of
+// 2 * B * 4 * num_m 64-bit words.
+int launch_tile_plan(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int64_t flags_stride_b,
+                     int64_t flags_stride_m, uint8_t* fine, int64_t fine_sb, int64_t fine_ss, int* order,
+                     int64_t order_sb, unsigned long long* keys, int B, int S, hipStream_t stream);
 int launch_materialize_mask(const int64_t* bf, int64_t bf_stride_b, uint8_t* out, int B, int S,
                             hipStream_t stream);
 int launch_flag_row_workloads(const int8_t* flags, int64_t flags_stride_b, int64_t flags_stride_m, int B, int num_m,

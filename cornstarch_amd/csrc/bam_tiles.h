@@ -96,6 +96,49 @@ struct TileStage {
     }
 };
 
+// 64-row tile made of two 32-row slices that sit anywhere in global memory: LDS rows [0, 32) come from slice
+// `lo`, rows [32, 64) from slice `hi` (the LDS layout is that of TileStage<D, 64, THREADS>).  Every copy
+// instruction of a wave covers 64 / (D / 8) <= 16 consecutive rows starting at a multiple of that, so it stays
+// inside one slice and only its (wave-uniform) base pointer depends on which.
+template <int D, int THREADS>
+struct SliceStage {
+    static constexpr int NCH = D / 8;
+    static constexpr int CHUNKS = 64 * NCH;
+    static constexpr int CPT = (CHUNKS + THREADS - 1) / THREADS;
+    static constexpr bool EXACT = (CHUNKS % THREADS) == 0;
+    unsigned goff[CPT];
+    int wave_first;  // first chunk slot this wave fills with instruction 0
+
+    __device__ __forceinline__ void setup(int64_t row_stride_bytes, int tid) {
+        wave_first = __builtin_amdgcn_readfirstlane(tid & ~63);
+#pragma unroll
+        for (int i = 0; i < CPT; ++i) {
+            const int id = tid + THREADS * i;
+            const int row = id / NCH, pc = id % NCH;
+            goff[i] = (unsigned)((row & 31) * row_stride_bytes + (pc ^ swz<D>(row)) * 16);
+        }
+    }
+    // lo / hi: first row of the two slices in global memory, tile_lds: lds_addr() of the LDS tile (wave-uniform)
+    template <int SITE = 0>
+    __device__ __forceinline__ void issue(int i, const char* lo, const char* hi, unsigned tile_lds) const {
+        if (EXACT || wave_first + THREADS * i < CHUNKS) {
+            const bool upper = (wave_first + THREADS * i) / NCH >= 32;
+            dma_b128<SITE>(upper ? hi : lo, goff[i], tile_lds + (unsigned)(THREADS * i + wave_first) * 16u);
+        }
+    }
+    // synchronous, zero-filling copy of ONE slice with only rows_valid (<= 32) rows in range into LDS rows
+    // [0, 32); rows [32, 64) are zeroed
+    __device__ __forceinline__ void load_ragged(const char* slice_base, u32x4* tile, int rows_valid, int tid) const {
+#pragma unroll
+        for (int i = 0; i < CPT; ++i) {
+            const int id = tid + THREADS * i;
+            u32x4 z = {0u, 0u, 0u, 0u};
+            if ((EXACT || id < CHUNKS) && id / NCH < rows_valid) z = *(const u32x4*)(slice_base + goff[i]);
+            if (EXACT || id < CHUNKS) tile[id] = z;
+        }
+    }
+};
+
 // One wave copies `DWORDS` consecutive dwords (a multiple of 64) global -> LDS asynchronously.
 template <int DWORDS>
 __device__ __forceinline__ void copy_dwords_async(const void* src, void* dst_lds, int lane) {
@@ -104,49 +147,93 @@ __device__ __forceinline__ void copy_dwords_async(const void* src, void* dst_lds
     for (int i = 0; i < DWORDS / 64; ++i) dma_b32(src, (unsigned)(lane * 4 + 256 * i), dst + 256u * i);
 }
 
-// List, in ascending order, the 64-key tiles a 128-row query block has to visit.
-// entry = (tile << 2) | cls ; cls 1: evaluate the mask, cls 2: every pair allowed.
-// A tile is "full" only when both of its 32-column flags say so AND it has no column past
+// The 32-row slice each of the four waves of a forward / dQ workgroup works on, and the row of tile classes
+// (one byte per 32-key column tile: 0 empty, 1 partial, 2 full) that says which keys that slice needs.
+// Without a plan the workgroup is a 128-row block in natural order and every wave reads the block's flag row;
+// with one, group `grp` takes the next four slices of the sorted order and every slice has a class row of its own.
+struct WaveSlices {
+    int slice[4];             // -1: no slice (the wave idles through the key loop)
+    const int8_t* cls_row[4]; // null where slice is -1
+};
+
+__device__ __forceinline__ WaveSlices pick_wave_slices(const AttnParams& p, int b, int grp) {
+    WaveSlices w;
+    if (p.fine != nullptr) {
+        const int* ord = p.order + (int64_t)b * p.order_sb + 4 * grp;
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+            w.slice[x] = ord[x];
+            w.cls_row[x] = w.slice[x] >= 0
+                               ? (const int8_t*)p.fine + (int64_t)b * p.fine_sb + (int64_t)w.slice[x] * p.fine_ss
+                               : nullptr;
+        }
+    } else {
+        const int m = p.num_m - 1 - grp;  // late query blocks (most keys under causality) first
+        const int8_t* row = p.flags + (int64_t)b * p.flags_sb + (int64_t)m * p.flags_sm;
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+            w.slice[x] = 4 * m + x;
+            w.cls_row[x] = row;
+        }
+    }
+    return w;
+}
+
+// List, in ascending order, the 64-key tiles the four slices of a workgroup have to visit.
+// entry = (tile << 8) | c0 | c1 << 2 | c2 << 4 | c3 << 6 ; c_w is the class of the tile for wave w's slice:
+// 0 nothing to do, 1 evaluate the mask, 2 every pair allowed.
+// A tile is "full" for a slice only when both of its 32-column classes say so AND it has no column past
 // the end of the sequence (those columns must still be masked out of the softmax).
 // Executed by wave 0; the caller synchronizes before reading.
-__device__ __forceinline__ void build_key_tile_list(const int8_t* flag_row, int num_n, int S, int lane,
-                                                    int* list, int* count_out) {
+__device__ __forceinline__ void build_key_tile_list(const WaveSlices& ws, int num_n, int S, int lane, int* list,
+                                                    int* count_out) {
     const int nkt = (S + 63) >> 6;
     int count = 0;
     for (int base = 0; base < nkt; base += 64) {
         const int kt = base + lane;
-        int cls = 0;
+        int packed = 0;
         if (kt < nkt) {
-            const int f0 = flag_row[2 * kt];
-            const int f1 = (2 * kt + 1 < num_n) ? flag_row[2 * kt + 1] : 0;
-            if (f0 > 0 || f1 > 0) cls = (f0 == 2 && f1 == 2 && (kt + 1) * 64 <= S) ? 2 : 1;
+            const bool second = 2 * kt + 1 < num_n, inside = (kt + 1) * 64 <= S;
+#pragma unroll
+            for (int x = 0; x < 4; ++x) {
+                if (ws.cls_row[x] == nullptr) continue;  // wave-uniform
+                const int f0 = ws.cls_row[x][2 * kt];
+                const int f1 = second ? ws.cls_row[x][2 * kt + 1] : 0;
+                int cls = 0;
+                if (f0 > 0 || f1 > 0) cls = (f0 == 2 && f1 == 2 && inside) ? 2 : 1;
+                packed |= cls << (2 * x);
+            }
         }
-        const unsigned long long bal = __ballot(cls != 0);
-        if (cls) list[count + __popcll(bal & ((1ull << lane) - 1ull))] = (kt << 2) | cls;
+        const unsigned long long bal = __ballot(packed != 0);
+        if (packed) list[count + __popcll(bal & ((1ull << lane) - 1ull))] = (kt << 8) | packed;
         count += __popcll(bal);
     }
     if (lane == 0) *count_out = count;
 }
 
-// List the 128-row query blocks that have work for a 128-key tile (4 flag columns).
-// entry = (m << 8) | cls0 | cls1 << 2 | cls2 << 4 | cls3 << 6, cls_w = flag of key column w.
-__device__ __forceinline__ void build_query_block_list(const int8_t* flags_b, int64_t flags_sm, int num_m,
-                                                       int num_n, int nt, int lane, int* list,
-                                                       int* count_out) {
+// List, in ascending order, the 32-row slices that have work for a 128-key tile (4 class columns).
+// entry = (slice << 8) | c0 | c1 << 2 | c2 << 4 | c3 << 6, c_w = class of (slice, key column 4 nt + w).
+// With a plan the classes are those of the 32 x 32 tiles; without one a slice inherits the flags of its
+// 128-row block.
+__device__ __forceinline__ void build_slice_list(const AttnParams& p, int b, int nt, int lane, int* list,
+                                                 int* count_out) {
+    const int ns = (p.Sq + 31) >> 5;
     int count = 0;
-    for (int base = 0; base < num_m; base += 64) {
-        const int m = base + lane;
+    for (int base = 0; base < ns; base += 64) {
+        const int s = base + lane;
         int packed = 0;
-        if (m < num_m) {
-            const int8_t* f = flags_b + (int64_t)m * flags_sm + 4 * nt;
+        if (s < ns) {
+            const int8_t* f = p.fine != nullptr
+                                  ? (const int8_t*)p.fine + (int64_t)b * p.fine_sb + (int64_t)s * p.fine_ss + 4 * nt
+                                  : p.flags + (int64_t)b * p.flags_sb + (int64_t)(s >> 2) * p.flags_sm + 4 * nt;
 #pragma unroll
             for (int w = 0; w < 4; ++w) {
-                const int fw = (4 * nt + w < num_n) ? f[w] : 0;
+                const int fw = (4 * nt + w < p.num_n) ? f[w] : 0;
                 packed |= (fw & 3) << (2 * w);
             }
         }
         const unsigned long long bal = __ballot(packed != 0);
-        if (packed) list[count + __popcll(bal & ((1ull << lane) - 1ull))] = (m << 8) | packed;
+        if (packed) list[count + __popcll(bal & ((1ull << lane) - 1ull))] = (s << 8) | packed;
         count += __popcll(bal);
     }
     if (lane == 0) *count_out = count;

@@ -48,9 +48,11 @@ __global__ __launch_bounds__(256) void bwd_preprocess_kernel(const AttnParams p)
 
 // ---------------------------------------------------------------------------------------
 // dK, dV.  One workgroup = one 128-key tile of one (batch, kv head), 8 waves: wave w owns keys
-// [32 (w & 3), +32) and works on query rows [32 (w >> 2), +32) of every 64-row tile of Q / dO
-// that streams through LDS (double buffered), so each SIMD holds two waves whose MFMA and
-// softmax phases interleave.  K and V of the tile sit in LDS for the whole kernel and are
+// [32 (w & 3), +32) and works on rows [32 (w >> 2), +32) of every 64-row tile of Q / dO that streams
+// through LDS (double buffered), so each SIMD holds two waves whose MFMA and softmax phases
+// interleave.  A 64-row tile is a PAIR of 32-row slices taken from the list of slices that have work
+// for this key tile (they need not be neighbours in the sequence), one slice per row stream; a wave
+// whose own 32 x 32 class is "empty" sits the tile out.  K and V of the tile sit in LDS for the whole kernel and are
 // read as MFMA B operands; dK^T and dV^T (d x keys) stay in accumulators.
 // With S = Q K^T computed as queries x keys, a lane of the C fragment owns ONE key and 16
 // query rows, so P and dS feed dV^T = dO^T P and dK^T = Q^T dS as B operands from registers;
@@ -77,7 +79,7 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
     __shared__ __attribute__((aligned(16))) int64_t sQbf[2][DKDV_QT];    // raw bitfields of the rows
     __shared__ __attribute__((aligned(16))) int sQpos[2][DKDV_QT];       // their global positions (IDX only)
     __shared__ __attribute__((aligned(16))) unsigned sWq[DKDV_THREADS / 64][5][32];  // per-wave rule constants
-    __shared__ int sList[MAX_LIST / 2];
+    __shared__ int sList[MAX_SLICE_LIST];
     __shared__ int sCount;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -92,9 +94,7 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
     const int b = ub % p.B;
     const int nt = ub / p.B;  // early key tiles (most queries under causality) first
 
-    if (wave == 0)
-        build_query_block_list(p.flags + (int64_t)b * p.flags_sb, p.flags_sm, p.num_m, p.num_n, nt, lane, sList,
-                               &sCount);
+    if (wave == 0) build_slice_list(p, b, nt, lane, sList, &sCount);
 
     // ---- K, V of the tile -> LDS (once) ---------------------------------------------------
     {
@@ -130,7 +130,7 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
     for (int i = 0; i < 16; ++i) zero16[i] = 0.f;
     const float c2 = BIAS ? LOG2E : p.scale * LOG2E;  // with a bias the scores become scale * s + bias first
 
-    typedef TileStage<D, DKDV_QT, DKDV_THREADS> Stage;
+    typedef SliceStage<D, DKDV_THREADS> Stage;
     constexpr int CPT = Stage::CPT;
     // copy instructions per wave and tile: Q, dO, one of the four small rows and (IDX) the row positions
     constexpr int NLOADS = 2 * CPT + 1 + (IDX ? 1 : 0);
@@ -146,39 +146,47 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
     const int small = DENSE ? (wave & 1) : (wave & 3);
     const unsigned ldsSmall = small == 0 ? lds_addr(sLse) : small == 1 ? lds_addr(sDelta) : lds_addr(sQbf) + (small - 2) * 256u;
     const unsigned smallBytes = small < 2 ? DKDV_QT * 4u : DKDV_QT * 8u;  // per buffer
-    // Copy instruction j of the full 64-row tile (head h, first row row0) into buffer buf.
-    auto issue_copy = [&](int j, int h, int row0, int buf) {
+    // Copy instruction j of the 64-row tile made of the slices starting at rows row_lo (LDS rows 0..31) and
+    // row_hi (LDS rows 32..63) of head h, into buffer buf.  row_lo <= row_hi, or the two are the same slice.
+    auto issue_copy = [&](int j, int h, int row_lo, int row_hi, int buf) {
         if (j < CPT) {
-            const char* qbase = (const char*)p.q.ptr + 2 * ((int64_t)b * p.q.sb + (int64_t)h * p.q.sh + (int64_t)row0 * p.q.ss);
-            stQ.issue(j, qbase, ldsQ + buf * TILE_BYTES);
+            const char* qh = (const char*)p.q.ptr + 2 * ((int64_t)b * p.q.sb + (int64_t)h * p.q.sh);
+            stQ.issue(j, qh + 2 * (int64_t)row_lo * p.q.ss, qh + 2 * (int64_t)row_hi * p.q.ss, ldsQ + buf * TILE_BYTES);
         } else if (j < 2 * CPT) {
-            const char* gbase = (const char*)p.dout.ptr + 2 * ((int64_t)b * p.dout.sb + (int64_t)h * p.dout.sh + (int64_t)row0 * p.dout.ss);
-            stDO.issue(j - CPT, gbase, ldsDO + buf * TILE_BYTES);
+            const char* gh = (const char*)p.dout.ptr + 2 * ((int64_t)b * p.dout.sb + (int64_t)h * p.dout.sh);
+            stDO.issue(j - CPT, gh + 2 * (int64_t)row_lo * p.dout.ss, gh + 2 * (int64_t)row_hi * p.dout.ss,
+                       ldsDO + buf * TILE_BYTES);
         } else if (j == 2 * CPT) {
-            const int64_t off = ((int64_t)b * p.Hq + h) * p.Sq_rounded + row0;
-            const void* src = small == 0 ? (const void*)(p.lse + off)
-                              : small == 1 ? (const void*)(p.delta + off)
-                                           : (const void*)((const char*)(bfrow + row0) + (small - 2) * 256);
-            dma_b32(src, (unsigned)(lane * 4), ldsSmall + buf * smallBytes);
-        } else {  // 64 row positions; every wave writes the same values
-            dma_b32(p.posq + row0, (unsigned)(lane * 4), lds_addr(sQpos) + buf * (DKDV_QT * 4u));
+            if (small < 2) {
+                // 32 floats of each slice: lanes 32..63 are moved from "the rows after row_lo + 31" to row_hi
+                const int64_t off = ((int64_t)b * p.Hq + h) * p.Sq_rounded + row_lo;
+                const unsigned voff = (unsigned)(lane * 4 + (lane >= 32 ? (row_hi - row_lo - 32) * 4 : 0));
+                dma_b32(small == 0 ? (const void*)(p.lse + off) : (const void*)(p.delta + off), voff,
+                        ldsSmall + buf * smallBytes);
+            } else {  // 32 int64 bitfields = 64 dwords: of slice lo (small == 2) or slice hi (small == 3)
+                dma_b32(bfrow + (small == 2 ? row_lo : row_hi), (unsigned)(lane * 4), ldsSmall + buf * smallBytes);
+            }
+        } else {  // 2 x 32 row positions; every wave writes the same values
+            const unsigned voff = (unsigned)(lane * 4 + (lane >= 32 ? (row_hi - row_lo - 32) * 4 : 0));
+            dma_b32(p.posq + row_lo, voff, lds_addr(sQpos) + buf * (DKDV_QT * 4u));
         }
     };
 
-    // One 64-row tile (rows row0.., held in buffer cur) against this wave's 32 keys.  With PREFETCH the
-    // copies of the next tile (head h_next, rows row0_next..) into the other buffer are issued one per MFMA
-    // of the S / dP phase, or back to back when this wave's own flag says there is nothing to compute.
+    // One 64-row tile held in buffer cur against this wave's 32 keys; the wave's 32 rows sit at sequence
+    // rows myrow0.. and its class for them is cls.  With PREFETCH the copies of the next tile (head h_next,
+    // slices at rows lo_next / hi_next) into the other buffer are issued one per MFMA of the S / dP phase, or
+    // back to back when this wave has nothing to compute.
     const int qr = 32 * st;  // this wave's rows inside the 64-row tile
     // The wave's flag class is extracted with a per-lane copy of the key group number on purpose: a branch
     // condition the compiler can prove wave-uniform makes it restructure the loop around that branch, and the
     // result needs far more registers than a wave has.
     const int kg_lane = (tid >> 6) & 3;
-    auto tile_step = [&](auto prefetch, int cur, int cls, int h_cur, int row0, int h_next, int row0_next) {
+    auto tile_step = [&](auto prefetch, int cur, int cls, int h_cur, int myrow0, int h_next, int lo_next, int hi_next) {
         constexpr bool PREFETCH = decltype(prefetch)::value;
         if (cls == 0) {
             if (PREFETCH) {
 #pragma unroll
-                for (int j = 0; j < NLOADS; ++j) issue_copy(j, h_next, row0_next, cur ^ 1);
+                for (int j = 0; j < NLOADS; ++j) issue_copy(j, h_next, lo_next, hi_next, cur ^ 1);
             }
             return;
         }
@@ -206,7 +214,7 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
                     dp = T::mfma(a[j], bb[j], j < 2 ? zero16 : dp);
                 else
                     s = T::mfma(a[j], bb[j], j < 2 ? zero16 : s);
-                if (PREFETCH && j < NLOADS) issue_copy(j, h_next, row0_next, cur ^ 1);
+                if (PREFETCH && j < NLOADS) issue_copy(j, h_next, lo_next, hi_next, cur ^ 1);
             }
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -218,7 +226,7 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
             const int64_t col = (int64_t)b * p.bias_sb + (int64_t)h_cur * p.bias_sh + key;
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
-                const int row = row0 + qr + 8 * (i >> 2) + 4 * hi + (i & 3);
+                const int row = myrow0 + 8 * (i >> 2) + 4 * hi + (i & 3);
                 float bv = 0.f;
                 if (kvalid && row < Sq) bv = load_bias1<T>(p.bias, col + (int64_t)row * p.bias_sm, p.bias_f32 != 0);
                 s[i] = fmaf(s[i], p.scale, bv);
@@ -233,11 +241,11 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
         if (DENSE) {
             if (cls == 1) {
                 // mask bytes of this lane's key column, one per row of the C fragment
-                const uint8_t* mcol = p.mask + ((int64_t)b * Sq + row0 + qr) * Sk + key;
+                const uint8_t* mcol = p.mask + ((int64_t)b * Sq + myrow0) * Sk + key;
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
                     const int r = 8 * (i >> 2) + 4 * hi + (i & 3);
-                    bool a = kvalid && row0 + qr + r < Sq;
+                    bool a = kvalid && myrow0 + r < Sq;
                     if (a && p.mask != nullptr) a = mcol[(int64_t)r * Sk] != 0;
                     s[i] = a ? s[i] : 0.f;
                 }
@@ -249,7 +257,7 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
             const unsigned mlo = (unsigned)mine, mhi = (unsigned)((uint64_t)mine >> 32);
             const unsigned flo = __builtin_amdgcn_readfirstlane(mlo), fhi = __builtin_amdgcn_readfirstlane(mhi);
             bool uniform = (mlo == flo) & (mhi == fhi);
-            int qpos0 = row0 + qr;  // position of this wave's first row
+            int qpos0 = myrow0;  // position of this wave's first row
             if (IDX) {              // ... and the 32 rows must sit at consecutive positions
                 const int rel0 = sQpos[cur][qr + l32] - l32;
                 qpos0 = __builtin_amdgcn_readfirstlane(rel0);
@@ -266,7 +274,7 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
                 // rule constants of this wave's 32 rows, derived once per row (lane r < 32 takes row r) and
                 // handed to all lanes through a wave-private LDS scratch
                 {
-                    const QueryBits qb = make_query_bits(mine, IDX ? sQpos[cur][qr + l32] : row0 + qr + l32);
+                    const QueryBits qb = make_query_bits(mine, IDX ? sQpos[cur][qr + l32] : myrow0 + l32);
                     if (hi == 0) {
                         sWq[wave][0][l32] = qb.a_lo;
                         sWq[wave][1][l32] = qb.a_hi;
@@ -332,47 +340,61 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
 
     __syncthreads();
     const int n_all = sCount;
-    // The last 128-row block of a sequence whose length is not a multiple of 128 (always the last list entry)
-    // is staged synchronously, with neutral values for the rows past the end, after the main loop.
-    const bool ragged = (Sq & (BLOCK_M - 1)) != 0 && n_all > 0 &&
-                        (__builtin_amdgcn_readfirstlane(sList[n_all > 0 ? n_all - 1 : 0]) >> 8) == p.num_m - 1;
+    // The last slice of a sequence whose length is not a multiple of 32 (always the last list entry) is
+    // staged synchronously, with neutral values for the rows past the end, after the main loop.
+    const bool ragged = (Sq & 31) != 0 && n_all > 0 &&
+                        (__builtin_amdgcn_readfirstlane(sList[n_all > 0 ? n_all - 1 : 0]) >> 8) == ((Sq - 1) >> 5);
     const int n = n_all - (ragged ? 1 : 0);
-    // Main loop: tiles t = 0 .. 2 n G - 1 -> (q head g of the group, list entry, 64-row half).  Query blocks are
-    // visited from the LAST one down: the workgroups of one kv head that are resident together then read the
-    // same Q / dO tile at about the same time, and all but the first of them find it in L2.
-    const int total = n * 2 * G;
+    // Main loop: the listed slices are taken in pairs from the END of the list (the workgroups of one kv head
+    // that are resident together then read the same Q / dO rows at about the same time, and all but the first
+    // of them find them in L2); pair r = entries n - 2 - 2 r (row stream 0) and n - 1 - 2 r (row stream 1).
+    // An odd count leaves the first entry alone: its pair repeats it with all classes cleared for stream 0.
+    // The q heads of the group follow one another: tile t = (head t / npairs, pair t % npairs).
+    const int npairs = (n + 1) >> 1;
+    const int total = npairs * G;
     if (total > 0) {
-        // (g, r) of the tile being computed and of the next two tiles; r counts 0 .. 2n-1 inside a head
-        auto entry_of = [&](int r) { return sList[n - 1 - (r >> 1)]; };
-        auto row0_of = [&](int entry, int r) { return (entry >> 8) * BLOCK_M + (1 - (r & 1)) * DKDV_QT; };
-        int g_cur = 0, r_cur = 0;
-        int g_nxt = 0, r_nxt = 1;  // 2 n >= 2, so tile 1 is in head 0
-        int entry = __builtin_amdgcn_readfirstlane(entry_of(0));
-        int next = __builtin_amdgcn_readfirstlane(entry_of(1));
+        auto entry_hi = [&](int r) { return sList[n - 1 - 2 * r]; };
+        auto entry_lo = [&](int r) { return n - 2 - 2 * r >= 0 ? sList[n - 2 - 2 * r] : (sList[0] & ~0xFF); };
+        auto advance = [&](int& g, int& r) {
+            if (++r == npairs) {
+                r = 0;
+                ++g;
+            }
+        };
+        int g_cur = 0, r_cur = 0, g_nxt = 0, r_nxt = 0;
+        advance(g_nxt, r_nxt);
+        int e_lo = __builtin_amdgcn_readfirstlane(entry_lo(0)), e_hi = __builtin_amdgcn_readfirstlane(entry_hi(0));
+        int n_lo = e_lo, n_hi = e_hi;
+        if (g_nxt < G) {
+            n_lo = __builtin_amdgcn_readfirstlane(entry_lo(r_nxt));
+            n_hi = __builtin_amdgcn_readfirstlane(entry_hi(r_nxt));
+        }
 #pragma unroll
-        for (int j = 0; j < NLOADS; ++j) issue_copy(j, hk * G, row0_of(entry, 0), 0);
+        for (int j = 0; j < NLOADS; ++j) issue_copy(j, hk * G, (e_lo >> 8) * 32, (e_hi >> 8) * 32, 0);
         wait_async();
         __syncthreads();
         for (int it = 0; it < total; ++it) {
             const int cur = it & 1;
-            // tile after next: its list entry is requested now and picked up at the end of the iteration
-            int g_aft = g_nxt, r_aft = r_nxt + 1;
-            if (r_aft == 2 * n) {
-                r_aft = 0;
-                ++g_aft;
-            }
-            const int after = entry_of(g_aft < G ? r_aft : 0);
+            // pair after next: its list entries are requested now and picked up at the end of the iteration
+            int g_aft = g_nxt, r_aft = r_nxt;
+            advance(g_aft, r_aft);
+            const int ra = g_aft < G ? r_aft : 0;
+            const int a_lo = entry_lo(ra), a_hi = entry_hi(ra);
             // past the last tile the copies simply fetch it again (into the buffer nobody reads any more)
             const bool more = it + 1 < total;
             const int h_next = hk * G + (more ? g_nxt : g_cur);
-            const int row0_next = more ? row0_of(next, r_nxt) : row0_of(entry, r_cur);
-            tile_step(std::true_type{}, cur, (entry >> (2 * kg_lane)) & 3, hk * G + g_cur, row0_of(entry, r_cur), h_next, row0_next);
+            const int lo_next = ((more ? n_lo : e_lo) >> 8) * 32, hi_next = ((more ? n_hi : e_hi) >> 8) * 32;
+            const int mine = st ? e_hi : e_lo;
+            tile_step(std::true_type{}, cur, (mine >> (2 * kg_lane)) & 3, hk * G + g_cur, (mine >> 8) * 32, h_next, lo_next,
+                      hi_next);
             g_cur = g_nxt;
             r_cur = r_nxt;
             g_nxt = g_aft;
             r_nxt = r_aft;
-            entry = next;
-            next = __builtin_amdgcn_readfirstlane(after);
+            e_lo = n_lo;
+            e_hi = n_hi;
+            n_lo = __builtin_amdgcn_readfirstlane(a_lo);
+            n_hi = __builtin_amdgcn_readfirstlane(a_hi);
             wait_async();
             __syncthreads();
         }
@@ -380,11 +402,9 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
     if (ragged) {
         wait_async();  // K, V of the tile, in case the main loop had nothing to do
         const int entry = __builtin_amdgcn_readfirstlane(sList[n_all - 1]);
-        for (int t = 0; t < 2 * G; ++t) {
-            const int g = t >> 1;
-            const int row0 = (entry >> 8) * BLOCK_M + (t & 1) * DKDV_QT;
-            const int rows = Sq - row0;  // rows of the tile inside the sequence
-            if (rows <= 0) continue;
+        const int row0 = (entry >> 8) * 32;
+        const int rows = Sq - row0;  // rows of the slice inside the sequence (1..31)
+        for (int g = 0; g < G; ++g) {
             const int h = hk * G + g;
             __syncthreads();  // everybody is done with buffer 0
             stQ.load_ragged((const char*)p.q.ptr + 2 * ((int64_t)b * p.q.sb + (int64_t)h * p.q.sh + (int64_t)row0 * p.q.ss), sQ[0], rows, tid);
@@ -398,7 +418,8 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
                 if (IDX) sQpos[0][tid] = ok ? p.posq[row0 + tid] : 0;
             }
             __syncthreads();
-            tile_step(std::false_type{}, 0, (entry >> (2 * kg_lane)) & 3, h, row0, 0, 0);
+            // the slice sits in LDS rows 0..31: row stream 0 computes it, row stream 1 has nothing to do
+            tile_step(std::false_type{}, 0, st ? 0 : (entry >> (2 * kg_lane)) & 3, h, row0, 0, 0, 0);
         }
     }
     // every copy has landed and every wave is done with the tiles: the epilogue reuses the tile arrays
@@ -495,6 +516,7 @@ __global__ __launch_bounds__(DQ_THREADS, D == 128 ? 2 : 3) void bwd_dq_kernel(co
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int hi = lane >> 5, l32 = lane & 31, half16 = (lane >> 4) & 1;
+    const int wave_lane = tid >> 6;
     const int Sq = p.Sq, Sk = p.Sk;
     const int G = p.Hq / p.Hkv;
 
@@ -503,15 +525,14 @@ __global__ __launch_bounds__(DQ_THREADS, D == 128 ? 2 : 3) void bwd_dq_kernel(co
     const int hk = unit % p.Hkv;
     const int ub = unit / p.Hkv;
     const int b = ub % p.B;
-    const int m = p.num_m - 1 - ub / p.B;
     const int h = hk * G + g;
+    const WaveSlices ws = pick_wave_slices(p, b, ub / p.B);  // group 0 is the heaviest
 
-    if (wave == 0)
-        build_key_tile_list(p.flags + (int64_t)b * p.flags_sb + (int64_t)m * p.flags_sm, p.num_n, Sk, lane,
-                            sList, &sCount);
+    if (wave == 0) build_key_tile_list(ws, p.num_n, Sk, lane, sList, &sCount);
 
-    const int qrow = m * BLOCK_M + wave * 32 + l32;
-    const bool qvalid = qrow < Sq;
+    const int slice = __builtin_amdgcn_readfirstlane(wave == 0 ? ws.slice[0] : wave == 1 ? ws.slice[1] : wave == 2 ? ws.slice[2] : ws.slice[3]);
+    const int qrow = (slice < 0 ? 0 : slice) * 32 + l32;
+    const bool qvalid = slice >= 0 && qrow < Sq;
     u32x4 qreg[KK], greg[KK];
     {
         const char* qp = (const char*)p.q.ptr + 2 * ((int64_t)b * p.q.sb + (int64_t)qrow * p.q.ss + (int64_t)h * p.q.sh);
@@ -583,7 +604,16 @@ __global__ __launch_bounds__(DQ_THREADS, D == 128 ? 2 : 3) void bwd_dq_kernel(co
     // are issued one per MFMA of the first S / dP block.
     auto tile_step = [&](auto prefetch, int cur, int entry, int kt_next) {
         constexpr bool PREFETCH = decltype(prefetch)::value;
-        const int kt = entry >> 2, cls = entry & 3;
+        // (the class is extracted with a per-lane copy of the wave number on purpose: a skip branch the compiler
+        // can prove wave-uniform makes it restructure the loop around it at the price of ~90 spilled registers)
+        const int kt = entry >> 8, cls = (entry >> (2 * wave_lane)) & 3;
+        if (cls == 0) {  // nothing for this wave's slice in the tile: only keep the copies of the next one going
+            if (PREFETCH) {
+#pragma unroll
+                for (int j = 0; j < NLOADS; ++j) issue_copy(j, kt_next, cur ^ 1);
+            }
+            return;
+        }
         const u32x4* tK = sK[cur];
         const u32x4* tV = sV[cur];
         // partial tile whose 64 keys all carry the same bitfield: the rule is one position compare
@@ -718,13 +748,13 @@ __global__ __launch_bounds__(DQ_THREADS, D == 128 ? 2 : 3) void bwd_dq_kernel(co
     // A tile that holds the end of a sequence whose length is not a multiple of 64 is always the last
     // entry of the list; it is staged synchronously (zero fill past the end) after the main loop.
     const bool ragged = (Sk & (DQ_KT - 1)) != 0 && n_all > 0 &&
-                        (__builtin_amdgcn_readfirstlane(sList[n_all > 0 ? n_all - 1 : 0]) >> 2) == ((Sk - 1) >> 6);
+                        (__builtin_amdgcn_readfirstlane(sList[n_all > 0 ? n_all - 1 : 0]) >> 8) == ((Sk - 1) >> 6);
     const int n = n_all - (ragged ? 1 : 0);
     if (n > 0) {
         int entry = __builtin_amdgcn_readfirstlane(sList[0]);
         int next = __builtin_amdgcn_readfirstlane(sList[n > 1 ? 1 : 0]);
 #pragma unroll
-        for (int j = 0; j < NLOADS; ++j) issue_copy(j, entry >> 2, 0);
+        for (int j = 0; j < NLOADS; ++j) issue_copy(j, entry >> 8, 0);
         wait_async();
         __syncthreads();
         for (int it = 0; it < n; ++it) {
@@ -732,7 +762,7 @@ __global__ __launch_bounds__(DQ_THREADS, D == 128 ? 2 : 3) void bwd_dq_kernel(co
             // entry after next, requested now and picked up at the end of the iteration; past the end of the
             // list the last tile is simply copied again (into the buffer nobody reads any more)
             const int after = sList[it + 2 < n ? it + 2 : n - 1];
-            tile_step(std::true_type{}, cur, entry, next >> 2);
+            tile_step(std::true_type{}, cur, entry, next >> 8);
             entry = next;
             next = __builtin_amdgcn_readfirstlane(after);
             wait_async();
@@ -741,7 +771,7 @@ __global__ __launch_bounds__(DQ_THREADS, D == 128 ? 2 : 3) void bwd_dq_kernel(co
     }
     if (ragged) {
         const int entry = __builtin_amdgcn_readfirstlane(sList[n_all - 1]);
-        const int kt = entry >> 2, rows = Sk - kt * DQ_KT;
+        const int kt = entry >> 8, rows = Sk - kt * DQ_KT;
         stK.load_ragged(kbase + kt * k_ts, sK[0], rows, tid);
         stV.load_ragged(vbase + kt * v_ts, sV[0], rows, tid);
         if (!DENSE && tid < DQ_KT) {

@@ -3,10 +3,11 @@
 // :1292-1436, which a single pass over the keys makes unnecessary).
 //
 // Work decomposition
-//   workgroup  = 128 query rows of one (batch, q head); 4 waves x 32 rows.
-//   key loop   = 64-key tiles taken from the flag row of this query block: empty tiles are
-//                never touched, "full" tiles skip the mask, "partial" tiles evaluate the
-//                bitfield rule in registers.
+//   workgroup  = four 32-row slices of one (batch, q head), one per wave: a 128-row block, or, with a plan,
+//                four slices that need about the same keys (sorted slice order).
+//   key loop   = 64-key tiles taken from the class rows of those slices: tiles no slice needs are never
+//                touched; a wave skips the tiles its own slice does not need, skips the mask where every
+//                pair of its slice is allowed, and evaluates the bitfield rule in registers otherwise.
 //   K/V tiles  = double buffered in LDS; the next tile is copied global -> LDS directly while
 //                the current one is consumed.
 // Math layout
@@ -53,16 +54,15 @@ __global__ __launch_bounds__(FWD_THREADS, D == 128 ? 2 : 3) void fwd_kernel(cons
     const int hk = unit % p.Hkv;
     const int ub = unit / p.Hkv;
     const int b = ub % p.B;
-    const int m = p.num_m - 1 - ub / p.B;  // late query blocks (most keys under causality) first
     const int h = hk * G + g;
+    const WaveSlices ws = pick_wave_slices(p, b, ub / p.B);  // group 0 is the heaviest
 
-    if (wave == 0)
-        build_key_tile_list(p.flags + (int64_t)b * p.flags_sb + (int64_t)m * p.flags_sm, p.num_n, Sk, lane,
-                            sList, &sCount);
+    if (wave == 0) build_key_tile_list(ws, p.num_n, Sk, lane, sList, &sCount);
 
     // ---- per-lane query state -------------------------------------------------------
-    const int qrow = m * BLOCK_M + wave * 32 + l32;
-    const bool qvalid = qrow < Sq;
+    const int slice = __builtin_amdgcn_readfirstlane(wave == 0 ? ws.slice[0] : wave == 1 ? ws.slice[1] : wave == 2 ? ws.slice[2] : ws.slice[3]);
+    const int qrow = (slice < 0 ? 0 : slice) * 32 + l32;
+    const bool qvalid = slice >= 0 && qrow < Sq;
     u32x4 qreg[KK];
     {
         const char* qp = (const char*)p.q.ptr + 2 * ((int64_t)b * p.q.sb + (int64_t)qrow * p.q.ss + (int64_t)h * p.q.sh);
@@ -133,7 +133,14 @@ __global__ __launch_bounds__(FWD_THREADS, D == 128 ? 2 : 3) void fwd_kernel(cons
     // buffer are issued one per MFMA of the S phase, where the wave has nothing else to wait for.
     auto tile_step = [&](auto prefetch, int cur, int entry, int kt_next) {
         constexpr bool PREFETCH = decltype(prefetch)::value;
-        const int kt = entry >> 2, cls = entry & 3;
+        const int kt = entry >> 8, cls = (entry >> (2 * wave)) & 3;
+        if (cls == 0) {  // nothing for this wave's slice in the tile: only keep the copies of the next one going
+            if (PREFETCH) {
+#pragma unroll
+                for (int j = 0; j < NLOADS; ++j) issue_copy(j, kt_next, cur ^ 1);
+            }
+            return;
+        }
         const u32x4* tK = sK[cur];
         const u32x4* tV = sV[cur];
 
@@ -317,13 +324,13 @@ __global__ __launch_bounds__(FWD_THREADS, D == 128 ? 2 : 3) void fwd_kernel(cons
     // A tile that holds the end of a sequence whose length is not a multiple of 64 is always the last
     // entry of the list; it is staged synchronously (zero fill past the end) after the main loop.
     const bool ragged = (Sk & (FWD_KT - 1)) != 0 && n_all > 0 &&
-                        (__builtin_amdgcn_readfirstlane(sList[n_all > 0 ? n_all - 1 : 0]) >> 2) == ((Sk - 1) >> 6);
+                        (__builtin_amdgcn_readfirstlane(sList[n_all > 0 ? n_all - 1 : 0]) >> 8) == ((Sk - 1) >> 6);
     const int n = n_all - (ragged ? 1 : 0);
     if (n > 0) {
         int entry = __builtin_amdgcn_readfirstlane(sList[0]);
         int next = __builtin_amdgcn_readfirstlane(sList[n > 1 ? 1 : 0]);
 #pragma unroll
-        for (int j = 0; j < NLOADS; ++j) issue_copy(j, entry >> 2, 0);
+        for (int j = 0; j < NLOADS; ++j) issue_copy(j, entry >> 8, 0);
         wait_async();
         __syncthreads();
         for (int it = 0; it < n; ++it) {
@@ -331,7 +338,7 @@ __global__ __launch_bounds__(FWD_THREADS, D == 128 ? 2 : 3) void fwd_kernel(cons
             // entry after next, requested now and picked up at the end of the iteration; past the end of the
             // list the last tile is simply copied again (into the buffer nobody reads any more)
             const int after = sList[it + 2 < n ? it + 2 : n - 1];
-            tile_step(std::true_type{}, cur, entry, next >> 2);
+            tile_step(std::true_type{}, cur, entry, next >> 8);
             entry = next;
             next = __builtin_amdgcn_readfirstlane(after);
             wait_async();
@@ -340,7 +347,7 @@ __global__ __launch_bounds__(FWD_THREADS, D == 128 ? 2 : 3) void fwd_kernel(cons
     }
     if (ragged) {
         const int entry = __builtin_amdgcn_readfirstlane(sList[n_all - 1]);
-        const int kt = entry >> 2, rows = Sk - kt * FWD_KT;
+        const int kt = entry >> 8, rows = Sk - kt * FWD_KT;
         stK.load_ragged(kbase + kt * k_ts, sK[0], rows, tid);
         stV.load_ragged(vbase + kt * v_ts, sV[0], rows, tid);
         if (!DENSE && tid < FWD_KT) {
@@ -354,7 +361,7 @@ __global__ __launch_bounds__(FWD_THREADS, D == 128 ? 2 : 3) void fwd_kernel(cons
     // ---- epilogue: normalize, write O (q dtype) and LSE (natural log) -------------------
     const float ltot = half_swap_sum(l_i);
     const float inv = ltot > 0.f ? 1.f / ltot : 0.f;
-    if (hi == 0)
+    if (hi == 0 && slice >= 0)
         p.lse[((int64_t)b * p.Hq + h) * p.Sq_rounded + qrow] =
             ltot > 0.f ? (m_i * c2 + __builtin_amdgcn_logf(ltot)) * LN2 : -INFINITY;
     if (qvalid) {

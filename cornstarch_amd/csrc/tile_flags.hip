@@ -16,11 +16,16 @@ constexpr int FLAG_WAVES = 4;
 constexpr int FLAG_TILES_PER_WAVE = 2;  // few tiles per wave: the grid, not the wave, covers the row of tiles
 constexpr int FLAG_COLS_PER_BLOCK = FLAG_WAVES * FLAG_TILES_PER_WAVE;
 
+// FINE: also write the class of every 32-row x 32-column tile (the four row slices of each flag tile) to
+// fine[b][4 m + w][n]; same 0 / 1 / 2 meaning, "full" again over the in-range cells only.
+template <bool FINE>
 __global__ __launch_bounds__(FLAG_WAVES * 64) void tile_flags_kernel(const int64_t* __restrict__ bf,
                                                                     int64_t bf_stride_b,
                                                                     int8_t* __restrict__ flags,
                                                                     int64_t flags_stride_b,
-                                                                    int64_t flags_stride_m, int S, int num_n) {
+                                                                    int64_t flags_stride_m, int S, int num_n,
+                                                                    uint8_t* __restrict__ fine, int64_t fine_sb,
+                                                                    int64_t fine_ss) {
     __shared__ int64_t q_bits[BLOCK_M];
     const int b = blockIdx.z, m = blockIdx.y;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -55,30 +60,57 @@ __global__ __launch_bounds__(FLAG_WAVES * 64) void tile_flags_kernel(const int64
                 const int64_t M = (((int64_t)1) << 62) - 1;
                 const int64_t qb = q0 & M, kb = k0 & M;
                 int8_t f;
+                const int r0 = m * BLOCK_M, c0 = n * BLOCK_N;
                 if (q0 & 1) {  // text rows: causal over keys that share a bit
-                    const int r0 = m * BLOCK_M, c0 = n * BLOCK_N;
                     f = (qb & kb) == 0 ? 0 : r0 >= c0 + BLOCK_N - 1 ? 2 : r0 + BLOCK_M - 1 < c0 ? 0 : 1;
                 } else {
                     f = (qb == kb && qb != 0) ? 2 : 0;
                 }
                 if (lane == 0) flags[(int64_t)b * flags_stride_b + (int64_t)m * flags_stride_m + n] = f;
+                if (FINE && lane < 4) {  // the same closed form for the 32 rows of slice `lane`
+                    const int rs = r0 + 32 * lane;
+                    int8_t fw = f;
+                    if (q0 & 1) fw = (qb & kb) == 0 ? 0 : rs >= c0 + BLOCK_N - 1 ? 2 : rs + 31 < c0 ? 0 : 1;
+                    fine[(int64_t)b * fine_sb + (int64_t)(4 * m + lane) * fine_ss + n] = (uint8_t)fw;
+                }
                 continue;
             }
         }
-        int cnt = 0;
+        int cnt_a = 0, cnt_b = 0;  // rows [64 half, +32) and [64 half + 32, +32)
 #pragma unroll 8
-        for (int r = 0; r < 64; ++r) {
+        for (int r = 0; r < 32; ++r) {
             const int ri = half * 64 + r;
-            cnt += allow_rule(q_bits[ri], kf, (int64_t)m * BLOCK_M + ri, j) ? 1 : 0;
+            cnt_a += allow_rule(q_bits[ri], kf, (int64_t)m * BLOCK_M + ri, j) ? 1 : 0;
+            cnt_b += allow_rule(q_bits[ri + 32], kf, (int64_t)m * BLOCK_M + ri + 32, j) ? 1 : 0;
         }
+        const int cols_in_range = min(BLOCK_N, S - n * BLOCK_N);
+        if (FINE) {
 #pragma unroll
-        for (int off = 32; off > 0; off >>= 1) cnt += __shfl_xor(cnt, off);
-        if (lane == 0) {
-            const int cols_in_range = min(BLOCK_N, S - n * BLOCK_N);
-            int8_t f = 0;
-            if (cnt > 0) f = 1;
-            if (cnt == rows_in_range * cols_in_range) f = 2;  // full over in-range cells (:149-153)
-            flags[(int64_t)b * flags_stride_b + (int64_t)m * flags_stride_m + n] = f;
+            for (int off = 16; off > 0; off >>= 1) {  // over the 32 columns, inside each half of the wave
+                cnt_a += __shfl_xor(cnt_a, off);
+                cnt_b += __shfl_xor(cnt_b, off);
+            }
+            if ((lane & 31) == 0) {
+#pragma unroll
+                for (int x = 0; x < 2; ++x) {
+                    const int w = 2 * half + x, c = x ? cnt_b : cnt_a;
+                    const int rows = max(0, min(32, S - (m * BLOCK_M + 32 * w)));
+                    fine[(int64_t)b * fine_sb + (int64_t)(4 * m + w) * fine_ss + n] =
+                        (uint8_t)(c == 0 ? 0 : c == rows * cols_in_range ? 2 : 1);
+                }
+            }
+            int cnt = cnt_a + cnt_b;
+            cnt += __shfl_xor(cnt, 32);
+            if (lane == 0)
+                flags[(int64_t)b * flags_stride_b + (int64_t)m * flags_stride_m + n] =
+                    cnt == 0 ? 0 : cnt == rows_in_range * cols_in_range ? 2 : 1;  // full over in-range cells (:149-153)
+        } else {
+            int cnt = cnt_a + cnt_b;
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) cnt += __shfl_xor(cnt, off);
+            if (lane == 0)
+                flags[(int64_t)b * flags_stride_b + (int64_t)m * flags_stride_m + n] =
+                    cnt == 0 ? 0 : cnt == rows_in_range * cols_in_range ? 2 : 1;  // full over in-range cells (:149-153)
         }
     }
 }
@@ -183,8 +215,79 @@ int launch_tile_flags(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int
                       int64_t flags_stride_m, int B, int S, hipStream_t stream) {
     const int num_m = (S + BLOCK_M - 1) / BLOCK_M, num_n = (S + BLOCK_N - 1) / BLOCK_N;
     dim3 grid((num_n + FLAG_COLS_PER_BLOCK - 1) / FLAG_COLS_PER_BLOCK, num_m, B);
-    hipLaunchKernelGGL(tile_flags_kernel, grid, dim3(FLAG_WAVES * 64), 0, stream, bf, bf_stride_b, flags,
-                       flags_stride_b, flags_stride_m, S, num_n);
+    hipLaunchKernelGGL(tile_flags_kernel<false>, grid, dim3(FLAG_WAVES * 64), 0, stream, bf, bf_stride_b, flags,
+                       flags_stride_b, flags_stride_m, S, num_n, (uint8_t*)nullptr, (int64_t)0, (int64_t)0);
+    return (int)hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// Slice order.  The forward and dQ kernels give each of the four waves of a workgroup one 32-row slice and walk
+// the union of the key tiles those slices need, so four slices that need the same keys should sit together:
+//   * slices holding a text row first, by descending position (they see their whole past; the latest see most),
+//   * then the slices made of modality rows only, grouped by the OR of their bitfields (equal value = same
+//     modality = same keys), by ascending position inside a group.
+// Step 1 writes a two-word sort key per slice, step 2 ranks every slice against all others of its sequence
+// (at most MAX_PLAN_SLICES of them) and scatters; slots past the last slice are set to -1.
+__global__ __launch_bounds__(256) void slice_keys_kernel(const int64_t* __restrict__ bf, int64_t bf_stride_b, int S,
+                                                         int ns, int slots, unsigned long long* __restrict__ keys) {
+    const int s = blockIdx.x * 256 + threadIdx.x, b = blockIdx.y;
+    if (s >= slots) return;
+    unsigned long long k1 = ~0ull, k2 = ~0ull;  // slots without rows sort last
+    if (s < ns) {
+        const int64_t M = (((int64_t)1) << 62) - 1;
+        const int64_t* row = bf + (int64_t)b * bf_stride_b;
+        int64_t sig = 0;
+        bool text = false;
+        for (int r = 0; r < 32; ++r) {
+            const int i = s * 32 + r;
+            const int64_t f = i < S ? row[i] : 0;
+            sig |= f & M;
+            text |= (f & 1) != 0;
+        }
+        k1 = text ? 0ull : (1ull << 62) | (unsigned long long)sig;
+        k2 = text ? (unsigned long long)(ns - 1 - s) : (unsigned long long)s;
+    }
+    keys[2 * ((int64_t)b * slots + s)] = k1;
+    keys[2 * ((int64_t)b * slots + s) + 1] = k2;
+}
+
+__global__ __launch_bounds__(256) void slice_rank_kernel(const unsigned long long* __restrict__ keys, int ns, int slots,
+                                                         int* __restrict__ order, int64_t order_sb) {
+    __shared__ unsigned long long sk[2 * 256];
+    const int s = blockIdx.x * 256 + threadIdx.x, b = blockIdx.y;
+    const unsigned long long* kb = keys + 2 * (int64_t)b * slots;
+    const unsigned long long my1 = s < slots ? kb[2 * s] : 0, my2 = s < slots ? kb[2 * s + 1] : 0;
+    int rank = 0;
+    for (int base = 0; base < ns; base += 256) {
+        __syncthreads();
+        if (base + threadIdx.x < ns) {
+            sk[2 * threadIdx.x] = kb[2 * (base + threadIdx.x)];
+            sk[2 * threadIdx.x + 1] = kb[2 * (base + threadIdx.x) + 1];
+        }
+        __syncthreads();
+        const int cnt = min(256, ns - base);
+        for (int j = 0; j < cnt; ++j) {
+            const unsigned long long o1 = sk[2 * j], o2 = sk[2 * j + 1];
+            rank += (o1 < my1 || (o1 == my1 && o2 < my2)) ? 1 : 0;  // (k1, k2) pairs are distinct
+        }
+    }
+    if (s < ns)
+        order[(int64_t)b * order_sb + rank] = s;
+    else if (s < slots)
+        order[(int64_t)b * order_sb + s] = -1;
+}
+
+int launch_tile_plan(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int64_t flags_stride_b,
+                     int64_t flags_stride_m, uint8_t* fine, int64_t fine_sb, int64_t fine_ss, int* order,
+                     int64_t order_sb, unsigned long long* keys, int B, int S, hipStream_t stream) {
+    const int num_m = (S + BLOCK_M - 1) / BLOCK_M, num_n = (S + BLOCK_N - 1) / BLOCK_N;
+    const int ns = (S + 31) / 32, slots = 4 * num_m;
+    dim3 grid((num_n + FLAG_COLS_PER_BLOCK - 1) / FLAG_COLS_PER_BLOCK, num_m, B);
+    hipLaunchKernelGGL(tile_flags_kernel<true>, grid, dim3(FLAG_WAVES * 64), 0, stream, bf, bf_stride_b, flags,
+                       flags_stride_b, flags_stride_m, S, num_n, fine, fine_sb, fine_ss);
+    dim3 sgrid((slots + 255) / 256, B);
+    hipLaunchKernelGGL(slice_keys_kernel, sgrid, dim3(256), 0, stream, bf, bf_stride_b, S, ns, slots, keys);
+    hipLaunchKernelGGL(slice_rank_kernel, sgrid, dim3(256), 0, stream, keys, ns, slots, order, order_sb);
     return (int)hipGetLastError();
 }
 

@@ -14,7 +14,7 @@ LIB_PATH = os.path.join(_PKG_DIR, "libbam_hip.so")
 BAM_DTYPE_F16 = 0
 BAM_DTYPE_BF16 = 1
 BAM_MAX_SEQLEN = 131072
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 _i64 = ctypes.c_int64
 _int = ctypes.c_int
@@ -48,18 +48,34 @@ class Bias(ctypes.Structure):
     ]
 
 
+class Plan(ctypes.Structure):
+    """``bam_plan`` of include/bam_hip.h (host struct holding device pointers into the plan workspace)."""
+
+    _fields_ = [
+        ("fine", ctypes.c_void_p),
+        ("fine_stride_b", ctypes.c_int64),
+        ("fine_stride_s", ctypes.c_int64),
+        ("order", ctypes.c_void_p),
+        ("order_stride_b", ctypes.c_int64),
+        ("B", ctypes.c_int32),
+        ("S", ctypes.c_int32),
+    ]
+
+
 _view = ctypes.POINTER(IndexView)
 _bias = ctypes.POINTER(Bias)
+_plan = ctypes.POINTER(Plan)
 
 # name -> argtypes, exactly the prototypes of include/bam_hip.h
 SIGNATURES = {
     "bam_tile_flags": [_ptr, _i64, _ptr, _i64, _i64, _int, _int, _ptr],
     "bam_materialize_mask": [_ptr, _i64, _ptr, _int, _int, _ptr],
-    "bam_fwd": [_ptr] * 7 + [_i64] * 15 + [_int] * 5 + [_f32, _int, _bias, _ptr],
+    "bam_tile_plan": [_ptr, _i64, _ptr, _i64, _i64, _ptr, _i64, _int, _int, _plan, _ptr],
+    "bam_fwd": [_ptr] * 7 + [_i64] * 15 + [_int] * 5 + [_f32, _int, _bias, _plan, _ptr],
     "bam_bwd_preprocess": [_ptr] * 3 + [_i64] * 6 + [_int] * 5 + [_ptr],
-    "bam_bwd": [_ptr] * 11 + [_i64] * 24 + [_int] * 5 + [_f32, _int, _int, _bias, _ptr],
-    "bam_bwd_dkdv": [_ptr] * 10 + [_i64] * 21 + [_int] * 5 + [_f32, _int, _int, _bias, _ptr],
-    "bam_bwd_dq": [_ptr] * 9 + [_i64] * 18 + [_int] * 5 + [_f32, _int, _int, _bias, _ptr],
+    "bam_bwd": [_ptr] * 11 + [_i64] * 24 + [_int] * 5 + [_f32, _int, _int, _bias, _plan, _ptr],
+    "bam_bwd_dkdv": [_ptr] * 10 + [_i64] * 21 + [_int] * 5 + [_f32, _int, _int, _bias, _plan, _ptr],
+    "bam_bwd_dq": [_ptr] * 9 + [_i64] * 18 + [_int] * 5 + [_f32, _int, _int, _bias, _plan, _ptr],
     "bam_mask_tile_flags": [_ptr, _ptr, _i64, _i64, _int, _int, _int, _ptr],
     "bam_fwd_masked": [_ptr] * 7 + [_i64] * 14 + [_int] * 6 + [_f32, _int, _bias, _ptr],
     "bam_bwd_dkdv_masked": [_ptr] * 10 + [_i64] * 20 + [_int] * 6 + [_f32, _int, _int, _bias, _ptr],
@@ -93,6 +109,8 @@ def load() -> ctypes.CDLL:
     lib.bam_last_error.argtypes = []
     lib.bam_abi_version.restype = _int
     lib.bam_abi_version.argtypes = []
+    lib.bam_plan_workspace_bytes.restype = _i64
+    lib.bam_plan_workspace_bytes.argtypes = [_int, _int]
     for name, argtypes in SIGNATURES.items():
         fn = getattr(lib, name)
         fn.argtypes = argtypes

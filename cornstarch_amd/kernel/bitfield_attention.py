@@ -70,6 +70,26 @@ def materialize_bitfield_mask(bitfield_mask: torch.Tensor) -> torch.Tensor:
     return out.bool()
 
 
+class _TilePlan:
+    """What the kernels use beyond the 128 x 32 flags to skip masked work (``bam_plan`` of include/bam_hip.h):
+    the class of every 32-row x 32-key tile and an order of the 32-row slices in which neighbours need the same
+    keys.  Built together with the flags, lives in one workspace tensor, and belongs to exactly one flags tensor."""
+
+    def __init__(self, workspace: torch.Tensor, struct: "_bam_hip.Plan", flags: torch.Tensor):
+        self.workspace = workspace  # keeps the device memory alive
+        self.struct = struct
+        self.flags = flags
+
+    def byref(self):
+        import ctypes
+
+        return ctypes.byref(self.struct)
+
+
+def _plan_arg(plan: Optional["_TilePlan"]):
+    return plan.byref() if plan is not None else None
+
+
 class BitfieldUtils:
     """Cache of the tile flags ("compressed mask") of the current bitfield mask.
 
@@ -87,12 +107,31 @@ class BitfieldUtils:
     compressed_mask_cache: Optional[torch.Tensor] = None
     _cache_key = None
     _cache_owner: Optional[torch.Tensor] = None  # the bitfield tensor the cached flags belong to
+    _plan: Optional[_TilePlan] = None            # built with the cached flags; None for very long sequences
 
     @classmethod
     def clear_cache(cls):
         cls.compressed_mask_cache = None
         cls._cache_key = None
         cls._cache_owner = None
+        cls._plan = None
+
+    @classmethod
+    def plan_for(cls, compressed_mask: torch.Tensor, bitfield_mask: torch.Tensor) -> Optional[_TilePlan]:
+        """The plan that was built together with ``compressed_mask``: only when that is the cached flags tensor
+        itself and ``bitfield_mask`` is still the (unchanged) mask they were computed from.  Callers that bring
+        their own flags (re-indexed context-parallel shards, for instance) get None and the kernels work from
+        the flags alone."""
+        plan = cls._plan
+        if plan is None or plan.flags is not cls.compressed_mask_cache:
+            return None
+        # the cache keeps its flags tensor alive, so equal address and shape mean "that tensor" (autograd may hand
+        # saved tensors back as new Python objects)
+        if compressed_mask.data_ptr() != plan.flags.data_ptr() or compressed_mask.shape != plan.flags.shape:
+            return None
+        if cls._cache_key != cls._key_of(bitfield_mask):
+            return None
+        return plan
 
     @staticmethod
     def _key_of(bitfield_mask: torch.Tensor):
@@ -121,14 +160,28 @@ class BitfieldUtils:
             dtype=torch.int8,
             device=bf.device,
         )
+        plan = None
         with torch.cuda.device(bf.device):
-            _bam_hip.call(
-                "bam_tile_flags", bf.data_ptr(), bf.stride(0), out.data_ptr(), out.stride(0), out.stride(1),
-                batch_size, seq_len, _stream_ptr(bf.device),
-            )
+            ws_bytes = _bam_hip.load().bam_plan_workspace_bytes(batch_size, seq_len)
+            if ws_bytes > 0:
+                workspace = torch.empty((ws_bytes,), dtype=torch.uint8, device=bf.device)
+                struct = _bam_hip.Plan()
+                import ctypes
+
+                _bam_hip.call(
+                    "bam_tile_plan", bf.data_ptr(), bf.stride(0), out.data_ptr(), out.stride(0), out.stride(1),
+                    workspace.data_ptr(), ws_bytes, batch_size, seq_len, ctypes.byref(struct), _stream_ptr(bf.device),
+                )
+                plan = _TilePlan(workspace, struct, out)
+            else:
+                _bam_hip.call(
+                    "bam_tile_flags", bf.data_ptr(), bf.stride(0), out.data_ptr(), out.stride(0), out.stride(1),
+                    batch_size, seq_len, _stream_ptr(bf.device),
+                )
         cls.compressed_mask_cache = out
         cls._cache_key = key
         cls._cache_owner = bitfield_mask
+        cls._plan = plan
         return out
 
     @classmethod
@@ -267,6 +320,7 @@ def _bitfield_attn_forward(
     flags = compressed_mask if compressed_mask.stride(-1) == 1 else compressed_mask.contiguous()
     num_m, num_n = -(-seqlen_q // BLOCK_M), -(-seqlen_k // BLOCK_N)
     assert flags.dtype == torch.int8 and flags.shape == (batch, num_m, num_n)
+    plan = BitfieldUtils.plan_for(compressed_mask, bitfield_mask) if view is None else None
 
     seqlen_q_rounded = num_m * BLOCK_M
     lse = torch.empty((batch, nheads, seqlen_q_rounded), device=q.device, dtype=torch.float32)
@@ -279,7 +333,7 @@ def _bitfield_attn_forward(
                 flags.data_ptr(), *_strides3(qk, kk, vk, o),
                 bf.stride(0), flags.stride(0), flags.stride(1),
                 batch, seqlen_q, nheads, nheads_k, dp, float(softmax_scale), _dtype_code(q.dtype),
-                _bias_arg(bias_view), _stream_ptr(q.device),
+                _bias_arg(bias_view), _plan_arg(plan), _stream_ptr(q.device),
             )
         else:
             _bam_hip.call(
@@ -312,7 +366,7 @@ def _launch_bwd_preprocess(o, do, delta):
         )
 
 
-def _launch_bwd_dkdv(q, k, v, do, lse, delta, dk, dv, bf, flags, softmax_scale, accumulate=True, bias=None):
+def _launch_bwd_dkdv(q, k, v, do, lse, delta, dk, dv, bf, flags, softmax_scale, accumulate=True, bias=None, plan=None):
     """accumulate=True: dk/dv are fp32 and added to; False: dk/dv have q's dtype and are overwritten.
     ``bf``: the (B, S) bitfield tensor, or an ``_IndexView`` for index-tensor attention.  ``bias``: a
     ``_BiasView`` or None."""
@@ -334,11 +388,11 @@ def _launch_bwd_dkdv(q, k, v, do, lse, delta, dk, dv, bf, flags, softmax_scale, 
             dk.data_ptr(), dv.data_ptr(), bf.data_ptr(), flags.data_ptr(),
             *_strides3(q, k, v, do, dk, dv), bf.stride(0), flags.stride(0), flags.stride(1),
             B, S, Hq, k.shape[2], D, float(softmax_scale), _dtype_code(q.dtype), int(accumulate),
-            _bias_arg(bias), _stream_ptr(q.device),
+            _bias_arg(bias), _plan_arg(plan), _stream_ptr(q.device),
         )
 
 
-def _launch_bwd_dq(q, k, v, do, lse, delta, dq, bf, flags, softmax_scale, accumulate=True, bias=None):
+def _launch_bwd_dq(q, k, v, do, lse, delta, dq, bf, flags, softmax_scale, accumulate=True, bias=None, plan=None):
     B, S, Hq, D = q.shape
     with torch.cuda.device(q.device):
         if isinstance(bf, _IndexView):
@@ -357,7 +411,7 @@ def _launch_bwd_dq(q, k, v, do, lse, delta, dq, bf, flags, softmax_scale, accumu
             dq.data_ptr(), bf.data_ptr(), flags.data_ptr(),
             *_strides3(q, k, v, do, dq), bf.stride(0), flags.stride(0), flags.stride(1),
             B, S, Hq, k.shape[2], D, float(softmax_scale), _dtype_code(q.dtype), int(accumulate),
-            _bias_arg(bias), _stream_ptr(q.device),
+            _bias_arg(bias), _plan_arg(plan), _stream_ptr(q.device),
         )
 
 
@@ -383,12 +437,13 @@ def _bitfield_attn_backward_overwrite(do, q, k, v, o, bitfield_mask, compressed_
     lse = lse.contiguous()
     bf = bitfield_mask if bitfield_mask.stride(1) == 1 else bitfield_mask.contiguous()
     flags = compressed_mask if compressed_mask.stride(-1) == 1 else compressed_mask.contiguous()
+    plan = BitfieldUtils.plan_for(compressed_mask, bitfield_mask)
     delta = torch.empty_like(lse)
     batch, seqlen_q, nheads, _ = q.shape
     bias_view = _BiasView(bias, q, batch, nheads, seqlen_q, k.shape[1], may_copy=False) if bias is not None else None
     _launch_bwd_preprocess(o, do, delta)
-    _launch_bwd_dkdv(q, k, v, do, lse, delta, dk, dv, bf, flags, softmax_scale, accumulate=False, bias=bias_view)
-    _launch_bwd_dq(q, k, v, do, lse, delta, dq, bf, flags, softmax_scale, accumulate=False, bias=bias_view)
+    _launch_bwd_dkdv(q, k, v, do, lse, delta, dk, dv, bf, flags, softmax_scale, accumulate=False, bias=bias_view, plan=plan)
+    _launch_bwd_dq(q, k, v, do, lse, delta, dq, bf, flags, softmax_scale, accumulate=False, bias=bias_view, plan=plan)
     return dq, dk, dv
 
 
@@ -445,11 +500,12 @@ def _bitfield_attn_backward(
         bf = view
     flags = compressed_mask if compressed_mask.stride(-1) == 1 else compressed_mask.contiguous()
     assert flags.shape == (batch, -(-seqlen_q // BLOCK_M), -(-seqlen_k // BLOCK_N))
+    plan = BitfieldUtils.plan_for(compressed_mask, bitfield_mask) if view is None else None
     delta = torch.empty_like(lse)
     wq, wk, wv = work
     _launch_bwd_preprocess(ok, gk, delta)
-    _launch_bwd_dkdv(qk, kk, vk, gk, lse, delta, wk, wv, bf, flags, softmax_scale, bias=bias_view)
-    _launch_bwd_dq(qk, kk, vk, gk, lse, delta, wq, bf, flags, softmax_scale, bias=bias_view)
+    _launch_bwd_dkdv(qk, kk, vk, gk, lse, delta, wk, wv, bf, flags, softmax_scale, bias=bias_view, plan=plan)
+    _launch_bwd_dq(qk, kk, vk, gk, lse, delta, wq, bf, flags, softmax_scale, bias=bias_view, plan=plan)
     # the kernels accumulated into `work`; hand the sums back if those were copies
     for dst, mid, w in zip((dq, dk, dv), acc, work):
         if dp != d:

@@ -33,7 +33,7 @@ extern "C" {
 #define BAM_DTYPE_F16 0
 #define BAM_DTYPE_BF16 1
 
-/* Upper bound on S accepted by the attention kernels (tile lists live in LDS). */
+/* Upper bound on S accepted by the attention kernels (tile and slice lists live in LDS). */
 #define BAM_MAX_SEQLEN 131072
 
 /*
@@ -75,6 +75,32 @@ typedef struct bam_bias {
     int32_t is_f32;
 } bam_bias;
 
+/*
+ * Plan: what the attention kernels can use beyond the 128 x 32 flags to avoid work on masked pairs.  It has no
+ * counterpart in the reference (whose kernels decide per 128 x 32 flag tile, bitfield_attention.py:360-361,
+ * 395-408); the flags stay exactly the reference's, the plan is derived from the same bitfields at the same time:
+ *   fine : uint8 (B, 4 * ceil(S/128), fine_stride_s) -- class 0 / 1 / 2 of every 32-row x 32-key tile (row slice
+ *          s = rows [32 s, 32 s + 32)), same meaning as the flags, "2" again over in-range cells only;
+ *   order: int32 (B, 4 * ceil(S/128)) -- the row slices of each sequence sorted so that four neighbours need
+ *          about the same keys (slices holding text rows first, latest first; then modality-only slices grouped
+ *          by modality), -1 in the unused tail.
+ * bam_tile_plan fills the arrays (inside a caller-provided device workspace) and this host struct; the plain
+ * bitfield entry points (bam_fwd, bam_bwd, bam_bwd_dkdv, bam_bwd_dq) take a `const bam_plan*` that may be null.
+ * With a plan, the forward and dQ kernels build their workgroups from four slices of `order` and every wave skips
+ * the key tiles its own slice does not need; dK/dV walks the slices that have work for its keys, two at a time.
+ * Results do not depend on whether a plan is given (same pairs, same arithmetic per pair; only the order in which
+ * fp32 partial sums meet can differ in dK/dV).
+ */
+typedef struct bam_plan {
+    const uint8_t* fine;
+    int64_t fine_stride_b;
+    int64_t fine_stride_s;
+    const int32_t* order;
+    int64_t order_stride_b;
+    int32_t B;
+    int32_t S;
+} bam_plan;
+
 const char* bam_last_error(void);
 
 /* ABI version of this library (bumped on any signature change). */
@@ -89,6 +115,17 @@ int bam_abi_version(void);
  */
 int bam_tile_flags(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int64_t flags_stride_b,
                    int64_t flags_stride_m, int B, int S, void* stream);
+
+/*
+ * Tile flags plus plan in one call.  workspace: device memory of at least bam_plan_workspace_bytes(B, S) bytes,
+ * 256-byte aligned, owned by the caller and alive as long as the plan is used; the library lays `fine`, `order`
+ * and its own sort keys out inside it.  bam_plan_workspace_bytes returns 0 when no plan is built for that size
+ * (S above 131072); bam_tile_plan then refuses, and the caller uses bam_tile_flags and passes no plan.
+ */
+int64_t bam_plan_workspace_bytes(int B, int S);
+int bam_tile_plan(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int64_t flags_stride_b,
+                  int64_t flags_stride_m, void* workspace, int64_t workspace_bytes, int B, int S, bam_plan* plan,
+                  void* stream);
 
 /*
  * Dense bool mask, uint8 (B, S, S) contiguous: the allow rule for every pair
@@ -128,7 +165,8 @@ int bam_fwd(const void* q, const void* k, const void* v, void* o, float* lse, co
             int64_t k_stride_b, int64_t k_stride_s, int64_t k_stride_h, int64_t v_stride_b,
             int64_t v_stride_s, int64_t v_stride_h, int64_t o_stride_b, int64_t o_stride_s,
             int64_t o_stride_h, int64_t bf_stride_b, int64_t flags_stride_b, int64_t flags_stride_m, int B,
-            int S, int Hq, int Hkv, int D, float scale, int dtype, const bam_bias* bias, void* stream);
+            int S, int Hq, int Hkv, int D, float scale, int dtype, const bam_bias* bias, const bam_plan* plan,
+            void* stream);
 
 /*
  * Forward with index tensors (`offsets_q` / `offsets_k` of `_bitfield_attn_forward`,
@@ -171,7 +209,8 @@ int bam_bwd(const void* q, const void* k, const void* v, const void* dout, const
             int64_t dq_stride_b, int64_t dq_stride_s, int64_t dq_stride_h, int64_t dk_stride_b,
             int64_t dk_stride_s, int64_t dk_stride_h, int64_t dv_stride_b, int64_t dv_stride_s,
             int64_t dv_stride_h, int64_t bf_stride_b, int64_t flags_stride_b, int64_t flags_stride_m, int B,
-            int S, int Hq, int Hkv, int D, float scale, int dtype, int accumulate, const bam_bias* bias, void* stream);
+            int S, int Hq, int Hkv, int D, float scale, int dtype, int accumulate, const bam_bias* bias,
+            const bam_plan* plan, void* stream);
 
 /*
  * The two halves of bam_bwd as separate launches (same reference kernel,
@@ -188,7 +227,7 @@ int bam_bwd_dkdv(const void* q, const void* k, const void* v, const void* dout, 
                  int64_t dk_stride_b, int64_t dk_stride_s, int64_t dk_stride_h, int64_t dv_stride_b,
                  int64_t dv_stride_s, int64_t dv_stride_h, int64_t bf_stride_b, int64_t flags_stride_b,
                  int64_t flags_stride_m, int B, int S, int Hq, int Hkv, int D, float scale, int dtype,
-                 int accumulate, const bam_bias* bias, void* stream);
+                 int accumulate, const bam_bias* bias, const bam_plan* plan, void* stream);
 
 int bam_bwd_dq(const void* q, const void* k, const void* v, const void* dout, const float* lse,
                const float* delta, void* dq, const int64_t* bf, const int8_t* flags, int64_t q_stride_b,
@@ -197,7 +236,7 @@ int bam_bwd_dq(const void* q, const void* k, const void* v, const void* dout, co
                int64_t do_stride_b, int64_t do_stride_s, int64_t do_stride_h, int64_t dq_stride_b,
                int64_t dq_stride_s, int64_t dq_stride_h, int64_t bf_stride_b, int64_t flags_stride_b,
                int64_t flags_stride_m, int B, int S, int Hq, int Hkv, int D, float scale, int dtype,
-               int accumulate, const bam_bias* bias, void* stream);
+               int accumulate, const bam_bias* bias, const bam_plan* plan, void* stream);
 
 /*
  * bam_bwd_dkdv / bam_bwd_dq with index tensors (`offsets_q` / `offsets_k` of

@@ -123,6 +123,13 @@ def test_full_size_mask_materialized_from_bitfields_gives_the_bitfield_result_bi
         qg, kg, vg = (t.clone().requires_grad_(True) for t in (q, k, v))
         o = fn(qg, kg, vg)
         outs.append((o.detach(), *torch.autograd.grad(o, (qg, kg, vg), do)))
-    for a, b in zip(*outs):
-        assert torch.equal(a, b)
+    # o and dq: every query row sees the same key tiles in the same order on both paths -> identical bits.
+    # dk, dv: the bitfield path pairs up the row slices that have work (its plan), the mask path walks whole
+    # 128-row blocks, so the fp32 partial sums of the two row streams meet in another order.
+    names = ("o", "dq", "dk", "dv")
+    for name, a, b in zip(names, *outs):
+        if name in ("o", "dq"):
+            assert torch.equal(a, b), name
+        else:
+            assert rel_l2(a.float(), b.float()) <= 2e-3, name
     BA.BitfieldUtils.clear_cache()

@@ -473,7 +473,7 @@ def test_combined_backward_entry_point(accumulate):
             got[0].data_ptr(), got[1].data_ptr(), got[2].data_ptr(), bf.data_ptr(), flags.data_ptr(),
             *BA._strides3(q, k, v, do, *got), bf.stride(0), flags.stride(0), flags.stride(1),
             B, S, Hq, Hkv, D, float(sc), BA._dtype_code(q.dtype), accumulate,
-            bview.byref() if bview is not None else None, BA._stream_ptr(d),
+            bview.byref() if bview is not None else None, None, BA._stream_ptr(d),
         )
         torch.cuda.synchronize()
         for a, b in zip(got, want):

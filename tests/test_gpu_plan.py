@@ -1,0 +1,160 @@
+"""The plan (classes of 32 x 32 tiles + slice order) the kernels use to skip masked work: its contents
+against a brute-force classification of the oracle's mask, and the attention results with and without it."""
+
+import ctypes
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from cornstarch_amd import workloads as W
+from cornstarch_amd.kernel import _bam_hip
+from cornstarch_amd.kernel import bitfield_attention as BA
+from oracle import bam_oracle as O
+from tests.helpers import random_bitfield, rel_l2
+
+pytestmark = pytest.mark.gpu
+
+
+def dev():
+    return torch.device("cuda:0")
+
+
+def build_plan(bf):
+    """flags, fine (B, slots, num_n) and order (B, slots) of a bitfield tensor on the device."""
+    BA.BitfieldUtils.clear_cache()
+    flags = BA.BitfieldUtils.materialize_compressed_mask_from_bitfield_mask(bf)
+    plan = BA.BitfieldUtils.plan_for(flags, bf)
+    assert plan is not None
+    st = plan.struct
+    B, S = bf.shape
+    slots, num_n = 4 * -(-S // 128), -(-S // 32)
+    ws = plan.workspace
+    base = ws.data_ptr()
+    fine = torch.as_strided(ws, (B, slots, num_n), (st.fine_stride_b, st.fine_stride_s, 1), st.fine - base)
+    order = torch.as_strided(ws.view(torch.int32), (B, slots), (st.order_stride_b, 1), (st.order - base) // 4)
+    torch.cuda.synchronize()
+    return flags, fine.clone(), order.clone(), plan
+
+
+def brute_force_fine(mask, S):
+    """Class of every 32 x 32 tile from the (B, S, S) bool mask: 0 nothing allowed, 2 every in-range cell."""
+    B = mask.shape[0]
+    n = -(-S // 32)
+    pad = n * 32 - S
+    m = F.pad(mask, (0, pad, 0, pad))
+    cnt = m.view(B, n, 32, n, 32).sum(dim=(2, 4))
+    cells = F.pad(torch.ones_like(mask), (0, pad, 0, pad)).view(B, n, 32, n, 32).sum(dim=(2, 4))
+    return torch.where(cnt == 0, 0, torch.where(cnt == cells, 2, 1)).to(torch.uint8)
+
+
+@pytest.mark.parametrize("S", [1, 31, 57, 128, 144, 283, 1000])
+@pytest.mark.parametrize("wide", [False, True])
+def test_fine_classes_and_order_on_irregular_bitfields(S, wide):
+    bf = random_bitfield(3, S, seed=S, pad=min(5, S - 1), wide=wide)
+    flags, fine, order, _ = build_plan(bf.to(dev()))
+    assert torch.equal(flags.cpu(), O.tile_flags(bf))  # the public flags are what they were
+    n = -(-S // 32)
+    want = brute_force_fine(O.materialize_mask(bf), S)
+    assert torch.equal(fine[:, :n].cpu(), want)
+    assert (fine[:, n:] == 0).all()  # slots past the last row slice need nothing
+    for b in range(3):
+        o = order[b].cpu().tolist()
+        assert sorted(o[:n]) == list(range(n)) and all(x == -1 for x in o[n:])
+        # slices holding a text row come first, latest first; modality-only slices are grouped by modality
+        rows = F.pad(bf[b], (0, n * 32 - S)).view(n, 32)
+        text = ((rows & 1) != 0).any(dim=1)
+        sig = torch.zeros(n, dtype=torch.int64)
+        for r in range(32):
+            sig |= rows[:, r] & ((1 << 62) - 1)
+        nt = int(text.sum())
+        assert all(text[s] for s in o[:nt]) and o[:nt] == sorted(o[:nt], reverse=True)
+        rest = o[nt:n]
+        groups = [int(sig[s]) for s in rest]
+        assert groups == sorted(groups)
+        for gval in set(groups):
+            members = [s for s in rest if int(sig[s]) == gval]
+            assert members == sorted(members)
+
+
+@pytest.mark.parametrize("name", ["C1", "C2", "C4"])
+def test_fine_classes_on_the_benchmark_workloads(name):
+    bf = W.make_bitfields(name).to(dev())
+    flags, fine, order, _ = build_plan(bf)
+    S = bf.shape[1]
+    n = S // 32
+    want = torch.cat([brute_force_fine(O.materialize_mask(bf[b : b + 1]), S) for b in range(bf.shape[0])])
+    assert torch.equal(fine[:, :n], want)
+    # a 128 x 32 flag is the summary of its four row slices
+    f4 = fine[:, :n].view(bf.shape[0], n // 4, 4, n)
+    derived = torch.where((f4 == 0).all(dim=2), 0, torch.where((f4 == 2).all(dim=2), 2, 1)).to(torch.int8)
+    assert torch.equal(derived, flags)
+
+
+def _run(q, k, v, do, bf, flags, plan, scale):
+    """forward + both backward kernels through the launch helpers, with or without a plan"""
+    B, S, Hq, D = q.shape
+    with torch.cuda.device(q.device):
+        o = torch.empty_like(q)
+        lse = torch.empty((B, Hq, flags.shape[1] * 128), dtype=torch.float32, device=q.device)
+        _bam_hip.call(
+            "bam_fwd", q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse.data_ptr(), bf.data_ptr(),
+            flags.data_ptr(), *BA._strides3(q, k, v, o), bf.stride(0), flags.stride(0), flags.stride(1),
+            B, S, Hq, k.shape[2], D, float(scale), BA._dtype_code(q.dtype), None,
+            plan.byref() if plan is not None else None, BA._stream_ptr(q.device),
+        )
+    delta = torch.empty_like(lse)
+    BA._launch_bwd_preprocess(o, do, delta)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    BA._launch_bwd_dkdv(q, k, v, do, lse, delta, dk, dv, bf, flags, scale, accumulate=False, plan=plan)
+    BA._launch_bwd_dq(q, k, v, do, lse, delta, dq, bf, flags, scale, accumulate=False, plan=plan)
+    torch.cuda.synchronize()
+    return o, lse[:, :, :S], dq, dk, dv
+
+
+@pytest.mark.parametrize("B,S,Hq,Hkv,D", [(2, 517, 4, 2, 128), (1, 1000, 4, 4, 64), (3, 200, 2, 1, 32), (1, 2048, 8, 2, 128)])
+def test_results_do_not_depend_on_the_plan(B, S, Hq, Hkv, D):
+    d = dev()
+    bf = random_bitfield(B, S, seed=S + D, pad=7).to(d)
+    g = torch.Generator().manual_seed(S)
+    q = (torch.randn(B, S, Hq, D, generator=g) * 0.5).bfloat16().to(d)
+    k = (torch.randn(B, S, Hkv, D, generator=g) * 0.5).bfloat16().to(d)
+    v = (torch.randn(B, S, Hkv, D, generator=g) * 0.5).bfloat16().to(d)
+    do = torch.randn(B, S, Hq, D, generator=g).bfloat16().to(d)
+    flags, _, _, plan = build_plan(bf)
+    scale = 1.0 / math.sqrt(D)
+    with_plan = _run(q, k, v, do, bf, flags, plan, scale)
+    without = _run(q, k, v, do, bf, flags, None, scale)
+    for name, a, b in zip(("o", "lse", "dq", "dk", "dv"), with_plan, without):
+        if name in ("dk", "dv"):  # the two row streams add their fp32 partial sums in another order
+            assert rel_l2(a.float(), b.float()) <= 2e-3, name
+        else:
+            assert torch.equal(a, b), name
+    o_ref, lse_ref = O.attention_forward(q, k, v, bf)
+    assert (with_plan[0].float() - o_ref).abs().max().item() <= 2e-2
+    for got, want in zip(with_plan[2:], O.attention_backward(q, k, v, bf, do)):
+        assert rel_l2(got.float(), want) <= 5e-2
+    BA.BitfieldUtils.clear_cache()
+
+
+def test_a_plan_of_another_problem_is_refused():
+    d = dev()
+    bf = random_bitfield(1, 256, seed=1).to(d)
+    flags, _, _, plan = build_plan(bf)
+    q = torch.zeros(1, 128, 2, 64, dtype=torch.bfloat16, device=d)
+    bf2 = bf[:, :128].contiguous()
+    fl2 = torch.zeros(1, 1, 4, dtype=torch.int8, device=d)
+    o = torch.empty_like(q)
+    lse = torch.empty(1, 2, 128, device=d)
+    with pytest.raises(_bam_hip.BamError, match="plan was built for"):
+        _bam_hip.call(
+            "bam_fwd", q.data_ptr(), q.data_ptr(), q.data_ptr(), o.data_ptr(), lse.data_ptr(), bf2.data_ptr(),
+            fl2.data_ptr(), *BA._strides3(q, q, q, o), bf2.stride(0), fl2.stride(0), fl2.stride(1),
+            1, 128, 2, 2, 64, 0.125, BA._dtype_code(q.dtype), None, plan.byref(), BA._stream_ptr(d),
+        )
+    # caller-provided flags (not the cached tensor) never pick up the cached plan
+    assert BA.BitfieldUtils.plan_for(flags.clone(), bf) is None
+    assert BA.BitfieldUtils.plan_for(flags, bf) is plan
+    BA.BitfieldUtils.clear_cache()
+    assert BA.BitfieldUtils.plan_for(flags, bf) is None

@@ -39,7 +39,11 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(lib, n), f"{n} is declared in include/bam_hip.h but not exported"
     assert _bam_hip.load().bam_abi_version() == _bam_hip.ABI_VERSION
     # the binding's prototypes cover every compute entry point of the header
-    assert set(_bam_hip.SIGNATURES) == set(names) - {"bam_last_error", "bam_abi_version"}
+    assert set(_bam_hip.SIGNATURES) == set(names) - {"bam_last_error", "bam_abi_version", "bam_plan_workspace_bytes"}
+    # plan workspace: sized without a GPU; no plan beyond 4096 row slices
+    lib2 = _bam_hip.load()
+    assert lib2.bam_plan_workspace_bytes(1, 8192) >= 256 * 256 + 256 * 4 and lib2.bam_plan_workspace_bytes(1, 8192) % 256 == 0
+    assert lib2.bam_plan_workspace_bytes(2, 131072) > 0 and lib2.bam_plan_workspace_bytes(1, 131073) == 0
 
 
 def test_abi_rejects_bad_arguments_without_touching_the_gpu():
@@ -47,21 +51,21 @@ def test_abi_rejects_bad_arguments_without_touching_the_gpu():
     # null pointers / unsupported head dim are refused before any HIP call
     rc = lib.bam_tile_flags(None, 0, None, 0, 0, 1, 128, None)
     assert rc == -1 and b"null" in lib.bam_last_error()
-    args = [ctypes.c_void_p(16)] * 7 + [8] * 15 + [1, 128, 4, 4, 48] + [0.125, 1, None, None]
+    args = [ctypes.c_void_p(16)] * 7 + [8] * 15 + [1, 128, 4, 4, 48] + [0.125, 1, None, None, None]
     rc = lib.bam_fwd(*args)
     assert rc == -2 and b"head dimension 48" in lib.bam_last_error()
-    args = [ctypes.c_void_p(16)] * 7 + [8] * 15 + [1, 128, 6, 4, 64] + [0.125, 1, None, None]
+    args = [ctypes.c_void_p(16)] * 7 + [8] * 15 + [1, 128, 6, 4, 64] + [0.125, 1, None, None, None]
     assert lib.bam_fwd(*args) == -1 and b"multiple of Hkv" in lib.bam_last_error()
-    args = [ctypes.c_void_p(8)] + [ctypes.c_void_p(16)] * 6 + [8] * 15 + [1, 128, 4, 4, 64] + [0.125, 1, None, None]
+    args = [ctypes.c_void_p(8)] + [ctypes.c_void_p(16)] * 6 + [8] * 15 + [1, 128, 4, 4, 64] + [0.125, 1, None, None, None]
     assert lib.bam_fwd(*args) == -1 and b"16-byte aligned" in lib.bam_last_error()
-    args = [ctypes.c_void_p(16)] * 7 + [8] * 15 + [1, 128, 4, 4, 64] + [-1.0, 1, None, None]
+    args = [ctypes.c_void_p(16)] * 7 + [8] * 15 + [1, 128, 4, 4, 64] + [-1.0, 1, None, None, None]
     assert lib.bam_fwd(*args) == -1 and b"scale" in lib.bam_last_error()
     # a bias descriptor without a pointer, or with a pointer that is not a multiple of its element size
     bias = _bam_hip.Bias(None, 0, 0, 0, 1)
-    args = [ctypes.c_void_p(16)] * 7 + [8] * 15 + [1, 128, 4, 4, 64] + [0.125, 1, ctypes.byref(bias), None]
+    args = [ctypes.c_void_p(16)] * 7 + [8] * 15 + [1, 128, 4, 4, 64] + [0.125, 1, ctypes.byref(bias), None, None]
     assert lib.bam_fwd(*args) == -1 and b"bias" in lib.bam_last_error()
     bias = _bam_hip.Bias(18, 0, 0, 0, 1)
-    args = [ctypes.c_void_p(16)] * 7 + [8] * 15 + [1, 128, 4, 4, 64] + [0.125, 1, ctypes.byref(bias), None]
+    args = [ctypes.c_void_p(16)] * 7 + [8] * 15 + [1, 128, 4, 4, 64] + [0.125, 1, ctypes.byref(bias), None, None]
     assert lib.bam_fwd(*args) == -1 and b"bias" in lib.bam_last_error()
     with pytest.raises(_bam_hip.BamError):
         _bam_hip.call("bam_materialize_mask", None, 0, None, 1, 8, None)
