@@ -99,23 +99,24 @@ def measured_traffic(workload, kernel):
     return None
 
 
-def issued_flops(flags, w):
-    """MFMA FLOPs the three attention kernels issue, from the tile lists they build out of the flags:
-    the forward and dQ kernels compute every 128-row x 64-key tile with a non-zero flag (4 resp. 6 D-deep
-    products per pair), dK/dV every 128-row x 32-key flag tile (8).  Partial tiles count in full."""
-    import torch
+def issued_flops(flags, plan, w):
+    """MFMA FLOPs the three attention kernels issue, from the tile lists they build: a wave of the forward
+    and dQ kernels computes a 32-row slice against every 64-key tile in which the slice has a non-empty class
+    (4 resp. 6 D-deep products per pair), a wave of dK/dV a 32-row slice against a 32-key group (8).  Partial
+    tiles count in full.  Without a plan a slice inherits the classes of its 128-row block."""
     import torch.nn.functional as F
 
-    nz = flags > 0
+    cls = plan.fine_classes() if plan is not None else flags.repeat_interleave(4, dim=1)
+    nz = cls > 0
     if nz.shape[-1] % 2:
         nz = F.pad(nz, (0, 1))
     tiles64 = int((nz[..., 0::2] | nz[..., 1::2]).sum())
     tiles32 = int(nz.sum())
     per_pair = w.D * w.Hq
     return {
-        "fwd": 4 * per_pair * tiles64 * 128 * 64,
-        "dkdv": 8 * per_pair * tiles32 * 128 * 32,
-        "dq": 6 * per_pair * tiles64 * 128 * 64,
+        "fwd": 4 * per_pair * tiles64 * 32 * 64,
+        "dkdv": 8 * per_pair * tiles32 * 32 * 32,
+        "dq": 6 * per_pair * tiles64 * 32 * 64,
     }
 
 
@@ -147,6 +148,7 @@ def run_workload(name, steps, warmup, dev):
         mark(0)
         BA.BitfieldUtils.clear_cache()
         flags = BA.BitfieldUtils.materialize_compressed_mask_from_bitfield_mask(bf)
+        plan = BA.BitfieldUtils.plan_for(flags, bf)  # built by the same launch as the flags
         mark(1)
         o, lse, _ = BA._bitfield_attn_forward(q, k, v, bf, flags, softmax_scale=scale)
         mark(2)
@@ -155,9 +157,9 @@ def run_workload(name, steps, warmup, dev):
         mark(3)
         BA._launch_bwd_preprocess(o, do, delta)
         mark(4)
-        BA._launch_bwd_dkdv(q, k, v, do, lse, delta, dk, dv, bf, flags, scale, accumulate=False)
+        BA._launch_bwd_dkdv(q, k, v, do, lse, delta, dk, dv, bf, flags, scale, accumulate=False, plan=plan)
         mark(5)
-        BA._launch_bwd_dq(q, k, v, do, lse, delta, dq, bf, flags, scale, accumulate=False)
+        BA._launch_bwd_dq(q, k, v, do, lse, delta, dq, bf, flags, scale, accumulate=False, plan=plan)
         mark(6)
         return o, (dq, dk, dv)
 
@@ -204,7 +206,7 @@ def run_workload(name, steps, warmup, dev):
 
     BA.BitfieldUtils.clear_cache()
     flags = BA.BitfieldUtils.materialize_compressed_mask_from_bitfield_mask(bf)
-    issued = issued_flops(flags, w)
+    issued = issued_flops(flags, BA.BitfieldUtils.plan_for(flags, bf), w)
     BA.BitfieldUtils.clear_cache()
     return {
         "w": w, "pairs": pairs, "f_fwd": f_fwd, "f_bwd": f_bwd,

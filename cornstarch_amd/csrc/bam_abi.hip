@@ -265,9 +265,9 @@ int bam_tile_flags(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int64_
 }
 
 namespace {
-// workspace layout: fine | order | sort keys, each part 256-byte aligned
+// workspace layout: fine | order, each part 256-byte aligned
 struct PlanLayout {
-    int64_t fine_ss, fine_sb, order_sb, fine_off, order_off, keys_off, bytes;
+    int64_t fine_ss, fine_sb, order_sb, fine_off, order_off, bytes;
 };
 PlanLayout plan_layout(int B, int S) {
     const int64_t num_m = (S + 127) / 128, num_n = (S + 31) / 32, slots = 4 * num_m;
@@ -278,8 +278,7 @@ PlanLayout plan_layout(int B, int S) {
     l.order_sb = slots;
     l.fine_off = 0;
     l.order_off = up(B * l.fine_sb, 256);
-    l.keys_off = l.order_off + up(B * slots * 4, 256);
-    l.bytes = l.keys_off + up(B * slots * 16, 256);
+    l.bytes = l.order_off + up(B * slots * 4, 256);
     return l;
 }
 }  // namespace
@@ -314,8 +313,8 @@ int bam_tile_plan(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int64_t
     plan->B = B;
     plan->S = S;
     return launched(bam::launch_tile_plan(bf, bf_stride_b, flags, flags_stride_b, flags_stride_m, (uint8_t*)(w + l.fine_off),
-                                          l.fine_sb, l.fine_ss, (int*)(w + l.order_off), l.order_sb,
-                                          (unsigned long long*)(w + l.keys_off), B, S, (hipStream_t)stream),
+                                          l.fine_sb, l.fine_ss, (int*)(w + l.order_off), l.order_sb, B, S,
+                                          (hipStream_t)stream),
                     "bam_tile_plan");
 }
 

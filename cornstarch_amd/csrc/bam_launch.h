@@ -63,11 +63,10 @@ struct AttnParams {
 
 int launch_tile_flags(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int64_t flags_stride_b,
                       int64_t flags_stride_m, int B, int S, hipStream_t stream);
-// Flags plus plan: fine (B, 4 * num_m, fine_ss) bytes, order (B, 4 * num_m) ints, keys: scratch of
-// 2 * B * 4 * num_m 64-bit words.
+// Flags plus plan in one launch: fine (B, 4 * num_m, fine_ss) bytes, order (B, 4 * num_m) ints.
 int launch_tile_plan(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int64_t flags_stride_b,
                      int64_t flags_stride_m, uint8_t* fine, int64_t fine_sb, int64_t fine_ss, int* order,
-                     int64_t order_sb, unsigned long long* keys, int B, int S, hipStream_t stream);
+                     int64_t order_sb, int B, int S, hipStream_t stream);
 int launch_materialize_mask(const int64_t* bf, int64_t bf_stride_b, uint8_t* out, int B, int S,
                             hipStream_t stream);
 int launch_flag_row_workloads(const int8_t* flags, int64_t flags_stride_b, int64_t flags_stride_m, int B, int num_m,

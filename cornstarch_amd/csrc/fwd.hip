@@ -45,6 +45,7 @@ __global__ __launch_bounds__(FWD_THREADS, D == 128 ? 2 : 3) void fwd_kernel(cons
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int hi = lane >> 5, l32 = lane & 31, half16 = (lane >> 4) & 1;
+    const int wave_lane = tid >> 6;
     constexpr bool IDX = MODE == MASK_INDEXED, DENSE = MODE == MASK_DENSE;
     const int Sq = p.Sq, Sk = p.Sk;
     const int G = p.Hq / p.Hkv;
@@ -133,7 +134,9 @@ __global__ __launch_bounds__(FWD_THREADS, D == 128 ? 2 : 3) void fwd_kernel(cons
     // buffer are issued one per MFMA of the S phase, where the wave has nothing else to wait for.
     auto tile_step = [&](auto prefetch, int cur, int entry, int kt_next) {
         constexpr bool PREFETCH = decltype(prefetch)::value;
-        const int kt = entry >> 8, cls = (entry >> (2 * wave)) & 3;
+        // (the class is extracted with a per-lane copy of the wave number on purpose: with a skip branch the
+        // compiler can prove wave-uniform it lays the loop out around that branch and the kernel loses ~8 %)
+        const int kt = entry >> 8, cls = (entry >> (2 * wave_lane)) & 3;
         if (cls == 0) {  // nothing for this wave's slice in the tile: only keep the copies of the next one going
             if (PREFETCH) {
 #pragma unroll

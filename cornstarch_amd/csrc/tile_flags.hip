@@ -16,6 +16,58 @@ constexpr int FLAG_WAVES = 4;
 constexpr int FLAG_TILES_PER_WAVE = 2;  // few tiles per wave: the grid, not the wave, covers the row of tiles
 constexpr int FLAG_COLS_PER_BLOCK = FLAG_WAVES * FLAG_TILES_PER_WAVE;
 
+// ---------------------------------------------------------------------------------------------------------
+// Slice order.  The forward and dQ kernels give each of the four waves of a workgroup one 32-row slice and walk
+// the union of the key tiles those slices need, so four slices that need the same keys should sit together:
+//   * slices holding a text row first, by descending position (they see their whole past; the latest see most),
+//   * then the slices made of modality rows only, grouped by the OR of their bitfields (equal value = same
+//     modality = same keys), by ascending position inside a group.
+// Every slice gets a two-word sort key and is ranked against all others of its sequence (at most
+// MAX_PLAN_SLICES of them); slots past the last slice are set to -1.  The work rides in the launch of the flag
+// kernel, as extra workgroups of its grid (it needs the bitfields only): workgroup `part` of sequence b ranks
+// slices [256 part, +256).
+__device__ __forceinline__ void slice_sort_key(const int64_t* __restrict__ row, int S, int ns, int s,
+                                               unsigned long long& k1, unsigned long long& k2) {
+    k1 = ~0ull;
+    k2 = ~0ull;
+    if (s >= ns) return;
+    const int64_t M = (((int64_t)1) << 62) - 1;
+    int64_t sig = 0;
+    bool text = false;
+    for (int r = 0; r < 32; ++r) {
+        const int i = s * 32 + r;
+        const int64_t f = i < S ? row[i] : 0;
+        sig |= f & M;
+        text |= (f & 1) != 0;
+    }
+    k1 = text ? 0ull : (1ull << 62) | (unsigned long long)sig;
+    k2 = text ? (unsigned long long)(ns - 1 - s) : (unsigned long long)s;
+}
+
+__device__ __forceinline__ void slice_order_part(const int64_t* __restrict__ row, int S, int part,
+                                                 int* __restrict__ order_row) {
+    __shared__ unsigned long long sk[2 * 256];
+    const int ns = (S + 31) / 32, slots = 4 * ((S + BLOCK_M - 1) / BLOCK_M);
+    const int tid = threadIdx.x, s = part * 256 + tid;
+    unsigned long long my1, my2;
+    slice_sort_key(row, S, ns, s, my1, my2);
+    int rank = 0;
+    for (int base = 0; base < ns; base += 256) {
+        __syncthreads();
+        slice_sort_key(row, S, ns, base + tid, sk[2 * tid], sk[2 * tid + 1]);
+        __syncthreads();
+        const int cnt = min(256, ns - base);
+        for (int j = 0; j < cnt; ++j) {
+            const unsigned long long o1 = sk[2 * j], o2 = sk[2 * j + 1];
+            rank += (o1 < my1 || (o1 == my1 && o2 < my2)) ? 1 : 0;  // (k1, k2) pairs are distinct
+        }
+    }
+    if (s < ns)
+        order_row[rank] = s;
+    else if (s < slots)
+        order_row[s] = -1;
+}
+
 // FINE: also write the class of every 32-row x 32-column tile (the four row slices of each flag tile) to
 // fine[b][4 m + w][n]; same 0 / 1 / 2 meaning, "full" again over the in-range cells only.
 template <bool FINE>
@@ -25,7 +77,14 @@ __global__ __launch_bounds__(FLAG_WAVES * 64) void tile_flags_kernel(const int64
                                                                     int64_t flags_stride_b,
                                                                     int64_t flags_stride_m, int S, int num_n,
                                                                     uint8_t* __restrict__ fine, int64_t fine_sb,
-                                                                    int64_t fine_ss) {
+                                                                    int64_t fine_ss, int* __restrict__ order,
+                                                                    int64_t order_sb, int flag_blocks_x) {
+    if (FINE && (int)blockIdx.x >= flag_blocks_x) {  // the workgroups that sort the slices (see slice_order_part)
+        const int part = blockIdx.y;
+        if (part * 256 < 4 * (int)gridDim.y)
+            slice_order_part(bf + (int64_t)blockIdx.z * bf_stride_b, S, part, order + (int64_t)blockIdx.z * order_sb);
+        return;
+    }
     __shared__ int64_t q_bits[BLOCK_M];
     const int b = blockIdx.z, m = blockIdx.y;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -216,78 +275,21 @@ int launch_tile_flags(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int
     const int num_m = (S + BLOCK_M - 1) / BLOCK_M, num_n = (S + BLOCK_N - 1) / BLOCK_N;
     dim3 grid((num_n + FLAG_COLS_PER_BLOCK - 1) / FLAG_COLS_PER_BLOCK, num_m, B);
     hipLaunchKernelGGL(tile_flags_kernel<false>, grid, dim3(FLAG_WAVES * 64), 0, stream, bf, bf_stride_b, flags,
-                       flags_stride_b, flags_stride_m, S, num_n, (uint8_t*)nullptr, (int64_t)0, (int64_t)0);
+                       flags_stride_b, flags_stride_m, S, num_n, (uint8_t*)nullptr, (int64_t)0, (int64_t)0, (int*)nullptr,
+                       (int64_t)0, 0);
     return (int)hipGetLastError();
-}
-
-// ---------------------------------------------------------------------------------------------------------
-// Slice order.  The forward and dQ kernels give each of the four waves of a workgroup one 32-row slice and walk
-// the union of the key tiles those slices need, so four slices that need the same keys should sit together:
-//   * slices holding a text row first, by descending position (they see their whole past; the latest see most),
-//   * then the slices made of modality rows only, grouped by the OR of their bitfields (equal value = same
-//     modality = same keys), by ascending position inside a group.
-// Step 1 writes a two-word sort key per slice, step 2 ranks every slice against all others of its sequence
-// (at most MAX_PLAN_SLICES of them) and scatters; slots past the last slice are set to -1.
-__global__ __launch_bounds__(256) void slice_keys_kernel(const int64_t* __restrict__ bf, int64_t bf_stride_b, int S,
-                                                         int ns, int slots, unsigned long long* __restrict__ keys) {
-    const int s = blockIdx.x * 256 + threadIdx.x, b = blockIdx.y;
-    if (s >= slots) return;
-    unsigned long long k1 = ~0ull, k2 = ~0ull;  // slots without rows sort last
-    if (s < ns) {
-        const int64_t M = (((int64_t)1) << 62) - 1;
-        const int64_t* row = bf + (int64_t)b * bf_stride_b;
-        int64_t sig = 0;
-        bool text = false;
-        for (int r = 0; r < 32; ++r) {
-            const int i = s * 32 + r;
-            const int64_t f = i < S ? row[i] : 0;
-            sig |= f & M;
-            text |= (f & 1) != 0;
-        }
-        k1 = text ? 0ull : (1ull << 62) | (unsigned long long)sig;
-        k2 = text ? (unsigned long long)(ns - 1 - s) : (unsigned long long)s;
-    }
-    keys[2 * ((int64_t)b * slots + s)] = k1;
-    keys[2 * ((int64_t)b * slots + s) + 1] = k2;
-}
-
-__global__ __launch_bounds__(256) void slice_rank_kernel(const unsigned long long* __restrict__ keys, int ns, int slots,
-                                                         int* __restrict__ order, int64_t order_sb) {
-    __shared__ unsigned long long sk[2 * 256];
-    const int s = blockIdx.x * 256 + threadIdx.x, b = blockIdx.y;
-    const unsigned long long* kb = keys + 2 * (int64_t)b * slots;
-    const unsigned long long my1 = s < slots ? kb[2 * s] : 0, my2 = s < slots ? kb[2 * s + 1] : 0;
-    int rank = 0;
-    for (int base = 0; base < ns; base += 256) {
-        __syncthreads();
-        if (base + threadIdx.x < ns) {
-            sk[2 * threadIdx.x] = kb[2 * (base + threadIdx.x)];
-            sk[2 * threadIdx.x + 1] = kb[2 * (base + threadIdx.x) + 1];
-        }
-        __syncthreads();
-        const int cnt = min(256, ns - base);
-        for (int j = 0; j < cnt; ++j) {
-            const unsigned long long o1 = sk[2 * j], o2 = sk[2 * j + 1];
-            rank += (o1 < my1 || (o1 == my1 && o2 < my2)) ? 1 : 0;  // (k1, k2) pairs are distinct
-        }
-    }
-    if (s < ns)
-        order[(int64_t)b * order_sb + rank] = s;
-    else if (s < slots)
-        order[(int64_t)b * order_sb + s] = -1;
 }
 
 int launch_tile_plan(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int64_t flags_stride_b,
                      int64_t flags_stride_m, uint8_t* fine, int64_t fine_sb, int64_t fine_ss, int* order,
-                     int64_t order_sb, unsigned long long* keys, int B, int S, hipStream_t stream) {
+                     int64_t order_sb, int B, int S, hipStream_t stream) {
     const int num_m = (S + BLOCK_M - 1) / BLOCK_M, num_n = (S + BLOCK_N - 1) / BLOCK_N;
-    const int ns = (S + 31) / 32, slots = 4 * num_m;
-    dim3 grid((num_n + FLAG_COLS_PER_BLOCK - 1) / FLAG_COLS_PER_BLOCK, num_m, B);
+    const int flag_blocks_x = (num_n + FLAG_COLS_PER_BLOCK - 1) / FLAG_COLS_PER_BLOCK;
+    // one more column of workgroups: (flag_blocks_x, part, b) ranks 256 slices; 4 num_m slots need
+    // ceil(4 num_m / 256) <= num_m parts
+    dim3 grid(flag_blocks_x + 1, num_m, B);
     hipLaunchKernelGGL(tile_flags_kernel<true>, grid, dim3(FLAG_WAVES * 64), 0, stream, bf, bf_stride_b, flags,
-                       flags_stride_b, flags_stride_m, S, num_n, fine, fine_sb, fine_ss);
-    dim3 sgrid((slots + 255) / 256, B);
-    hipLaunchKernelGGL(slice_keys_kernel, sgrid, dim3(256), 0, stream, bf, bf_stride_b, S, ns, slots, keys);
-    hipLaunchKernelGGL(slice_rank_kernel, sgrid, dim3(256), 0, stream, keys, ns, slots, order, order_sb);
+                       flags_stride_b, flags_stride_m, S, num_n, fine, fine_sb, fine_ss, order, order_sb, flag_blocks_x);
     return (int)hipGetLastError();
 }
 

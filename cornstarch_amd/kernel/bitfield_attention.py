@@ -85,6 +85,18 @@ class _TilePlan:
 
         return ctypes.byref(self.struct)
 
+    def fine_classes(self) -> torch.Tensor:
+        """uint8 (B, 4 * ceil(S/128), ceil(S/32)) view: class 0 / 1 / 2 of every 32-row x 32-key tile."""
+        st, ws = self.struct, self.workspace
+        slots, num_n = 4 * self.flags.shape[1], self.flags.shape[2]
+        return torch.as_strided(ws, (st.B, slots, num_n), (st.fine_stride_b, st.fine_stride_s, 1), st.fine - ws.data_ptr())
+
+    def slice_order(self) -> torch.Tensor:
+        """int32 (B, 4 * ceil(S/128)) view: the 32-row slices in the order the forward / dQ kernels take them."""
+        st, ws = self.struct, self.workspace
+        return torch.as_strided(ws.view(torch.int32), (st.B, 4 * self.flags.shape[1]), (st.order_stride_b, 1),
+                                (st.order - ws.data_ptr()) // 4)
+
 
 def _plan_arg(plan: Optional["_TilePlan"]):
     return plan.byref() if plan is not None else None

@@ -118,8 +118,8 @@ int bam_tile_flags(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int64_
 
 /*
  * Tile flags plus plan in one call.  workspace: device memory of at least bam_plan_workspace_bytes(B, S) bytes,
- * 256-byte aligned, owned by the caller and alive as long as the plan is used; the library lays `fine`, `order`
- * and its own sort keys out inside it.  bam_plan_workspace_bytes returns 0 when no plan is built for that size
+ * 256-byte aligned, owned by the caller and alive as long as the plan is used; the library lays `fine` and `order`
+ * out inside it.  bam_plan_workspace_bytes returns 0 when no plan is built for that size
  * (S above 131072); bam_tile_plan then refuses, and the caller uses bam_tile_flags and passes no plan.
  */
 int64_t bam_plan_workspace_bytes(int B, int S);

@@ -27,13 +27,7 @@ def build_plan(bf):
     flags = BA.BitfieldUtils.materialize_compressed_mask_from_bitfield_mask(bf)
     plan = BA.BitfieldUtils.plan_for(flags, bf)
     assert plan is not None
-    st = plan.struct
-    B, S = bf.shape
-    slots, num_n = 4 * -(-S // 128), -(-S // 32)
-    ws = plan.workspace
-    base = ws.data_ptr()
-    fine = torch.as_strided(ws, (B, slots, num_n), (st.fine_stride_b, st.fine_stride_s, 1), st.fine - base)
-    order = torch.as_strided(ws.view(torch.int32), (B, slots), (st.order_stride_b, 1), (st.order - base) // 4)
+    fine, order = plan.fine_classes(), plan.slice_order()
     torch.cuda.synchronize()
     return flags, fine.clone(), order.clone(), plan
 
