@@ -157,15 +157,14 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
             stDO.issue(j - CPT, gh + 2 * (int64_t)row_lo * p.dout.ss, gh + 2 * (int64_t)row_hi * p.dout.ss,
                        ldsDO + buf * TILE_BYTES);
         } else if (j == 2 * CPT) {
-            if (small < 2) {
-                // 32 floats of each slice: lanes 32..63 are moved from "the rows after row_lo + 31" to row_hi
-                const int64_t off = ((int64_t)b * p.Hq + h) * p.Sq_rounded + row_lo;
-                const unsigned voff = (unsigned)(lane * 4 + (lane >= 32 ? (row_hi - row_lo - 32) * 4 : 0));
-                dma_b32(small == 0 ? (const void*)(p.lse + off) : (const void*)(p.delta + off), voff,
-                        ldsSmall + buf * smallBytes);
-            } else {  // 32 int64 bitfields = 64 dwords: of slice lo (small == 2) or slice hi (small == 3)
-                dma_b32(bfrow + (small == 2 ? row_lo : row_hi), (unsigned)(lane * 4), ldsSmall + buf * smallBytes);
-            }
+            // lse / delta (small < 2): 32 floats of each slice, lanes 32..63 are moved from "the rows after
+            // row_lo + 31" to row_hi.  Bitfields: 32 int64 = 64 dwords of slice lo (small == 2) or hi (small == 3).
+            const int64_t off = ((int64_t)b * p.Hq + h) * p.Sq_rounded + row_lo;
+            const void* src = small == 0   ? (const void*)(p.lse + off)
+                              : small == 1 ? (const void*)(p.delta + off)
+                                           : (const void*)(bfrow + (small == 2 ? row_lo : row_hi));
+            const int shift = small < 2 ? (row_hi - row_lo - 32) * 4 : 0;
+            dma_b32(src, (unsigned)(lane * 4 + (lane >= 32 ? shift : 0)), ldsSmall + buf * smallBytes);
         } else {  // 2 x 32 row positions; every wave writes the same values
             const unsigned voff = (unsigned)(lane * 4 + (lane >= 32 ? (row_hi - row_lo - 32) * 4 : 0));
             dma_b32(p.posq + row_lo, voff, lds_addr(sQpos) + buf * (DKDV_QT * 4u));
