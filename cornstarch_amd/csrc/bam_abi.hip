@@ -7,7 +7,15 @@
 
 #include "bam_launch.h"
 
+// Built-in plan workspace of bam_tile_plan_static: device memory that exists once per GPU for as long as the
+// process lives.  In host code this name is only a handle for hipGetSymbolAddress; kernels and the other entry
+// points are handed the address that call returns for the current device (g_static_plan_ptr).
+static __device__ __align__(256) unsigned char g_static_plan_scratch[BAM_STATIC_PLAN_BYTES];
+
 namespace {
+
+constexpr int kMaxDevices = 64;
+void* g_static_plan_ptr[kMaxDevices] = {};  // per device, resolved on first use
 
 thread_local char g_error[512] = "";
 
@@ -316,6 +324,30 @@ int bam_tile_plan(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int64_t
                                           l.fine_sb, l.fine_ss, (int*)(w + l.order_off), l.order_sb, B, S,
                                           (hipStream_t)stream),
                     "bam_tile_plan");
+}
+
+int bam_tile_plan_static(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int64_t flags_stride_b,
+                         int64_t flags_stride_m, int B, int S, bam_plan* plan, void* stream) {
+    if (B <= 0 || S <= 0) return fail(BAM_ERR_INVALID_ARGUMENT, "bam_tile_plan_static: B and S must be positive");
+    const int64_t need = bam_plan_workspace_bytes(B, S);
+    if (need == 0 || need > BAM_STATIC_PLAN_BYTES)
+        return fail(BAM_ERR_UNSUPPORTED,
+                    "bam_tile_plan_static: B = %d, S = %d needs a plan workspace of %lld bytes, the built-in one holds %lld "
+                    "(use bam_tile_plan with a workspace of your own)",
+                    B, S, (long long)need, (long long)BAM_STATIC_PLAN_BYTES);
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices)
+        return fail(BAM_ERR_LAUNCH, "bam_tile_plan_static: no current device (or more than %d devices)", kMaxDevices);
+    if (g_static_plan_ptr[dev] == nullptr) {
+        // once per device, with that device current: the array's own address on this GPU
+        void* ptr = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(g_static_plan_scratch));
+        if (e != hipSuccess || ptr == nullptr)
+            return fail(BAM_ERR_LAUNCH, "bam_tile_plan_static: hipGetSymbolAddress failed: %s", hipGetErrorString(e));
+        g_static_plan_ptr[dev] = ptr;
+    }
+    return bam_tile_plan(bf, bf_stride_b, flags, flags_stride_b, flags_stride_m, g_static_plan_ptr[dev],
+                         BAM_STATIC_PLAN_BYTES, B, S, plan, stream);
 }
 
 int bam_materialize_mask(const int64_t* bf, int64_t bf_stride_b, uint8_t* out, int B, int S, void* stream) {

@@ -14,6 +14,7 @@ LIB_PATH = os.path.join(_PKG_DIR, "libbam_hip.so")
 BAM_DTYPE_F16 = 0
 BAM_DTYPE_BF16 = 1
 BAM_MAX_SEQLEN = 131072
+BAM_STATIC_PLAN_BYTES = 8 << 20
 ABI_VERSION = 6
 
 _i64 = ctypes.c_int64
@@ -71,6 +72,7 @@ SIGNATURES = {
     "bam_tile_flags": [_ptr, _i64, _ptr, _i64, _i64, _int, _int, _ptr],
     "bam_materialize_mask": [_ptr, _i64, _ptr, _int, _int, _ptr],
     "bam_tile_plan": [_ptr, _i64, _ptr, _i64, _i64, _ptr, _i64, _int, _int, _plan, _ptr],
+    "bam_tile_plan_static": [_ptr, _i64, _ptr, _i64, _i64, _int, _int, _plan, _ptr],
     "bam_fwd": [_ptr] * 7 + [_i64] * 15 + [_int] * 5 + [_f32, _int, _bias, _plan, _ptr],
     "bam_bwd_preprocess": [_ptr] * 3 + [_i64] * 6 + [_int] * 5 + [_ptr],
     "bam_bwd": [_ptr] * 11 + [_i64] * 24 + [_int] * 5 + [_f32, _int, _int, _bias, _plan, _ptr],

@@ -128,6 +128,20 @@ int bam_tile_plan(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int64_t
                   void* stream);
 
 /*
+ * bam_tile_plan without a workspace argument, for callers that cannot allocate device memory (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.
+ * The plan is laid out in a device array built into the library (BAM_STATIC_PLAN_BYTES per GPU, held until the
+ * process ends); the call allocates nothing and launches the same kernel as bam_tile_plan.  Sizes whose plan does
+ * not fit (bam_plan_workspace_bytes(B, S) > BAM_STATIC_PLAN_BYTES, e.g. one sequence above ~90k tokens) are refused
+ * with BAM_ERR_UNSUPPORTED.  Every call on a GPU reuses that GPU's array: the plan it returns is valid until the
+ * next call of this function on the same GPU, and calls whose work overlaps on one GPU (two streams, two threads)
+ * race.  Nothing in the array has to start at zero: every byte a later kernel reads is rewritten by each call.
+ */
+#define BAM_STATIC_PLAN_BYTES (8 << 20)
+int bam_tile_plan_static(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int64_t flags_stride_b,
+                         int64_t flags_stride_m, int B, int S, bam_plan* plan, void* stream);
+
+/*
  * Dense bool mask, uint8 (B, S, S) contiguous: the allow rule for every pair
  * (device function `_materialize_bitfield_mask_block`, bitfield_attention.py:60-101,
  * which the reference's test wraps in a kernel of its own,
