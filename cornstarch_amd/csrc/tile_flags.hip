@@ -34,7 +34,8 @@ __device__ __forceinline__ void slice_sort_key(const int64_t* __restrict__ row, 
     const int64_t M = (((int64_t)1) << 62) - 1;
     int64_t sig = 0;
     bool text = false;
-    for (int r = 0; r < 32; ++r) {
+#pragma unroll
+    for (int r = 0; r < 32; ++r) {  // 32 independent loads, all in flight together
         const int i = s * 32 + r;
         const int64_t f = i < S ? row[i] : 0;
         sig |= f & M;
@@ -54,7 +55,12 @@ __device__ __forceinline__ void slice_order_part(const int64_t* __restrict__ row
     int rank = 0;
     for (int base = 0; base < ns; base += 256) {
         __syncthreads();
-        slice_sort_key(row, S, ns, base + tid, sk[2 * tid], sk[2 * tid + 1]);
+        if (base == part * 256) {  // this workgroup's own slices: the keys are already there
+            sk[2 * tid] = my1;
+            sk[2 * tid + 1] = my2;
+        } else {
+            slice_sort_key(row, S, ns, base + tid, sk[2 * tid], sk[2 * tid + 1]);
+        }
         __syncthreads();
         const int cnt = min(256, ns - base);
         for (int j = 0; j < cnt; ++j) {
@@ -86,9 +92,13 @@ __global__ __launch_bounds__(FLAG_WAVES * 64) void tile_flags_kernel(const int64
         return;
     }
     __shared__ int64_t q_bits[BLOCK_M];
+    // classes of this workgroup's eight column tiles: row 0 the flag, rows 1..4 the four row slices; written out
+    // together at the end (eight bytes per row in one store where the layout guarantees alignment)
+    __shared__ __attribute__((aligned(8))) uint8_t s_out[5][FLAG_COLS_PER_BLOCK];
     const int b = blockIdx.z, m = blockIdx.y;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int64_t* row = bf + (int64_t)b * bf_stride_b;
+    if (tid < 5 * FLAG_COLS_PER_BLOCK) s_out[0][tid] = 0;
     if (tid < BLOCK_M) {
         const int i = m * BLOCK_M + tid;
         q_bits[tid] = (i < S) ? row[i] : 0;  // out-of-range positions read 0 (reference :86-87)
@@ -125,12 +135,13 @@ __global__ __launch_bounds__(FLAG_WAVES * 64) void tile_flags_kernel(const int64
                 } else {
                     f = (qb == kb && qb != 0) ? 2 : 0;
                 }
-                if (lane == 0) flags[(int64_t)b * flags_stride_b + (int64_t)m * flags_stride_m + n] = f;
+                const int col = wave * FLAG_TILES_PER_WAVE + t;
+                if (lane == 0) s_out[0][col] = (uint8_t)f;
                 if (FINE && lane < 4) {  // the same closed form for the 32 rows of slice `lane`
                     const int rs = r0 + 32 * lane;
                     int8_t fw = f;
                     if (q0 & 1) fw = (qb & kb) == 0 ? 0 : rs >= c0 + BLOCK_N - 1 ? 2 : rs + 31 < c0 ? 0 : 1;
-                    fine[(int64_t)b * fine_sb + (int64_t)(4 * m + lane) * fine_ss + n] = (uint8_t)fw;
+                    s_out[1 + lane][col] = (uint8_t)fw;
                 }
                 continue;
             }
@@ -143,6 +154,7 @@ __global__ __launch_bounds__(FLAG_WAVES * 64) void tile_flags_kernel(const int64
             cnt_b += allow_rule(q_bits[ri + 32], kf, (int64_t)m * BLOCK_M + ri + 32, j) ? 1 : 0;
         }
         const int cols_in_range = min(BLOCK_N, S - n * BLOCK_N);
+        const int col = wave * FLAG_TILES_PER_WAVE + t;
         if (FINE) {
 #pragma unroll
             for (int off = 16; off > 0; off >>= 1) {  // over the 32 columns, inside each half of the wave
@@ -154,23 +166,29 @@ __global__ __launch_bounds__(FLAG_WAVES * 64) void tile_flags_kernel(const int64
                 for (int x = 0; x < 2; ++x) {
                     const int w = 2 * half + x, c = x ? cnt_b : cnt_a;
                     const int rows = max(0, min(32, S - (m * BLOCK_M + 32 * w)));
-                    fine[(int64_t)b * fine_sb + (int64_t)(4 * m + w) * fine_ss + n] =
-                        (uint8_t)(c == 0 ? 0 : c == rows * cols_in_range ? 2 : 1);
+                    s_out[1 + w][col] = (uint8_t)(c == 0 ? 0 : c == rows * cols_in_range ? 2 : 1);
                 }
             }
             int cnt = cnt_a + cnt_b;
             cnt += __shfl_xor(cnt, 32);
-            if (lane == 0)
-                flags[(int64_t)b * flags_stride_b + (int64_t)m * flags_stride_m + n] =
-                    cnt == 0 ? 0 : cnt == rows_in_range * cols_in_range ? 2 : 1;  // full over in-range cells (:149-153)
+            // full over in-range cells (:149-153)
+            if (lane == 0) s_out[0][col] = (uint8_t)(cnt == 0 ? 0 : cnt == rows_in_range * cols_in_range ? 2 : 1);
         } else {
             int cnt = cnt_a + cnt_b;
 #pragma unroll
             for (int off = 32; off > 0; off >>= 1) cnt += __shfl_xor(cnt, off);
-            if (lane == 0)
-                flags[(int64_t)b * flags_stride_b + (int64_t)m * flags_stride_m + n] =
-                    cnt == 0 ? 0 : cnt == rows_in_range * cols_in_range ? 2 : 1;  // full over in-range cells (:149-153)
+            if (lane == 0) s_out[0][col] = (uint8_t)(cnt == 0 ? 0 : cnt == rows_in_range * cols_in_range ? 2 : 1);
         }
+    }
+    __syncthreads();
+    const int n0 = blockIdx.x * FLAG_COLS_PER_BLOCK;
+    if (tid < FLAG_COLS_PER_BLOCK && n0 + tid < num_n)  // the flag row may start anywhere: single bytes
+        flags[(int64_t)b * flags_stride_b + (int64_t)m * flags_stride_m + n0 + tid] = (int8_t)s_out[0][tid];
+    if (FINE && tid >= 64 && tid < 68) {  // rows of the class matrix are padded to 16 bytes: one 8-byte store
+        static_assert(FLAG_COLS_PER_BLOCK == 8, "one 64-bit word per row");
+        const int w = tid - 64;
+        *(unsigned long long*)(fine + (int64_t)b * fine_sb + (int64_t)(4 * m + w) * fine_ss + n0) =
+            *(const unsigned long long*)s_out[1 + w];
     }
 }
 

@@ -127,6 +127,7 @@ class BitfieldUtils:
         cls._cache_key = None
         cls._cache_owner = None
         cls._plan = None
+        _IndexView.forget()
 
     @classmethod
     def plan_for(cls, compressed_mask: torch.Tensor, bitfield_mask: torch.Tensor) -> Optional[_TilePlan]:
@@ -290,6 +291,31 @@ class _IndexView:
 
         return ctypes.byref(self.struct)
 
+    # The context-parallel caller runs the forward and, later, the backward of one shard with the same three
+    # tensors (context_parallel_bitfield_attention.py:137-147, 270-294): the last view is kept, together with the
+    # tensors it was gathered from (so their addresses cannot be handed to other tensors meanwhile), and reused
+    # while those are unchanged.
+    _last = None
+
+    @staticmethod
+    def _tensor_key(t: torch.Tensor):
+        return (t.data_ptr(), tuple(t.shape), tuple(t.stride()), t._version, t.device, t.dtype)
+
+    @classmethod
+    def get(cls, bitfield_mask: torch.Tensor, offsets_q: torch.Tensor, offsets_k: torch.Tensor) -> "_IndexView":
+        if offsets_q is None or offsets_k is None:
+            raise ValueError("offsets_q and offsets_k must be given together")
+        key = tuple(cls._tensor_key(t) for t in (bitfield_mask, offsets_q, offsets_k))
+        if cls._last is not None and cls._last[0] == key:
+            return cls._last[1]
+        view = cls(bitfield_mask, offsets_q, offsets_k)
+        cls._last = (key, view, (bitfield_mask, offsets_q, offsets_k))
+        return view
+
+    @classmethod
+    def forget(cls):
+        cls._last = None
+
 
 def _bitfield_attn_forward(
     q: torch.Tensor,
@@ -317,7 +343,7 @@ def _bitfield_attn_forward(
     bias_view = _BiasView(bias, q, batch, nheads, seqlen_q, seqlen_k) if bias is not None else None
     view = None
     if offsets_q is not None or offsets_k is not None:
-        view = _IndexView(bitfield_mask, offsets_q, offsets_k)
+        view = _IndexView.get(bitfield_mask, offsets_q, offsets_k)
         assert (view.seqlen_q, view.seqlen_k) == (seqlen_q, seqlen_k), "one offset per local query row / key"
     else:
         assert seqlen_q == seqlen_k, "without index tensors query and key sequence lengths must match"
@@ -493,7 +519,7 @@ def _bitfield_attn_backward(
     bias_view = _BiasView(bias, q, batch, nheads, seqlen_q, seqlen_k, may_copy=False) if bias is not None else None
     view = None
     if offsets_q is not None or offsets_k is not None:
-        view = _IndexView(bitfield_mask, offsets_q, offsets_k)
+        view = _IndexView.get(bitfield_mask, offsets_q, offsets_k)
         assert (view.seqlen_q, view.seqlen_k) == (seqlen_q, seqlen_k), "one offset per local query row / key"
     else:
         assert seqlen_q == seqlen_k, "without index tensors query and key sequence lengths must match"

@@ -144,3 +144,33 @@ def test_one_offset_tensor_without_the_other_is_rejected():
     flags = torch.zeros((1, 1, 4), dtype=torch.int8, device=d)
     with pytest.raises(ValueError):
         BA._bitfield_attn_forward(q, q, q, bf, flags, offsets_q=torch.arange(128, device=d))
+
+
+def test_index_view_is_gathered_once_per_forward_backward_pair():
+    # the backward of a shard reuses the gathered bitfields / positions of its forward; a changed offset tensor
+    # (new tensor, or the same tensor written in place) is gathered again
+    d = dev()
+    S = 300
+    bf = random_bitfield(1, S, seed=4).to(d)
+    q, k, v, do = (t.to(d) for t in inputs(1, S, 2, 1, 64, torch.bfloat16, seed=4))
+    off = torch.randperm(S, generator=torch.Generator().manual_seed(1)).to(d)
+    BA.BitfieldUtils.clear_cache()
+    assert BA._IndexView._last is None
+    view_flags = O.tile_flags_indexed(bf.cpu(), off.cpu(), off.cpu()).to(d)
+    o, lse, sc = BA._bitfield_attn_forward(q, k, v, bf, view_flags, offsets_q=off, offsets_k=off)
+    first = BA._IndexView._last[1]
+    grads = [torch.zeros_like(t, dtype=torch.float32) for t in (q, k, v)]
+    BA._bitfield_attn_backward(do, q, k, v, o, bf, view_flags, lse, *grads, offsets_q=off, offsets_k=off)
+    assert BA._IndexView._last[1] is first
+    off2 = off.clone()
+    BA._bitfield_attn_forward(q, k, v, bf, view_flags, offsets_q=off2, offsets_k=off2)
+    assert BA._IndexView._last[1] is not first
+    second = BA._IndexView._last[1]
+    off2[:2] = off2[:2].flip(0)  # in-place edit: version bump
+    fl2 = O.tile_flags_indexed(bf.cpu(), off2.cpu(), off2.cpu()).to(d)
+    o2, _, _ = BA._bitfield_attn_forward(q, k, v, bf, fl2, offsets_q=off2, offsets_k=off2)
+    assert BA._IndexView._last[1] is not second
+    o_ref, _ = O.attention_forward(q.cpu(), k.cpu(), v.cpu(), bf.cpu(), idx_q=off2.cpu(), idx_k=off2.cpu())
+    assert (o2.float().cpu() - o_ref).abs().max().item() <= O_MAX_ABS
+    BA.BitfieldUtils.clear_cache()
+    assert BA._IndexView._last is None
