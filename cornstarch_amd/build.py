@@ -16,7 +16,8 @@ from concurrent.futures import ThreadPoolExecutor
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_PATH = os.path.join(PKG_DIR, "libbam_hip.so")
-SOURCES = ["bam_abi.hip", "tile_flags.hip", "fwd.hip", "bwd.hip"]
+# the longest compilations first: they are spread over the workers
+SOURCES = ["bwd_long.hip", "bwd_dkdv.hip", "bwd_dq.hip", "fwd_long.hip", "fwd.hip", "tile_flags.hip", "bam_abi.hip"]
 ARCH = "gfx950"
 FLAGS = [
     f"--offload-arch={ARCH}",
@@ -58,7 +59,7 @@ def build_library(force: bool = True, verbose: bool = False) -> str:
             sys.stderr.write(r.stderr)
         return obj
 
-    with ThreadPoolExecutor(max_workers=4) as ex:
+    with ThreadPoolExecutor(max_workers=min(len(SOURCES), os.cpu_count() or 4)) as ex:
         objs = list(ex.map(compile_one, SOURCES))
     tmp = LIB_PATH + ".tmp"
     r = subprocess.run([hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", tmp, *objs],

@@ -10,11 +10,13 @@ constexpr int MASK_BITFIELD = 0;  // bitfield rule, position = row / column numb
 constexpr int MASK_INDEXED = 1;   // bitfield rule on gathered bitfields and explicit global positions
 constexpr int MASK_DENSE = 2;     // a materialized bool mask (B, Sq, Sk), one byte per pair (or none: all pairs allowed)
 
-// Longest sequence the attention kernels accept: a workgroup lists its 64-key tiles (forward, dQ) or its 32-row
-// slices (dK/dV) in LDS.
-constexpr int MAX_SEQLEN = 131072;
-constexpr int MAX_LIST = MAX_SEQLEN / 64;         // 64-key tiles of a row
-constexpr int MAX_SLICE_LIST = MAX_SEQLEN / 32;   // 32-row slices of a column
+// A workgroup lists its 64-key tiles (forward, dQ) or its 32-row slices (dK/dV) in LDS, this many at a time;
+// sequences beyond 131072 tokens take several passes.
+constexpr int MAX_LIST = 2048;         // 64-key tiles per pass
+constexpr int MAX_SLICE_LIST = 4096;   // 32-row slices per pass
+// Longest sequence the entry points accept (tile numbers are packed with eight class bits into 32-bit list entries,
+// positions are 32-bit; the bound leaves a wide margin to both).
+constexpr int MAX_SEQLEN = 1 << 22;
 // A plan (fine classes + slice order) is only built for sequences up to this many 32-row slices.
 constexpr int MAX_PLAN_SLICES = 4096;
 

@@ -179,17 +179,18 @@ __device__ __forceinline__ WaveSlices pick_wave_slices(const AttnParams& p, int 
     return w;
 }
 
-// List, in ascending order, the 64-key tiles the four slices of a workgroup have to visit.
+// List, in ascending order, the 64-key tiles the four slices of a workgroup have to visit, among the (at most
+// MAX_LIST) tiles starting at tile kt_begin; longer sequences are walked in several passes.
 // entry = (tile << 8) | c0 | c1 << 2 | c2 << 4 | c3 << 6 ; c_w is the class of the tile for wave w's slice:
 // 0 nothing to do, 1 evaluate the mask, 2 every pair allowed.
 // A tile is "full" for a slice only when both of its 32-column classes say so AND it has no column past
 // the end of the sequence (those columns must still be masked out of the softmax).
 // Executed by wave 0; the caller synchronizes before reading.
-__device__ __forceinline__ void build_key_tile_list(const WaveSlices& ws, int num_n, int S, int lane, int* list,
-                                                    int* count_out) {
-    const int nkt = (S + 63) >> 6;
+__device__ __forceinline__ void build_key_tile_list(const WaveSlices& ws, int num_n, int S, int lane, int kt_begin,
+                                                    int* list, int* count_out) {
+    const int nkt = min((S + 63) >> 6, kt_begin + MAX_LIST);
     int count = 0;
-    for (int base = 0; base < nkt; base += 64) {
+    for (int base = kt_begin; base < nkt; base += 64) {
         const int kt = base + lane;
         int packed = 0;
         if (kt < nkt) {
@@ -211,15 +212,16 @@ __device__ __forceinline__ void build_key_tile_list(const WaveSlices& ws, int nu
     if (lane == 0) *count_out = count;
 }
 
-// List, in ascending order, the 32-row slices that have work for a 128-key tile (4 class columns).
+// List, in ascending order, the 32-row slices among [s_begin, s_end) (at most MAX_SLICE_LIST of them; longer
+// sequences are walked in several passes) that have work for a 128-key tile (4 class columns).
 // entry = (slice << 8) | c0 | c1 << 2 | c2 << 4 | c3 << 6, c_w = class of (slice, key column 4 nt + w).
 // With a plan the classes are those of the 32 x 32 tiles; without one a slice inherits the flags of its
 // 128-row block.
-__device__ __forceinline__ void build_slice_list(const AttnParams& p, int b, int nt, int lane, int* list,
-                                                 int* count_out) {
-    const int ns = (p.Sq + 31) >> 5;
+__device__ __forceinline__ void build_slice_list(const AttnParams& p, int b, int nt, int lane, int s_begin, int s_end,
+                                                 int* list, int* count_out) {
+    const int ns = s_end;
     int count = 0;
-    for (int base = 0; base < ns; base += 64) {
+    for (int base = s_begin; base < ns; base += 64) {
         const int s = base + lane;
         int packed = 0;
         if (s < ns) {

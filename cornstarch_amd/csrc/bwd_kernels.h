@@ -1,4 +1,5 @@
-// Backward kernels of bitfield-masked attention for gfx950.
+// Backward kernels of bitfield-masked attention for gfx950 (templates; instantiated by bwd_dkdv.hip, bwd_dq.hip
+// and bwd_long.hip).
 // Reference semantics: cornstarch/kernel/bitfield_attention.py:527-572 (delta) and :598-929
 // (dQ, dK, dV).  The reference accumulates dQ, dK and dV with fp32 atomics; here every output
 // element has exactly one owner, so nothing is atomic and the sums are deterministic:
@@ -7,6 +8,7 @@
 //   dq kernel   : one workgroup per (batch, q head, 128-query block), looping over key tiles
 //                 exactly like the forward kernel.
 // Both recompute P = exp(scale * s - lse) from the saved log-sum-exp.
+#pragma once
 #include "bam_common.h"
 #include "bam_launch.h"
 #include "bam_tiles.h"
@@ -66,7 +68,9 @@ constexpr int DKDV_THREADS = 512;
 // MODE (MASK_*): MASK_INDEXED = explicit global positions p.posq / p.posk and gathered bitfield arrays;
 // MASK_DENSE = a materialized bool mask read from global memory in partial tiles.
 // BIAS: the forward added p.bias to scale * q.k (reference bitfield_attention.py:815-835); P is recomputed with it.
-template <typename T, int D, int MODE, bool BIAS>
+// LONG: sequences of more than MAX_SLICE_LIST 32-row slices (131072 rows), walked in several passes; the short form has
+// no pass loop at all (a loop around the main loop costs registers and a few per cent).
+template <typename T, int D, int MODE, bool BIAS, bool LONG>
 __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnParams p) {
     constexpr bool IDX = MODE == MASK_INDEXED, DENSE = MODE == MASK_DENSE;
     constexpr int NCH = D / 8, KK = D / 16, DB = D / 32;
@@ -94,7 +98,9 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
     const int b = ub % p.B;
     const int nt = ub / p.B;  // early key tiles (most queries under causality) first
 
-    if (wave == 0) build_slice_list(p, b, nt, lane, sList, &sCount);
+    const int ns_total = (Sq + 31) >> 5;
+    // first pass (usually the only one): the last MAX_SLICE_LIST slices
+    if (wave == 0) build_slice_list(p, b, nt, lane, max(0, ns_total - MAX_SLICE_LIST), ns_total, sList, &sCount);
 
     // ---- K, V of the tile -> LDS (once) ---------------------------------------------------
     {
@@ -337,89 +343,98 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
         }
     };
 
-    __syncthreads();
-    const int n_all = sCount;
-    // The last slice of a sequence whose length is not a multiple of 32 (always the last list entry) is
-    // staged synchronously, with neutral values for the rows past the end, after the main loop.
-    const bool ragged = (Sq & 31) != 0 && n_all > 0 &&
-                        (__builtin_amdgcn_readfirstlane(sList[n_all > 0 ? n_all - 1 : 0]) >> 8) == ((Sq - 1) >> 5);
-    const int n = n_all - (ragged ? 1 : 0);
-    // Main loop: the listed slices are taken in pairs from the END of the list (the workgroups of one kv head
-    // that are resident together then read the same Q / dO rows at about the same time, and all but the first
-    // of them find them in L2); pair r = entries n - 2 - 2 r (row stream 0) and n - 1 - 2 r (row stream 1).
-    // An odd count leaves the first entry alone: its pair repeats it with all classes cleared for stream 0.
-    // The q heads of the group follow one another: tile t = (head t / npairs, pair t % npairs).
-    const int npairs = (n + 1) >> 1;
-    const int total = npairs * G;
-    if (total > 0) {
-        auto entry_hi = [&](int r) { return sList[n - 1 - 2 * r]; };
-        auto entry_lo = [&](int r) { return n - 2 - 2 * r >= 0 ? sList[n - 2 - 2 * r] : (sList[0] & ~0xFF); };
-        auto advance = [&](int& g, int& r) {
-            if (++r == npairs) {
-                r = 0;
-                ++g;
-            }
-        };
-        int g_cur = 0, r_cur = 0, g_nxt = 0, r_nxt = 0;
-        advance(g_nxt, r_nxt);
-        int e_lo = __builtin_amdgcn_readfirstlane(entry_lo(0)), e_hi = __builtin_amdgcn_readfirstlane(entry_hi(0));
-        int n_lo = e_lo, n_hi = e_hi;
-        if (g_nxt < G) {
-            n_lo = __builtin_amdgcn_readfirstlane(entry_lo(r_nxt));
-            n_hi = __builtin_amdgcn_readfirstlane(entry_hi(r_nxt));
-        }
-#pragma unroll
-        for (int j = 0; j < NLOADS; ++j) issue_copy(j, hk * G, (e_lo >> 8) * 32, (e_hi >> 8) * 32, 0);
-        wait_async();
+    // Sequences of more than MAX_SLICE_LIST slices are walked in several passes, from the end, each with a list
+    // of its own; dK and dV live in registers and simply carry over.
+    for (int s_end = ns_total;;) {
         __syncthreads();
-        for (int it = 0; it < total; ++it) {
-            const int cur = it & 1;
-            // pair after next: its list entries are requested now and picked up at the end of the iteration
-            int g_aft = g_nxt, r_aft = r_nxt;
-            advance(g_aft, r_aft);
-            const int ra = g_aft < G ? r_aft : 0;
-            const int a_lo = entry_lo(ra), a_hi = entry_hi(ra);
-            // past the last tile the copies simply fetch it again (into the buffer nobody reads any more)
-            const bool more = it + 1 < total;
-            const int h_next = hk * G + (more ? g_nxt : g_cur);
-            const int lo_next = ((more ? n_lo : e_lo) >> 8) * 32, hi_next = ((more ? n_hi : e_hi) >> 8) * 32;
-            const int mine = st ? e_hi : e_lo;
-            tile_step(std::true_type{}, cur, (mine >> (2 * kg_lane)) & 3, hk * G + g_cur, (mine >> 8) * 32, h_next, lo_next,
-                      hi_next);
-            g_cur = g_nxt;
-            r_cur = r_nxt;
-            g_nxt = g_aft;
-            r_nxt = r_aft;
-            e_lo = n_lo;
-            e_hi = n_hi;
-            n_lo = __builtin_amdgcn_readfirstlane(a_lo);
-            n_hi = __builtin_amdgcn_readfirstlane(a_hi);
+        const int n_all = sCount;
+        // The last slice of a sequence whose length is not a multiple of 32 (always the last list entry) is
+        // staged synchronously, with neutral values for the rows past the end, after the main loop.
+        const bool ragged = (Sq & 31) != 0 && n_all > 0 &&
+                            (__builtin_amdgcn_readfirstlane(sList[n_all > 0 ? n_all - 1 : 0]) >> 8) == ((Sq - 1) >> 5);
+        const int n = n_all - (ragged ? 1 : 0);
+        // Main loop: the listed slices are taken in pairs from the END of the list (the workgroups of one kv head
+        // that are resident together then read the same Q / dO rows at about the same time, and all but the first
+        // of them find them in L2); pair r = entries n - 2 - 2 r (row stream 0) and n - 1 - 2 r (row stream 1).
+        // An odd count leaves the first entry alone: its pair repeats it with all classes cleared for stream 0.
+        // The q heads of the group follow one another: tile t = (head t / npairs, pair t % npairs).
+        const int npairs = (n + 1) >> 1;
+        const int total = npairs * G;
+        if (total > 0) {
+            auto entry_hi = [&](int r) { return sList[n - 1 - 2 * r]; };
+            auto entry_lo = [&](int r) { return n - 2 - 2 * r >= 0 ? sList[n - 2 - 2 * r] : (sList[0] & ~0xFF); };
+            auto advance = [&](int& g, int& r) {
+                if (++r == npairs) {
+                    r = 0;
+                    ++g;
+                }
+            };
+            int g_cur = 0, r_cur = 0, g_nxt = 0, r_nxt = 0;
+            advance(g_nxt, r_nxt);
+            int e_lo = __builtin_amdgcn_readfirstlane(entry_lo(0)), e_hi = __builtin_amdgcn_readfirstlane(entry_hi(0));
+            int n_lo = e_lo, n_hi = e_hi;
+            if (g_nxt < G) {
+                n_lo = __builtin_amdgcn_readfirstlane(entry_lo(r_nxt));
+                n_hi = __builtin_amdgcn_readfirstlane(entry_hi(r_nxt));
+            }
+    #pragma unroll
+            for (int j = 0; j < NLOADS; ++j) issue_copy(j, hk * G, (e_lo >> 8) * 32, (e_hi >> 8) * 32, 0);
             wait_async();
             __syncthreads();
-        }
-    }
-    if (ragged) {
-        wait_async();  // K, V of the tile, in case the main loop had nothing to do
-        const int entry = __builtin_amdgcn_readfirstlane(sList[n_all - 1]);
-        const int row0 = (entry >> 8) * 32;
-        const int rows = Sq - row0;  // rows of the slice inside the sequence (1..31)
-        for (int g = 0; g < G; ++g) {
-            const int h = hk * G + g;
-            __syncthreads();  // everybody is done with buffer 0
-            stQ.load_ragged((const char*)p.q.ptr + 2 * ((int64_t)b * p.q.sb + (int64_t)h * p.q.sh + (int64_t)row0 * p.q.ss), sQ[0], rows, tid);
-            stDO.load_ragged((const char*)p.dout.ptr + 2 * ((int64_t)b * p.dout.sb + (int64_t)h * p.dout.sh + (int64_t)row0 * p.dout.ss), sDO[0], rows, tid);
-            if (tid < DKDV_QT) {
-                const int64_t off = ((int64_t)b * p.Hq + h) * p.Sq_rounded + row0;
-                const bool ok = tid < rows;
-                sLse[0][tid] = ok ? p.lse[off + tid] : INFINITY;  // lse = +inf gives P = 0
-                sDelta[0][tid] = ok ? p.delta[off + tid] : 0.f;
-                if (!DENSE) sQbf[0][tid] = ok ? bfrow[row0 + tid] : 0;
-                if (IDX) sQpos[0][tid] = ok ? p.posq[row0 + tid] : 0;
+            for (int it = 0; it < total; ++it) {
+                const int cur = it & 1;
+                // pair after next: its list entries are requested now and picked up at the end of the iteration
+                int g_aft = g_nxt, r_aft = r_nxt;
+                advance(g_aft, r_aft);
+                const int ra = g_aft < G ? r_aft : 0;
+                const int a_lo = entry_lo(ra), a_hi = entry_hi(ra);
+                // past the last tile the copies simply fetch it again (into the buffer nobody reads any more)
+                const bool more = it + 1 < total;
+                const int h_next = hk * G + (more ? g_nxt : g_cur);
+                const int lo_next = ((more ? n_lo : e_lo) >> 8) * 32, hi_next = ((more ? n_hi : e_hi) >> 8) * 32;
+                const int mine = st ? e_hi : e_lo;
+                tile_step(std::true_type{}, cur, (mine >> (2 * kg_lane)) & 3, hk * G + g_cur, (mine >> 8) * 32, h_next, lo_next,
+                          hi_next);
+                g_cur = g_nxt;
+                r_cur = r_nxt;
+                g_nxt = g_aft;
+                r_nxt = r_aft;
+                e_lo = n_lo;
+                e_hi = n_hi;
+                n_lo = __builtin_amdgcn_readfirstlane(a_lo);
+                n_hi = __builtin_amdgcn_readfirstlane(a_hi);
+                wait_async();
+                __syncthreads();
             }
-            __syncthreads();
-            // the slice sits in LDS rows 0..31: row stream 0 computes it, row stream 1 has nothing to do
-            tile_step(std::false_type{}, 0, st ? 0 : (entry >> (2 * kg_lane)) & 3, h, row0, 0, 0, 0);
         }
+        if (ragged) {
+            wait_async();  // K, V of the tile, in case the main loop had nothing to do
+            const int entry = __builtin_amdgcn_readfirstlane(sList[n_all - 1]);
+            const int row0 = (entry >> 8) * 32;
+            const int rows = Sq - row0;  // rows of the slice inside the sequence (1..31)
+            for (int g = 0; g < G; ++g) {
+                const int h = hk * G + g;
+                __syncthreads();  // everybody is done with buffer 0
+                stQ.load_ragged((const char*)p.q.ptr + 2 * ((int64_t)b * p.q.sb + (int64_t)h * p.q.sh + (int64_t)row0 * p.q.ss), sQ[0], rows, tid);
+                stDO.load_ragged((const char*)p.dout.ptr + 2 * ((int64_t)b * p.dout.sb + (int64_t)h * p.dout.sh + (int64_t)row0 * p.dout.ss), sDO[0], rows, tid);
+                if (tid < DKDV_QT) {
+                    const int64_t off = ((int64_t)b * p.Hq + h) * p.Sq_rounded + row0;
+                    const bool ok = tid < rows;
+                    sLse[0][tid] = ok ? p.lse[off + tid] : INFINITY;  // lse = +inf gives P = 0
+                    sDelta[0][tid] = ok ? p.delta[off + tid] : 0.f;
+                    if (!DENSE) sQbf[0][tid] = ok ? bfrow[row0 + tid] : 0;
+                    if (IDX) sQpos[0][tid] = ok ? p.posq[row0 + tid] : 0;
+                }
+                __syncthreads();
+                // the slice sits in LDS rows 0..31: row stream 0 computes it, row stream 1 has nothing to do
+                tile_step(std::false_type{}, 0, st ? 0 : (entry >> (2 * kg_lane)) & 3, h, row0, 0, 0, 0);
+            }
+        }
+        if (!LONG) break;
+        s_end = max(0, s_end - MAX_SLICE_LIST);
+        if (s_end == 0) break;
+        __syncthreads();  // everybody has read the list of the pass that just ended
+        if (wave == 0) build_slice_list(p, b, nt, lane, max(0, s_end - MAX_SLICE_LIST), s_end, sList, &sCount);
     }
     // every copy has landed and every wave is done with the tiles: the epilogue reuses the tile arrays
     wait_async();
@@ -502,7 +517,8 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
 constexpr int DQ_KT = 64;
 constexpr int DQ_THREADS = 256;
 
-template <typename T, int D, int MODE, bool BIAS>
+// LONG: as in the dK/dV kernel, for more than MAX_LIST 64-key tiles.
+template <typename T, int D, int MODE, bool BIAS, bool LONG>
 __global__ __launch_bounds__(DQ_THREADS, D == 128 ? 2 : 3) void bwd_dq_kernel(const AttnParams p) {
     constexpr bool IDX = MODE == MASK_INDEXED, DENSE = MODE == MASK_DENSE;
     constexpr int NCH = D / 8, KK = D / 16, DB = D / 32;
@@ -527,7 +543,7 @@ __global__ __launch_bounds__(DQ_THREADS, D == 128 ? 2 : 3) void bwd_dq_kernel(co
     const int h = hk * G + g;
     const WaveSlices ws = pick_wave_slices(p, b, ub / p.B);  // group 0 is the heaviest
 
-    if (wave == 0) build_key_tile_list(ws, p.num_n, Sk, lane, sList, &sCount);
+    if (wave == 0) build_key_tile_list(ws, p.num_n, Sk, lane, 0, sList, &sCount);  // first pass (usually the only one)
 
     const int slice = __builtin_amdgcn_readfirstlane(wave == 0 ? ws.slice[0] : wave == 1 ? ws.slice[1] : wave == 2 ? ws.slice[2] : ws.slice[3]);
     const int qrow = (slice < 0 ? 0 : slice) * 32 + l32;
@@ -742,43 +758,52 @@ __global__ __launch_bounds__(DQ_THREADS, D == 128 ? 2 : 3) void bwd_dq_kernel(co
         }
     };
 
-    __syncthreads();
-    const int n_all = sCount;
-    // A tile that holds the end of a sequence whose length is not a multiple of 64 is always the last
-    // entry of the list; it is staged synchronously (zero fill past the end) after the main loop.
-    const bool ragged = (Sk & (DQ_KT - 1)) != 0 && n_all > 0 &&
-                        (__builtin_amdgcn_readfirstlane(sList[n_all > 0 ? n_all - 1 : 0]) >> 8) == ((Sk - 1) >> 6);
-    const int n = n_all - (ragged ? 1 : 0);
-    if (n > 0) {
-        int entry = __builtin_amdgcn_readfirstlane(sList[0]);
-        int next = __builtin_amdgcn_readfirstlane(sList[n > 1 ? 1 : 0]);
-#pragma unroll
-        for (int j = 0; j < NLOADS; ++j) issue_copy(j, entry >> 8, 0);
-        wait_async();
+    // Sequences of more than MAX_LIST 64-key tiles are walked in several passes, each with a list of its own.
+    const int nkt_total = (Sk + DQ_KT - 1) / DQ_KT;
+    for (int kt_begin = 0;;) {
         __syncthreads();
-        for (int it = 0; it < n; ++it) {
-            const int cur = it & 1;
-            // entry after next, requested now and picked up at the end of the iteration; past the end of the
-            // list the last tile is simply copied again (into the buffer nobody reads any more)
-            const int after = sList[it + 2 < n ? it + 2 : n - 1];
-            tile_step(std::true_type{}, cur, entry, next >> 8);
-            entry = next;
-            next = __builtin_amdgcn_readfirstlane(after);
+        const int n_all = sCount;
+        // A tile that holds the end of a sequence whose length is not a multiple of 64 is always the last
+        // entry of the list; it is staged synchronously (zero fill past the end) after the main loop.
+        const bool ragged = (Sk & (DQ_KT - 1)) != 0 && n_all > 0 &&
+                            (__builtin_amdgcn_readfirstlane(sList[n_all > 0 ? n_all - 1 : 0]) >> 8) == ((Sk - 1) >> 6);
+        const int n = n_all - (ragged ? 1 : 0);
+        if (n > 0) {
+            int entry = __builtin_amdgcn_readfirstlane(sList[0]);
+            int next = __builtin_amdgcn_readfirstlane(sList[n > 1 ? 1 : 0]);
+    #pragma unroll
+            for (int j = 0; j < NLOADS; ++j) issue_copy(j, entry >> 8, 0);
             wait_async();
             __syncthreads();
+            for (int it = 0; it < n; ++it) {
+                const int cur = it & 1;
+                // entry after next, requested now and picked up at the end of the iteration; past the end of the
+                // list the last tile is simply copied again (into the buffer nobody reads any more)
+                const int after = sList[it + 2 < n ? it + 2 : n - 1];
+                tile_step(std::true_type{}, cur, entry, next >> 8);
+                entry = next;
+                next = __builtin_amdgcn_readfirstlane(after);
+                wait_async();
+                __syncthreads();
+            }
         }
-    }
-    if (ragged) {
-        const int entry = __builtin_amdgcn_readfirstlane(sList[n_all - 1]);
-        const int kt = entry >> 8, rows = Sk - kt * DQ_KT;
-        stK.load_ragged(kbase + kt * k_ts, sK[0], rows, tid);
-        stV.load_ragged(vbase + kt * v_ts, sV[0], rows, tid);
-        if (!DENSE && tid < DQ_KT) {
-            sKbf[0][tid] = (tid < rows) ? bfrow[kt * DQ_KT + tid] : 0;
-            if (IDX) sKpos[0][tid] = (tid < rows) ? p.posk[kt * DQ_KT + tid] : 0;
+        if (ragged) {
+            const int entry = __builtin_amdgcn_readfirstlane(sList[n_all - 1]);
+            const int kt = entry >> 8, rows = Sk - kt * DQ_KT;
+            stK.load_ragged(kbase + kt * k_ts, sK[0], rows, tid);
+            stV.load_ragged(vbase + kt * v_ts, sV[0], rows, tid);
+            if (!DENSE && tid < DQ_KT) {
+                sKbf[0][tid] = (tid < rows) ? bfrow[kt * DQ_KT + tid] : 0;
+                if (IDX) sKpos[0][tid] = (tid < rows) ? p.posk[kt * DQ_KT + tid] : 0;
+            }
+            __syncthreads();
+            tile_step(std::false_type{}, 0, entry, 0);
         }
-        __syncthreads();
-        tile_step(std::false_type{}, 0, entry, 0);
+        if (!LONG) break;
+        kt_begin += MAX_LIST;
+        if (kt_begin >= nkt_total) break;
+        __syncthreads();  // everybody has read the list of the pass that just ended
+        if (wave == 0) build_key_tile_list(ws, p.num_n, Sk, lane, kt_begin, sList, &sCount);
     }
 
     if (qvalid && p.grad_typed) {  // overwrite mode: dq has the input dtype
@@ -807,45 +832,32 @@ __global__ __launch_bounds__(DQ_THREADS, D == 128 ? 2 : 3) void bwd_dq_kernel(co
     }
 }
 
+
 // ---------------------------------------------------------------------------------------
-template <typename T, int D>
-static int launch_pre_t(const AttnParams& p, hipStream_t stream) {
-    const int64_t threads = (int64_t)p.B * p.Sq * p.Hq * (D / 8);
-    const int64_t blocks = (threads + 255) / 256;
-    hipLaunchKernelGGL((bwd_preprocess_kernel<T, D>), dim3((unsigned)blocks), dim3(256), 0, stream, p);
-    return (int)hipGetLastError();
-}
-template <typename T, int D, bool BIAS>
+template <typename T, int D, bool BIAS, bool LONG>
 static int launch_dkdv_b(const AttnParams& p, hipStream_t stream) {
     const int blocks = p.num_kt * p.B * p.Hkv;  // one workgroup per 128-key tile
     if (p.mask_mode == MASK_INDEXED)
-        hipLaunchKernelGGL((bwd_dkdv_kernel<T, D, MASK_INDEXED, BIAS>), dim3(blocks), dim3(DKDV_THREADS), 0, stream, p);
+        hipLaunchKernelGGL((bwd_dkdv_kernel<T, D, MASK_INDEXED, BIAS, LONG>), dim3(blocks), dim3(DKDV_THREADS), 0, stream, p);
     else if (p.mask_mode == MASK_DENSE)
-        hipLaunchKernelGGL((bwd_dkdv_kernel<T, D, MASK_DENSE, BIAS>), dim3(blocks), dim3(DKDV_THREADS), 0, stream, p);
+        hipLaunchKernelGGL((bwd_dkdv_kernel<T, D, MASK_DENSE, BIAS, LONG>), dim3(blocks), dim3(DKDV_THREADS), 0, stream, p);
     else
-        hipLaunchKernelGGL((bwd_dkdv_kernel<T, D, MASK_BITFIELD, BIAS>), dim3(blocks), dim3(DKDV_THREADS), 0, stream, p);
+        hipLaunchKernelGGL((bwd_dkdv_kernel<T, D, MASK_BITFIELD, BIAS, LONG>), dim3(blocks), dim3(DKDV_THREADS), 0, stream, p);
     return (int)hipGetLastError();
 }
-template <typename T, int D>
-static int launch_dkdv_t(const AttnParams& p, hipStream_t stream) {
-    return p.bias != nullptr ? launch_dkdv_b<T, D, true>(p, stream) : launch_dkdv_b<T, D, false>(p, stream);
-}
-template <typename T, int D, bool BIAS>
+template <typename T, int D, bool BIAS, bool LONG>
 static int launch_dq_b(const AttnParams& p, hipStream_t stream) {
     const int blocks = p.num_m * p.B * p.Hq;
     if (p.mask_mode == MASK_INDEXED)
-        hipLaunchKernelGGL((bwd_dq_kernel<T, D, MASK_INDEXED, BIAS>), dim3(blocks), dim3(DQ_THREADS), 0, stream, p);
+        hipLaunchKernelGGL((bwd_dq_kernel<T, D, MASK_INDEXED, BIAS, LONG>), dim3(blocks), dim3(DQ_THREADS), 0, stream, p);
     else if (p.mask_mode == MASK_DENSE)
-        hipLaunchKernelGGL((bwd_dq_kernel<T, D, MASK_DENSE, BIAS>), dim3(blocks), dim3(DQ_THREADS), 0, stream, p);
+        hipLaunchKernelGGL((bwd_dq_kernel<T, D, MASK_DENSE, BIAS, LONG>), dim3(blocks), dim3(DQ_THREADS), 0, stream, p);
     else
-        hipLaunchKernelGGL((bwd_dq_kernel<T, D, MASK_BITFIELD, BIAS>), dim3(blocks), dim3(DQ_THREADS), 0, stream, p);
+        hipLaunchKernelGGL((bwd_dq_kernel<T, D, MASK_BITFIELD, BIAS, LONG>), dim3(blocks), dim3(DQ_THREADS), 0, stream, p);
     return (int)hipGetLastError();
 }
-template <typename T, int D>
-static int launch_dq_t(const AttnParams& p, hipStream_t stream) {
-    return p.bias != nullptr ? launch_dq_b<T, D, true>(p, stream) : launch_dq_b<T, D, false>(p, stream);
-}
 
+// fn<T, D>(p, stream) for the element type and head dimension of the call
 #define BAM_DISPATCH(fn)                                       \
     if (dtype == 1) {                                          \
         if (p.D == 128) return fn<BF16, 128>(p, stream);       \
@@ -855,9 +867,5 @@ static int launch_dq_t(const AttnParams& p, hipStream_t stream) {
     if (p.D == 128) return fn<F16, 128>(p, stream);            \
     if (p.D == 64) return fn<F16, 64>(p, stream);              \
     return fn<F16, 32>(p, stream);
-
-int launch_bwd_preprocess(const AttnParams& p, int dtype, hipStream_t stream) { BAM_DISPATCH(launch_pre_t) }
-int launch_bwd_dkdv(const AttnParams& p, int dtype, hipStream_t stream) { BAM_DISPATCH(launch_dkdv_t) }
-int launch_bwd_dq(const AttnParams& p, int dtype, hipStream_t stream) { BAM_DISPATCH(launch_dq_t) }
 
 }  // namespace bam

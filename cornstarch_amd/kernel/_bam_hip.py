@@ -13,7 +13,7 @@ LIB_PATH = os.path.join(_PKG_DIR, "libbam_hip.so")
 
 BAM_DTYPE_F16 = 0
 BAM_DTYPE_BF16 = 1
-BAM_MAX_SEQLEN = 131072
+BAM_MAX_SEQLEN = 4194304
 BAM_STATIC_PLAN_BYTES = 8 << 20
 ABI_VERSION = 6
 

@@ -33,8 +33,9 @@ extern "C" {
 #define BAM_DTYPE_F16 0
 #define BAM_DTYPE_BF16 1
 
-/* Upper bound on S accepted by the attention kernels (tile and slice lists live in LDS). */
-#define BAM_MAX_SEQLEN 131072
+/* Upper bound on S accepted by the attention kernels (a sanity bound: the kernels walk sequences beyond 131072
+ * tokens in several passes, so there is no structural limit short of 32-bit tile numbers). */
+#define BAM_MAX_SEQLEN 4194304
 
 /*
  * Index-tensor attention (context-parallel shards): the local query rows and keys are arbitrary

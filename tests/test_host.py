@@ -67,6 +67,9 @@ def test_abi_rejects_bad_arguments_without_touching_the_gpu():
     bias = _bam_hip.Bias(18, 0, 0, 0, 1)
     args = [ctypes.c_void_p(16)] * 7 + [8] * 15 + [1, 128, 4, 4, 64] + [0.125, 1, ctypes.byref(bias), None, None]
     assert lib.bam_fwd(*args) == -1 and b"bias" in lib.bam_last_error()
+    # a sequence beyond the sanity bound is refused with a clear error, before anything is launched
+    args = [ctypes.c_void_p(16)] * 7 + [8] * 15 + [1, _bam_hip.BAM_MAX_SEQLEN + 1, 4, 4, 64] + [0.125, 1, None, None, None]
+    assert lib.bam_fwd(*args) == -2 and b"BAM_MAX_SEQLEN" in lib.bam_last_error()
     with pytest.raises(_bam_hip.BamError):
         _bam_hip.call("bam_materialize_mask", None, 0, None, 1, 8, None)
 
