@@ -136,6 +136,19 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
     for (int i = 0; i < 16; ++i) zero16[i] = 0.f;
     const float c2 = BIAS ? LOG2E : p.scale * LOG2E;  // with a bias the scores become scale * s + bias first
 
+    // Flip the sign of every element of the V tile in LDS (once per workgroup, after the tile has landed and
+    // before anybody reads it; the caller brackets it with workgroup barriers).
+    auto negate_v_tile = [&]() {
+#pragma unroll
+        for (int i = 0; i < (128 * NCH) / DKDV_THREADS; ++i) {
+            u32x4 x = sV[tid + DKDV_THREADS * i];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) x[e] ^= 0x80008000u;
+            sV[tid + DKDV_THREADS * i] = x;
+        }
+    };
+    bool v_negated = false;
+
     typedef SliceStage<D, DKDV_THREADS> Stage;
     constexpr int CPT = Stage::CPT;
     // copy instructions per wave and tile: Q, dO, one of the four small rows and (IDX) the row positions
@@ -199,12 +212,23 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
         const u32x4* tG = sDO[cur];
         // ---- S = Q K^T and dP = dO V^T : 32 queries x 32 keys, two accumulator chains; both operands of
         // every MFMA come from LDS and are requested AHEAD MFMAs in front of their use
+        // The V tile in LDS is NEGATED (see negate_v_tile), and the dP accumulator starts from delta instead of
+        // zero: the chain then delivers delta - dO V^T = -(dP - delta) with no subtraction left for the VALU.
+        // The sign is carried through dS into dK and taken back by the epilogue.
         f32x16 s, dp;
         {
             constexpr int NOP = 2 * KK, AHEAD = 3;  // MFMA j: S (j even) or dP (j odd), k-slice j / 2
             u32x4 a[NOP], bb[NOP];
+            a[0] = lds_read_chunk<D>(tQ, qr + l32, hi);  // the operands of the first MFMA go first
+            bb[0] = lds_read_chunk<D>(sK, 32 * kg + l32, hi);
 #pragma unroll
-            for (int j = 0; j < AHEAD; ++j) {
+            for (int grp = 0; grp < 4; ++grp) {
+                const f32x4 d4 = *(const f32x4*)&sDelta[cur][qr + 8 * grp + 4 * hi];
+#pragma unroll
+                for (int x = 0; x < 4; ++x) dp[4 * grp + x] = d4[x];
+            }
+#pragma unroll
+            for (int j = 1; j < AHEAD; ++j) {
                 a[j] = lds_read_chunk<D>((j & 1) ? tG : tQ, qr + l32, 2 * (j >> 1) + hi);
                 bb[j] = lds_read_chunk<D>((j & 1) ? sV : sK, 32 * kg + l32, 2 * (j >> 1) + hi);
             }
@@ -216,14 +240,14 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
                     bb[j + AHEAD] = lds_read_chunk<D>(((j + AHEAD) & 1) ? sV : sK, 32 * kg + l32, 2 * ((j + AHEAD) >> 1) + hi);
                 }
                 if (j & 1)
-                    dp = T::mfma(a[j], bb[j], j < 2 ? zero16 : dp);
+                    dp = T::mfma(a[j], bb[j], dp);
                 else
                     s = T::mfma(a[j], bb[j], j < 2 ? zero16 : s);
                 if (PREFETCH && j < NLOADS) issue_copy(j, h_next, lo_next, hi_next, cur ^ 1);
             }
             __builtin_amdgcn_sched_barrier(0);
         }
-        // ---- P = exp(scale s - lse) on allowed pairs, dS/scale = P (dP - delta)   (the factor `scale` of dS
+        // ---- P = exp(scale s - lse) on allowed pairs, -dS/scale = P (delta - dP)   (the factor `-scale` of dS
         // is applied once to dK in the epilogue).  C fragment: register i <-> query row
         // 8*(i/4) + 4*hi + i%4 of this wave's 32 rows.
         if (BIAS) {
@@ -311,11 +335,7 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
             }
         }
 #pragma unroll
-        for (int grp = 0; grp < 4; ++grp) {
-            const f32x4 d4 = *(const f32x4*)&sDelta[cur][qr + 8 * grp + 4 * hi];
-#pragma unroll
-            for (int x = 0; x < 4; ++x) dp[4 * grp + x] = s[4 * grp + x] * (dp[4 * grp + x] - d4[x]);
-        }
+        for (int i = 0; i < 16; ++i) dp[i] = s[i] * dp[i];  // -dS / scale
         u32x4 pb[2], dsb[2];
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
@@ -381,6 +401,11 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
             for (int j = 0; j < NLOADS; ++j) issue_copy(j, hk * G, (e_lo >> 8) * 32, (e_hi >> 8) * 32, 0);
             wait_async();
             __syncthreads();
+            if (!v_negated) {  // K, V and the first tile have landed
+                negate_v_tile();
+                v_negated = true;
+                __syncthreads();
+            }
             for (int it = 0; it < total; ++it) {
                 const int cur = it & 1;
                 // pair after next: its list entries are requested now and picked up at the end of the iteration
@@ -409,6 +434,11 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
         }
         if (ragged) {
             wait_async();  // K, V of the tile, in case the main loop had nothing to do
+            if (!v_negated) {
+                __syncthreads();
+                negate_v_tile();
+                v_negated = true;  // (the barrier at the top of the loop below publishes it)
+            }
             const int entry = __builtin_amdgcn_readfirstlane(sList[n_all - 1]);
             const int row0 = (entry >> 8) * 32;
             const int rows = Sq - row0;  // rows of the slice inside the sequence (1..31)
@@ -468,7 +498,7 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
 #pragma unroll
                     for (int x = 0; x < 4; ++x) {
                         const int i = 4 * grp + x;
-                        a[x] = (dk[db][i] + park[(db * 16 + i) * 64 + lane]) * p.scale;
+                        a[x] = (dk[db][i] + park[(db * 16 + i) * 64 + lane]) * -p.scale;  // dk holds -dK / scale
                         c[x] = dv[db][i] + park[((DB + db) * 16 + i) * 64 + lane];
                     }
                     const int d0 = 32 * db + 8 * grp + 4 * hi;
@@ -498,7 +528,7 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
                     f32x4 a = *(f32x4*)(dkp + d0), c = *(f32x4*)(dvp + d0);
 #pragma unroll
                     for (int x = 0; x < 4; ++x) {
-                        a[x] = fmaf(dk[db][4 * grp + x], p.scale, a[x]);
+                        a[x] = fmaf(dk[db][4 * grp + x], -p.scale, a[x]);  // dk holds -dK / scale
                         c[x] += dv[db][4 * grp + x];
                     }
                     *(f32x4*)(dkp + d0) = a;
