@@ -34,7 +34,8 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="C2", choices=["C2", "C3", "C4", "C5"])
+    ap.add_argument("--workload", default="C2", choices=["C1", "C2", "C3", "C4", "C5"],
+                    help="C1 is the forward-only plumbing configuration (fp32 values rounded to bf16 for the kernels)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-other-workloads", action="store_true",
                     help="skip the short C3 / C4 / C5 records that accompany the default (C2) run")
@@ -47,8 +48,8 @@ def parse():
 
 def cpu_baseline(name):
     """Oracle (port of the reference tests' ground truth): bool mask from the bitfields +
-    library SDPA in fp32 on the host, fwd+bwd.  Bounded sample: the first KV group is timed first; if
-    that took under 2 s (C2, C4) the whole workload is timed, otherwise the one group stands."""
+    library SDPA in fp32 on the host, fwd+bwd (forward only for C1).  Bounded sample: the first KV group is timed
+    first; if that took under 2 s (C1, C2, C4) the whole workload is timed, otherwise the one group stands."""
     import torch
 
     from cornstarch_amd import workloads as W
@@ -60,28 +61,30 @@ def cpu_baseline(name):
     torch.set_num_threads(int(os.environ.get("OMP_NUM_THREADS") or 0) or os.cpu_count() or 1)
     bf = W.make_bitfields(name)
 
-    def timed(heads, reps):
+    def timed(heads, backward):
         q, k, v, do = (t.float() for t in W.make_tensors(name, heads=heads))
-        times = []
-        for _ in range(reps):
-            t0 = time.perf_counter()
-            O.sdpa_forward_backward(q, k, v, bf, do, row_chunk=2048)
-            times.append(time.perf_counter() - t0)
-        return min(times)
+        t0 = time.perf_counter()
+        O.sdpa_forward_backward(q, k, v, bf, do if backward else None, row_chunk=2048)
+        return time.perf_counter() - t0
 
-    t = timed((0, G), 2)
-    q_heads, sample = G, f"{name} q-heads 0..{G - 1} + kv-head 0, all {w.B} sequences"
+    backward = w.backward
+    heads, q_heads, sample = (0, G), G, f"{name} q-heads 0..{G - 1} + kv-head 0, all {w.B} sequences"
+    t = timed(heads, backward)
     if t < 2.0 and w.Hkv > 1:
-        t = timed(None, 1)
-        q_heads, sample = w.Hq, f"{name}, the whole workload"
-    flops = 14 * w.D * q_heads * O.unmasked_pairs(bf)
+        heads, q_heads, sample = None, w.Hq, f"{name}, the whole workload"
+        t = timed(heads, backward)
+    if t < 10.0:  # a second repetition where it is cheap; the faster one counts
+        t = min(t, timed(heads, backward))
+    t_fwd = timed(heads, False) if backward else t
+    flops = (14 if backward else 4) * w.D * q_heads * O.unmasked_pairs(bf)
     return {
         "value": flops / t / 1e12,
         "unit": "TFLOP/s",
         "cores": torch.get_num_threads(),
         "kind": "port",
         "seconds": t,
-        "sample": sample + ", fwd+bwd fp32 materialized-mask SDPA (oracle)",
+        "fwd_seconds": t_fwd,
+        "sample": sample + (", fwd+bwd" if backward else ", forward only") + " fp32 materialized-mask SDPA (oracle)",
     }
 
 
@@ -131,10 +134,13 @@ def run_workload(name, steps, warmup, dev):
 
     w = W.WORKLOADS[name]
     q, k, v, do = (t.to(dev) for t in W.make_tensors(name))
+    if q.dtype == torch.float32:  # C1: the kernels take the fp32 values rounded to bf16
+        q, k, v, do = (t.bfloat16() for t in (q, k, v, do))
+    backward = w.backward
     bf = W.make_bitfields(name).to(dev)
     pairs = O.unmasked_pairs(bf)  # exact, on the GPU through torch ops (setup, untimed)
     f_fwd = 4 * w.D * w.Hq * pairs
-    f_bwd = 10 * w.D * w.Hq * pairs
+    f_bwd = 10 * w.D * w.Hq * pairs if backward else 0
     scale = 1.0 / math.sqrt(w.D)
 
     stages = ["flags", "fwd", "alloc", "delta", "dkdv", "dq"]
@@ -152,6 +158,10 @@ def run_workload(name, steps, warmup, dev):
         mark(1)
         o, lse, _ = BA._bitfield_attn_forward(q, k, v, bf, flags, softmax_scale=scale)
         mark(2)
+        if not backward:
+            for i in range(3, n_ev):
+                mark(i)
+            return o, None
         dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
         delta = torch.empty_like(lse)
         mark(3)
@@ -188,6 +198,9 @@ def run_workload(name, steps, warmup, dev):
 
     def api_step():
         BA.BitfieldUtils.clear_cache()
+        if not backward:
+            with torch.no_grad():
+                return BA.bitfield_attn_func(qg, kg, vg, bf)
         o = BA.bitfield_attn_func(qg, kg, vg, bf)
         return torch.autograd.grad(o, (qg, kg, vg), do)
 
@@ -269,7 +282,8 @@ def main():
         "dtype": "bf16",
         "data": "synthetic",
         "config": {
-            "workload": f"{name}: B={w.B} S={w.S} Hq={w.Hq} Hkv={w.Hkv} D={w.D} bf16 fwd+bwd, {w.description}",
+            "workload": f"{name}: B={w.B} S={w.S} Hq={w.Hq} Hkv={w.Hkv} D={w.D} bf16 "
+                        f"{'fwd+bwd' if w.backward else 'forward only'}, {w.description}",
             "unmasked_pairs": pairs,
             "flops_fwd": f_fwd,
             "flops_bwd": f_bwd,
@@ -291,6 +305,10 @@ def main():
             "dkdv": round(r["issued"]["dkdv"] / (8 * w.D * w.Hq * pairs), 4),
             "dq": round(r["issued"]["dq"] / (6 * w.D * w.Hq * pairs), 4),
         },
+        # what the measurements say holds the dominant kernel back: no single saturated unit -- MFMA pipe 40-53 %
+        # busy, 29-35 % of wave time at s_waitcnt / barriers, 4-5 other vector instructions per MFMA
+        # (profiles/bam_kernels_C2_counters.txt)
+        "limiter": "latency / instruction mix, not a saturated unit",
         "roofline": {
             "kernel": kname[dom],
             "bound": "mfma",
