@@ -126,6 +126,19 @@ struct SliceStage {
             dma_b128<SITE>(upper ? hi : lo, goff[i], tile_lds + (unsigned)(THREADS * i + wave_first) * 16u);
         }
     }
+    // Does copy instruction i of this wave fill LDS rows 32..63 (slice `hi`)?  Wave-uniform, and a compile-time
+    // constant where every instruction covers whole 32-row halves (D = 128 with 512 threads).
+    __device__ __forceinline__ bool upper(int i) const {
+        if ((THREADS * (i + 1)) / NCH <= 32) return false;
+        if ((THREADS * i) / NCH >= 32) return true;
+        return (wave_first + THREADS * i) / NCH >= 32;
+    }
+    // As issue(), with the slice's base pointer already chosen by the caller (see upper()).
+    template <int SITE = 0>
+    __device__ __forceinline__ void issue_from(int i, const char* slice_base, unsigned tile_lds) const {
+        if (EXACT || wave_first + THREADS * i < CHUNKS)
+            dma_b128<SITE>(slice_base, goff[i], tile_lds + (unsigned)(THREADS * i + wave_first) * 16u);
+    }
     // synchronous, zero-filling copy of ONE slice with only rows_valid (<= 32) rows in range into LDS rows
     // [0, 32); rows [32, 64) are zeroed
     __device__ __forceinline__ void load_ragged(const char* slice_base, u32x4* tile, int rows_valid, int tid) const {
@@ -238,7 +251,12 @@ __device__ __forceinline__ void build_slice_list(const AttnParams& p, int b, int
         if (packed) list[count + __popcll(bal & ((1ull << lane) - 1ull))] = (s << 8) | packed;
         count += __popcll(bal);
     }
-    if (lane == 0) *count_out = count;
+    // list[-1] (the caller leaves room for it) repeats the first entry with all classes cleared: a consumer that
+    // takes the entries in pairs from the end finds a harmless partner for the first entry of an odd count there.
+    if (lane == 0) {
+        *count_out = count;
+        if (count > 0) list[-1] = list[0] & ~0xFF;
+    }
 }
 
 }  // namespace bam

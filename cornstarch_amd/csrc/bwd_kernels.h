@@ -83,7 +83,8 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
     __shared__ __attribute__((aligned(16))) int64_t sQbf[2][DKDV_QT];    // raw bitfields of the rows
     __shared__ __attribute__((aligned(16))) int sQpos[2][DKDV_QT];       // their global positions (IDX only)
     __shared__ __attribute__((aligned(16))) unsigned sWq[DKDV_THREADS / 64][5][32];  // per-wave rule constants
-    __shared__ int sList[MAX_SLICE_LIST];
+    __shared__ int sListStore[MAX_SLICE_LIST + 1];  // entry -1: partner of the first entry of an odd count
+    int* const sList = sListStore + 1;
     __shared__ int sCount;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -165,46 +166,85 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
     const int small = DENSE ? (wave & 1) : (wave & 3);
     const unsigned ldsSmall = small == 0 ? lds_addr(sLse) : small == 1 ? lds_addr(sDelta) : lds_addr(sQbf) + (small - 2) * 256u;
     const unsigned smallBytes = small < 2 ? DKDV_QT * 4u : DKDV_QT * 8u;  // per buffer
-    // Copy instruction j of the 64-row tile made of the slices starting at rows row_lo (LDS rows 0..31) and
-    // row_hi (LDS rows 32..63) of head h, into buffer buf.  row_lo <= row_hi, or the two are the same slice.
-    auto issue_copy = [&](int j, int h, int row_lo, int row_hi, int buf) {
-        if (j < CPT) {
-            const char* qh = (const char*)p.q.ptr + 2 * ((int64_t)b * p.q.sb + (int64_t)h * p.q.sh);
-            stQ.issue(j, qh + 2 * (int64_t)row_lo * p.q.ss, qh + 2 * (int64_t)row_hi * p.q.ss, ldsQ + buf * TILE_BYTES);
-        } else if (j < 2 * CPT) {
-            const char* gh = (const char*)p.dout.ptr + 2 * ((int64_t)b * p.dout.sb + (int64_t)h * p.dout.sh);
-            stDO.issue(j - CPT, gh + 2 * (int64_t)row_lo * p.dout.ss, gh + 2 * (int64_t)row_hi * p.dout.ss,
-                       ldsDO + buf * TILE_BYTES);
-        } else if (j == 2 * CPT) {
-            // lse / delta (small < 2): 32 floats of each slice, lanes 32..63 are moved from "the rows after
-            // row_lo + 31" to row_hi.  Bitfields: 32 int64 = 64 dwords of slice lo (small == 2) or hi (small == 3).
-            const int64_t off = ((int64_t)b * p.Hq + h) * p.Sq_rounded + row_lo;
-            const void* src = small == 0   ? (const void*)(p.lse + off)
-                              : small == 1 ? (const void*)(p.delta + off)
-                                           : (const void*)(bfrow + (small == 2 ? row_lo : row_hi));
-            const int shift = small < 2 ? (row_hi - row_lo - 32) * 4 : 0;
-            dma_b32(src, (unsigned)(lane * 4 + (lane >= 32 ? shift : 0)), ldsSmall + buf * smallBytes);
-        } else {  // 2 x 32 row positions; every wave writes the same values
-            const unsigned voff = (unsigned)(lane * 4 + (lane >= 32 ? (row_hi - row_lo - 32) * 4 : 0));
-            dma_b32(p.posq + row_lo, voff, lds_addr(sQpos) + buf * (DKDV_QT * 4u));
+    // Where the copies of a tile read.  The scalar unit is shared by the whole compute unit, so the address
+    // arithmetic is kept short: per-head base pointers are carried along and bumped when the head changes, row
+    // offsets are 32 x 32 -> 64 bit unsigned products (rows < 2^22, row strides < 2^25 bytes by the host checks).
+    struct HeadBase {
+        const char* q;      // first row of the head in q
+        const char* g;      // ... in dout
+        const char* small;  // this wave's small row: lse / delta of the head, or the bitfields (head independent)
+    };
+    const unsigned q_rs = (unsigned)(2 * p.q.ss), g_rs = (unsigned)(2 * p.dout.ss);  // row strides in bytes
+    const int64_t small_head_step = small < 2 ? (int64_t)p.Sq_rounded * 4 : 0;
+    auto head_base = [&](int h) {
+        HeadBase hb;
+        hb.q = (const char*)p.q.ptr + 2 * ((int64_t)b * p.q.sb + (int64_t)h * p.q.sh);
+        hb.g = (const char*)p.dout.ptr + 2 * ((int64_t)b * p.dout.sb + (int64_t)h * p.dout.sh);
+        hb.small = small == 0   ? (const char*)(p.lse + ((int64_t)b * p.Hq + h) * p.Sq_rounded)
+                   : small == 1 ? (const char*)(p.delta + ((int64_t)b * p.Hq + h) * p.Sq_rounded)
+                                : (const char*)bfrow;
+        return hb;
+    };
+    auto next_head = [&](HeadBase& hb) {
+        hb.q += 2 * (int64_t)p.q.sh;
+        hb.g += 2 * (int64_t)p.dout.sh;
+        hb.small += small_head_step;
+    };
+    // lanes 32..63 of a copy of 2 x 32 consecutive floats / ints take the second slice: their byte offset moves
+    // from "the rows after the first slice" to it
+    const unsigned upper_lanes = lane >= 32 ? 0xFFFFFFFFu : 0u;
+    struct TileSource {
+        const char* q[CPT];
+        const char* g[CPT];
+        const char* small;
+        const int* pos;
+        unsigned small_voff, pos_voff;
+    };
+    // the 64-row tile made of the slices starting at rows row_lo (LDS rows 0..31) and row_hi (LDS rows 32..63)
+    auto tile_source = [&](const HeadBase& hb, int row_lo, int row_hi) {
+        TileSource t;
+#pragma unroll
+        for (int i = 0; i < CPT; ++i) {
+            const unsigned row = (unsigned)(stQ.upper(i) ? row_hi : row_lo);
+            t.q[i] = hb.q + (uint64_t)row * q_rs;
+            t.g[i] = hb.g + (uint64_t)row * g_rs;
         }
+        // lse / delta (small < 2): 32 floats of each slice.  Bitfields: 32 int64 = 64 dwords of slice lo
+        // (small == 2) or hi (small == 3).
+        const unsigned srow = (unsigned)(small == 3 ? row_hi : row_lo);
+        t.small = hb.small + (small < 2 ? srow * 4u : srow * 8u);
+        const unsigned shift = (unsigned)((row_hi - row_lo - 32) * 4);
+        t.pos_voff = (unsigned)(lane * 4) + (shift & upper_lanes);
+        t.small_voff = small < 2 ? t.pos_voff : (unsigned)(lane * 4);
+        t.pos = IDX ? p.posq + row_lo : nullptr;
+        return t;
+    };
+    // copy instruction j of a tile into buffer buf
+    auto issue_copy = [&](int j, const TileSource& t, int buf) {
+        if (j < CPT)
+            stQ.issue_from(j, t.q[j], ldsQ + buf * TILE_BYTES);
+        else if (j < 2 * CPT)
+            stDO.issue_from(j - CPT, t.g[j - CPT], ldsDO + buf * TILE_BYTES);
+        else if (j == 2 * CPT)
+            dma_b32(t.small, t.small_voff, ldsSmall + buf * smallBytes);
+        else  // 2 x 32 row positions; every wave writes the same values
+            dma_b32(t.pos, t.pos_voff, lds_addr(sQpos) + buf * (DKDV_QT * 4u));
     };
 
     // One 64-row tile held in buffer cur against this wave's 32 keys; the wave's 32 rows sit at sequence
-    // rows myrow0.. and its class for them is cls.  With PREFETCH the copies of the next tile (head h_next,
-    // slices at rows lo_next / hi_next) into the other buffer are issued one per MFMA of the S / dP phase, or
-    // back to back when this wave has nothing to compute.
+    // rows myrow0.. and its class for them is cls.  With PREFETCH the copies of the next tile into the other buffer
+    // are issued one per MFMA of the S / dP phase, or back to back when this wave has nothing to compute.
     const int qr = 32 * st;  // this wave's rows inside the 64-row tile
     // The wave's flag class is extracted with a per-lane copy of the key group number on purpose: a branch
     // condition the compiler can prove wave-uniform makes it restructure the loop around that branch, and the
     // result needs far more registers than a wave has.
     const int kg_lane = (tid >> 6) & 3;
-    auto tile_step = [&](auto prefetch, int cur, int cls, int h_cur, int myrow0, int h_next, int lo_next, int hi_next) {
+    auto tile_step = [&](auto prefetch, int cur, int cls, int h_cur, int myrow0, const TileSource& next) {
         constexpr bool PREFETCH = decltype(prefetch)::value;
         if (cls == 0) {
             if (PREFETCH) {
 #pragma unroll
-                for (int j = 0; j < NLOADS; ++j) issue_copy(j, h_next, lo_next, hi_next, cur ^ 1);
+                for (int j = 0; j < NLOADS; ++j) issue_copy(j, next, cur ^ 1);
             }
             return;
         }
@@ -243,7 +283,7 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
                     dp = T::mfma(a[j], bb[j], dp);
                 else
                     s = T::mfma(a[j], bb[j], j < 2 ? zero16 : s);
-                if (PREFETCH && j < NLOADS) issue_copy(j, h_next, lo_next, hi_next, cur ^ 1);
+                if (PREFETCH && j < NLOADS) issue_copy(j, next, cur ^ 1);
             }
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -382,23 +422,25 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
         const int total = npairs * G;
         if (total > 0) {
             auto entry_hi = [&](int r) { return sList[n - 1 - 2 * r]; };
-            auto entry_lo = [&](int r) { return n - 2 - 2 * r >= 0 ? sList[n - 2 - 2 * r] : (sList[0] & ~0xFF); };
-            auto advance = [&](int& g, int& r) {
-                if (++r == npairs) {
-                    r = 0;
-                    ++g;
+            auto entry_lo = [&](int r) { return sList[n - 2 - 2 * r]; };  // entry -1 where the count is odd
+            // current tile (g_cur, entries e_*), next tile (g_nxt, r_nxt, entries n_*, head base hb_nxt); past the
+            // last tile "next" keeps walking through pairs of the last head, whose copies nobody reads
+            int g_cur = 0, g_nxt = 0, r_nxt = 0;
+            HeadBase hb_nxt = head_base(hk * G);
+            int e_lo = __builtin_amdgcn_readfirstlane(entry_lo(0)), e_hi = __builtin_amdgcn_readfirstlane(entry_hi(0));
+            {
+                const TileSource first = tile_source(hb_nxt, (e_lo >> 8) * 32, (e_hi >> 8) * 32);
+#pragma unroll
+                for (int j = 0; j < NLOADS; ++j) issue_copy(j, first, 0);
+            }
+            auto advance = [&]() {
+                if (++r_nxt == npairs) {
+                    r_nxt = 0;
+                    if (++g_nxt < G) next_head(hb_nxt);
                 }
             };
-            int g_cur = 0, r_cur = 0, g_nxt = 0, r_nxt = 0;
-            advance(g_nxt, r_nxt);
-            int e_lo = __builtin_amdgcn_readfirstlane(entry_lo(0)), e_hi = __builtin_amdgcn_readfirstlane(entry_hi(0));
-            int n_lo = e_lo, n_hi = e_hi;
-            if (g_nxt < G) {
-                n_lo = __builtin_amdgcn_readfirstlane(entry_lo(r_nxt));
-                n_hi = __builtin_amdgcn_readfirstlane(entry_hi(r_nxt));
-            }
-    #pragma unroll
-            for (int j = 0; j < NLOADS; ++j) issue_copy(j, hk * G, (e_lo >> 8) * 32, (e_hi >> 8) * 32, 0);
+            advance();
+            int n_lo = __builtin_amdgcn_readfirstlane(entry_lo(r_nxt)), n_hi = __builtin_amdgcn_readfirstlane(entry_hi(r_nxt));
             wait_async();
             __syncthreads();
             if (!v_negated) {  // K, V and the first tile have landed
@@ -409,23 +451,15 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
             for (int it = 0; it < total; ++it) {
                 const int cur = it & 1;
                 // pair after next: its list entries are requested now and picked up at the end of the iteration
-                int g_aft = g_nxt, r_aft = r_nxt;
-                advance(g_aft, r_aft);
-                const int ra = g_aft < G ? r_aft : 0;
-                const int a_lo = entry_lo(ra), a_hi = entry_hi(ra);
-                // past the last tile the copies simply fetch it again (into the buffer nobody reads any more)
-                const bool more = it + 1 < total;
-                const int h_next = hk * G + (more ? g_nxt : g_cur);
-                const int lo_next = ((more ? n_lo : e_lo) >> 8) * 32, hi_next = ((more ? n_hi : e_hi) >> 8) * 32;
+                const int r_aft = r_nxt + 1 == npairs ? 0 : r_nxt + 1;
+                const int a_lo = entry_lo(r_aft), a_hi = entry_hi(r_aft);
+                const TileSource next = tile_source(hb_nxt, (n_lo >> 8) * 32, (n_hi >> 8) * 32);
                 const int mine = st ? e_hi : e_lo;
-                tile_step(std::true_type{}, cur, (mine >> (2 * kg_lane)) & 3, hk * G + g_cur, (mine >> 8) * 32, h_next, lo_next,
-                          hi_next);
+                tile_step(std::true_type{}, cur, (mine >> (2 * kg_lane)) & 3, hk * G + g_cur, (mine >> 8) * 32, next);
                 g_cur = g_nxt;
-                r_cur = r_nxt;
-                g_nxt = g_aft;
-                r_nxt = r_aft;
                 e_lo = n_lo;
                 e_hi = n_hi;
+                advance();
                 n_lo = __builtin_amdgcn_readfirstlane(a_lo);
                 n_hi = __builtin_amdgcn_readfirstlane(a_hi);
                 wait_async();
@@ -457,7 +491,7 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
                 }
                 __syncthreads();
                 // the slice sits in LDS rows 0..31: row stream 0 computes it, row stream 1 has nothing to do
-                tile_step(std::false_type{}, 0, st ? 0 : (entry >> (2 * kg_lane)) & 3, h, row0, 0, 0, 0);
+                tile_step(std::false_type{}, 0, st ? 0 : (entry >> (2 * kg_lane)) & 3, h, row0, TileSource{});
             }
         }
         if (!LONG) break;
