@@ -265,10 +265,16 @@ __global__ __launch_bounds__(FWD_THREADS, D == 128 ? 2 : 3) void fwd_kernel(cons
         }
 
         // ---- online softmax (per-lane scalars) ----------------------------------------------
-        float mloc = fmaxf(s[0][0], s[1][0]);
+        // (four short chains instead of one long one: the wave issues in order and would sit out the latency of
+        // every link)
+        float mx[4];
 #pragma unroll
-        for (int i = 1; i < 16; ++i) mloc = fmaxf(fmaxf(mloc, s[0][i]), s[1][i]);
-        mloc = half_swap_max(mloc);
+        for (int c = 0; c < 4; ++c) {
+            mx[c] = fmaxf(s[0][4 * c], s[1][4 * c]);
+#pragma unroll
+            for (int i = 1; i < 4; ++i) mx[c] = fmaxf(fmaxf(mx[c], s[0][4 * c + i]), s[1][4 * c + i]);
+        }
+        float mloc = half_swap_max(fmaxf(fmaxf(mx[0], mx[1]), fmaxf(mx[2], mx[3])));
         if (__any(mloc > m_i + rescale_thr)) {  // wave-uniform; rare after the first tiles
             const float mnew = fmaxf(m_i, mloc);
             const float muse = (mnew == -INFINITY) ? 0.f : mnew;
