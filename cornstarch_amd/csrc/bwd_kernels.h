@@ -149,6 +149,21 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
         }
     };
     bool v_negated = false;
+    // Head dims up to 64 leave room for this wave's K and (negated) V operands of the S / dP phase in registers:
+    // they are the same for every tile, and the phase then reads half as much from LDS.
+    constexpr bool KV_REGS = D <= 64;
+    u32x4 kfrag[KV_REGS ? KK : 1], vfrag[KV_REGS ? KK : 1];
+    bool kv_loaded = false;
+    auto load_kv_operands = [&]() {  // after the V tile has been negated and a barrier has published it
+        if (KV_REGS && !kv_loaded) {
+#pragma unroll
+            for (int kk = 0; kk < KK; ++kk) {
+                kfrag[kk] = lds_read_chunk<D>(sK, 32 * kg + l32, 2 * kk + hi);
+                vfrag[kk] = lds_read_chunk<D>(sV, 32 * kg + l32, 2 * kk + hi);
+            }
+            kv_loaded = true;
+        }
+    };
 
     typedef SliceStage<D, DKDV_THREADS> Stage;
     constexpr int CPT = Stage::CPT;
@@ -260,7 +275,7 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
             constexpr int NOP = 2 * KK, AHEAD = 3;  // MFMA j: S (j even) or dP (j odd), k-slice j / 2
             u32x4 a[NOP], bb[NOP];
             a[0] = lds_read_chunk<D>(tQ, qr + l32, hi);  // the operands of the first MFMA go first
-            bb[0] = lds_read_chunk<D>(sK, 32 * kg + l32, hi);
+            bb[0] = KV_REGS ? kfrag[0] : lds_read_chunk<D>(sK, 32 * kg + l32, hi);
 #pragma unroll
             for (int grp = 0; grp < 4; ++grp) {
                 const f32x4 d4 = *(const f32x4*)&sDelta[cur][qr + 8 * grp + 4 * hi];
@@ -270,14 +285,16 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
 #pragma unroll
             for (int j = 1; j < AHEAD; ++j) {
                 a[j] = lds_read_chunk<D>((j & 1) ? tG : tQ, qr + l32, 2 * (j >> 1) + hi);
-                bb[j] = lds_read_chunk<D>((j & 1) ? sV : sK, 32 * kg + l32, 2 * (j >> 1) + hi);
+                bb[j] = KV_REGS ? ((j & 1) ? vfrag[j >> 1] : kfrag[j >> 1])
+                                : lds_read_chunk<D>((j & 1) ? sV : sK, 32 * kg + l32, 2 * (j >> 1) + hi);
             }
 #pragma unroll
             for (int j = 0; j < NOP; ++j) {
                 __builtin_amdgcn_sched_barrier(0);
                 if (j + AHEAD < NOP) {
                     a[j + AHEAD] = lds_read_chunk<D>(((j + AHEAD) & 1) ? tG : tQ, qr + l32, 2 * ((j + AHEAD) >> 1) + hi);
-                    bb[j + AHEAD] = lds_read_chunk<D>(((j + AHEAD) & 1) ? sV : sK, 32 * kg + l32, 2 * ((j + AHEAD) >> 1) + hi);
+                    bb[j + AHEAD] = KV_REGS ? (((j + AHEAD) & 1) ? vfrag[(j + AHEAD) >> 1] : kfrag[(j + AHEAD) >> 1])
+                                            : lds_read_chunk<D>(((j + AHEAD) & 1) ? sV : sK, 32 * kg + l32, 2 * ((j + AHEAD) >> 1) + hi);
                 }
                 if (j & 1)
                     dp = T::mfma(a[j], bb[j], dp);
@@ -448,6 +465,7 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
                 v_negated = true;
                 __syncthreads();
             }
+            load_kv_operands();
             for (int it = 0; it < total; ++it) {
                 const int cur = it & 1;
                 // pair after next: its list entries are requested now and picked up at the end of the iteration
@@ -490,6 +508,7 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
                     if (IDX) sQpos[0][tid] = ok ? p.posq[row0 + tid] : 0;
                 }
                 __syncthreads();
+                load_kv_operands();
                 // the slice sits in LDS rows 0..31: row stream 0 computes it, row stream 1 has nothing to do
                 tile_step(std::false_type{}, 0, st ? 0 : (entry >> (2 * kg_lane)) & 3, h, row0, TileSource{});
             }
