@@ -303,6 +303,30 @@ def test_irregular_bitfields_with_padding(S, D, Hq, Hkv, wide):
     check_against_oracle(q, k, v, do, bf)
 
 
+@pytest.mark.parametrize("S", [2, 3, 17, 31, 33, 65, 97])
+@pytest.mark.parametrize("D", [32, 64, 128])
+def test_very_short_sequences(S, D):
+    # one ragged slice, one slice and a ragged one, odd slice counts: the corner cases of the slice pairs of dK/dV
+    bf = random_bitfield(2, S, seed=S + D)
+    q, k, v, do = make_inputs(2, S, 4, 2, D, torch.bfloat16, seed=S)
+    check_against_oracle(q, k, v, do, bf)
+
+
+@pytest.mark.parametrize("D", [32, 64, 128])
+def test_single_token_sequence(D):
+    # a token that sees only itself: o = v, lse = scale * q.k, dv = do, and dq = dk = 0 up to the rounding of o
+    bf = torch.full((2, 1), (1 << 62) | 1 | 2, dtype=torch.int64)
+    q, k, v, do = make_inputs(2, 1, 4, 2, D, torch.bfloat16, seed=D)
+    o, lse, dq, dk, dv = run_hip(q, k, v, bf, do)
+    kv_of_head = torch.arange(4) // 2
+    assert torch.equal(o.cpu(), v[:, :, kv_of_head])
+    want_lse = (q.float() * k.float()[:, :, kv_of_head]).sum(-1).transpose(1, 2) / math.sqrt(D)
+    assert (lse[:, :, :1].cpu() - want_lse).abs().max().item() <= 1e-2
+    want_dv = do.float().view(2, 1, 2, 2, D).sum(3)
+    assert (dv.float().cpu() - want_dv).abs().max().item() <= 4e-2
+    assert dq.float().abs().max().item() <= 1e-2 and dk.float().abs().max().item() <= 1e-2
+
+
 def test_all_text_bitfield_is_causal_attention():
     # tests/test_shardformer/utils.py:388-391
     S = 300
