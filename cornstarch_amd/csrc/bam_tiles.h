@@ -39,6 +39,12 @@ __device__ __forceinline__ void dma_b32(const void* sbase, unsigned voff, unsign
 // All direct global-to-LDS copies this wave has issued have landed (pair with a barrier).
 __device__ __forceinline__ void wait_async() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
+// All LDS accesses this wave has issued are complete.  The compiler puts this wait in front of a barrier by itself --
+// except, as the generated code showed, in front of a barrier at the head of a loop that is reached over the back
+// edge with LDS stores still in flight (the list rebuilt for the next pass over a long sequence: other waves then
+// read the old count or old entries).  So whoever writes LDS ahead of such a barrier states the wait.
+__device__ __forceinline__ void wait_lds() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+
 // ROWS x D tile of 2-byte elements copied global -> LDS by THREADS threads, 16 bytes per lane.
 // Full tiles use the direct global-to-LDS load (no staging registers, no LDS write
 // instructions): a wave's 64 lanes fill 64 consecutive chunk slots of the LDS tile, so the
@@ -223,6 +229,7 @@ __device__ __forceinline__ void build_key_tile_list(const WaveSlices& ws, int nu
         count += __popcll(bal);
     }
     if (lane == 0) *count_out = count;
+    wait_lds();
 }
 
 // List, in ascending order, the 32-row slices among [s_begin, s_end) (at most MAX_SLICE_LIST of them; longer
@@ -257,6 +264,7 @@ __device__ __forceinline__ void build_slice_list(const AttnParams& p, int b, int
         *count_out = count;
         if (count > 0) list[-1] = list[0] & ~0xFF;
     }
+    wait_lds();
 }
 
 }  // namespace bam
