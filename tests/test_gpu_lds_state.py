@@ -33,6 +33,7 @@ def _long_layout(S):
     [
         (131072 + 4096 + 57, 32, 2, 1, "long", 40),  # two passes in all three attention kernels, ragged
         (131072 + 4096 + 57, 128, 2, 1, "long", 8),
+        (2 * 131072 + 4096 + 57, 32, 2, 1, "long", 6),  # three passes
         (131072, 64, 2, 1, "long", 4),               # the longest single-pass sequence, with a plan
         (2000 + 57, 128, 4, 2, "random", 6),
         (517, 64, 4, 4, "random", 6),
