@@ -305,10 +305,11 @@ def main():
             "dkdv": round(r["issued"]["dkdv"] / (8 * w.D * w.Hq * pairs), 4),
             "dq": round(r["issued"]["dq"] / (6 * w.D * w.Hq * pairs), 4),
         },
-        # what the measurements say holds the dominant kernel back: no single saturated unit -- MFMA pipe 40-53 %
-        # busy, 29-35 % of wave time at s_waitcnt / barriers, 4-5 other vector instructions per MFMA
-        # (profiles/bam_kernels_C2_counters.txt)
-        "limiter": "latency / instruction mix, not a saturated unit",
+        # what the measurements say holds the dominant kernel back: no single saturated unit -- MFMA pipe 43-54 %
+        # busy, ~30 % of wave time at s_waitcnt / barriers, 4-5 other vector instructions per MFMA
+        # (profiles/bam_kernels_C2_counters.txt); in dK/dV the LDS operand traffic (1.5 KB per MFMA against 256 B
+        # per clock and compute unit) would saturate at ~1.3x the present MFMA rate
+        "limiter": "latency / instruction mix; dK/dV within 1.3x of its LDS operand bandwidth",
         "roofline": {
             "kernel": kname[dom],
             "bound": "mfma",
