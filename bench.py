@@ -307,9 +307,9 @@ def main():
         },
         # what the measurements say holds the dominant kernel back: no single saturated unit -- MFMA pipe 43-54 %
         # busy, ~30 % of wave time at s_waitcnt / barriers, 4-5 other vector instructions per MFMA
-        # (profiles/bam_kernels_C2_counters.txt); in dK/dV the LDS operand traffic (1.5 KB per MFMA against 256 B
-        # per clock and compute unit) would saturate at ~1.3x the present MFMA rate
-        "limiter": "latency / instruction mix; dK/dV within 1.3x of its LDS operand bandwidth",
+        # (profiles/bam_kernels_C2_counters.txt); dK/dV reads 1.5 KB of LDS operands per MFMA (2 KB in its S / dP
+        # phase): at the MFMA peak that is 75 % (100 %) of the 256 B per clock a compute unit's LDS delivers
+        "limiter": "latency / instruction mix, not a saturated unit (dK/dV: LDS operand traffic = 75 % of LDS peak at MFMA peak)",
         "roofline": {
             "kernel": kname[dom],
             "bound": "mfma",
