@@ -39,11 +39,16 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(lib, n), f"{n} is declared in include/bam_hip.h but not exported"
     assert _bam_hip.load().bam_abi_version() == _bam_hip.ABI_VERSION
     # the binding's prototypes cover every compute entry point of the header
-    assert set(_bam_hip.SIGNATURES) == set(names) - {"bam_last_error", "bam_abi_version", "bam_plan_workspace_bytes"}
+    assert set(_bam_hip.SIGNATURES) == set(names) - {
+        "bam_last_error", "bam_abi_version", "bam_plan_workspace_bytes", "bam_plan_workspace_bytes_rect"}
     # plan workspace: sized without a GPU; no plan beyond 4096 row slices
     lib2 = _bam_hip.load()
     assert lib2.bam_plan_workspace_bytes(1, 8192) >= 256 * 256 + 256 * 4 and lib2.bam_plan_workspace_bytes(1, 8192) % 256 == 0
     assert lib2.bam_plan_workspace_bytes(2, 131072) > 0 and lib2.bam_plan_workspace_bytes(1, 131073) == 0
+    # rectangular problems (context-parallel shards, materialized masks): rows bound the plan, keys only size it
+    assert lib2.bam_plan_workspace_bytes_rect(1, 8192, 8192) == lib2.bam_plan_workspace_bytes(1, 8192)
+    assert lib2.bam_plan_workspace_bytes_rect(1, 4096, 8192) >= 128 * 256 + 128 * 4
+    assert lib2.bam_plan_workspace_bytes_rect(1, 131073, 64) == 0 and lib2.bam_plan_workspace_bytes_rect(1, 64, 262144) > 0
 
 
 def test_abi_rejects_bad_arguments_without_touching_the_gpu():
@@ -130,19 +135,102 @@ def test_adapter_requires_int64_mask():
     q = torch.randn(1, 2, 8, 32)
     with pytest.raises(AssertionError, match="int64"):
         interface.bitfield_attention_forward(M(), q, q, q, torch.ones(1, 8, dtype=torch.bool))
-    # single-token decode of an eval-mode module never reaches the bitfield kernel
+    # the single-token decode step of an eval-mode module never looks at the mask, and like the rest of the
+    # product path it has no CPU fallback
     m = M().eval()
-    q1 = torch.randn(1, 4, 1, 32)
-    kv = torch.randn(1, 2, 9, 32)
-    out, w = interface.bitfield_attention_forward(m, q1, kv, kv, None)
-    assert out.shape == (1, 1, 4, 32) and w is None
-    want = torch.softmax(
-        (q1 @ kv.repeat_interleave(2, 1).transpose(-1, -2)) / 32**0.5, -1) @ kv.repeat_interleave(2, 1)
-    assert torch.allclose(out, want.transpose(1, 2), atol=1e-5)
-    # a window or a logit cap would change the decode logits: refused, not dropped
-    for kw in ({"sliding_window": 4}, {"softcap": 30.0}):
-        with pytest.raises(NotImplementedError):
-            interface.bitfield_attention_forward(m, q1, kv, kv, None, **kw)
+    q1 = torch.randn(1, 4, 1, 32, dtype=torch.bfloat16)
+    kv = torch.randn(1, 2, 9, 32, dtype=torch.bfloat16)
+    with pytest.raises(AssertionError, match="GPU only"):
+        interface.bitfield_attention_forward(m, q1, kv, kv, None)
+
+
+def test_decode_entry_rejects_bad_arguments_without_touching_the_gpu():
+    lib = _bam_hip.load()
+    P = ctypes.c_void_p
+    good = [P(16)] * 4 + [8] * 10 + [1, 64, 4, 2, 64] + [0.125, 1, 0, 0.0, None]
+    bad_window = list(good)
+    bad_window[21] = -3
+    assert lib.bam_decode(*bad_window) == -1 and b"window" in lib.bam_last_error()
+    bad_cap = list(good)
+    bad_cap[22] = -1.0
+    assert lib.bam_decode(*bad_cap) == -1 and b"softcap" in lib.bam_last_error()
+    bad_heads = list(good)
+    bad_heads[16:18] = [4, 3]
+    assert lib.bam_decode(*bad_heads) == -1 and b"multiple of Hkv" in lib.bam_last_error()
+    assert lib.bam_decode(*([None] + good[1:])) == -1 and b"null" in lib.bam_last_error()
+
+
+# The import statements of the reference's callers, verbatim (file:line of /root/reference/cornstarch/...).
+REFERENCE_IMPORT_LINES = [
+    # shardformer/layers/utils.py:11-12
+    "from cornstarch.kernel.attention import BLOCK_M, BLOCK_N",
+    "from cornstarch.kernel.bitfield_attention import BitfieldUtils",
+    # shardformer/layers/context_parallel_bitfield_attention.py:7-10
+    "from cornstarch.kernel.bitfield_attention import (\n    _bitfield_attn_backward,\n    _bitfield_attn_forward,\n)",
+    # shardformer/modeling/llama.py:31 (and gemma, gemma2, gemma3, llama4, mistral, mixtral, phi3, qwen2, qwen3, qwen3_moe)
+    "from cornstarch.kernel.bitfield_attention import BitfieldUtils",
+    # models/multimodal_language_model/modeling_multimodal_language_model.py:37
+    "from cornstarch.kernel.interface import bitfield_attention_forward",
+    # kernel/interface.py:9-10
+    "from cornstarch.kernel.attention import flash_attn_func",
+    "from cornstarch.kernel.bitfield_attention import bitfield_attn_func",
+    # tests/test_kernel/test_attention.py:5-7, tests/test_shardformer/test_context_parallel.py:16,
+    # tests/test_shardformer/utils.py:42-45
+    "from cornstarch.kernel.attention import (\n    flash_attn_func as my_flash_attn_func_triton,\n)",
+    "from cornstarch.kernel.bitfield_attention import BitfieldUtils, bitfield_attn_func",
+    "from cornstarch.kernel.interface import (\n    bitfield_attention_forward,\n    create_bitfield_attention_mask,\n)",
+]
+
+
+@pytest.mark.parametrize("line", REFERENCE_IMPORT_LINES)
+def test_import_statements_of_the_reference_callers_resolve_here(line):
+    ns = {}
+    exec(line, ns)
+    impl = {"BitfieldUtils": BA.BitfieldUtils, "_bitfield_attn_forward": BA._bitfield_attn_forward,
+            "_bitfield_attn_backward": BA._bitfield_attn_backward, "bitfield_attn_func": BA.bitfield_attn_func,
+            "flash_attn_func": sibling.flash_attn_func, "my_flash_attn_func_triton": sibling.flash_attn_func,
+            "bitfield_attention_forward": interface.bitfield_attention_forward,
+            "create_bitfield_attention_mask": interface.create_bitfield_attention_mask,
+            "BLOCK_M": 128, "BLOCK_N": 32}
+    got = {k: v for k, v in ns.items() if k != "__builtins__"}
+    assert got and all(got[k] is impl[k] or got[k] == impl[k] for k in got)
+
+
+def test_cornstarch_kernel_modules_are_the_implementation_modules():
+    import importlib
+
+    for name, impl in (("bitfield_attention", BA), ("attention", sibling), ("interface", interface)):
+        assert importlib.import_module(f"cornstarch.kernel.{name}") is impl
+    # the registration the reference performs at import time
+    # (models/multimodal_language_model/modeling_multimodal_language_model.py:42) works through either name
+    from transformers.modeling_utils import ALL_ATTENTION_FUNCTIONS
+
+    from cornstarch.kernel.interface import bitfield_attention_forward
+
+    ALL_ATTENTION_FUNCTIONS.update({"bitfield_attention": bitfield_attention_forward})
+    assert ALL_ATTENTION_FUNCTIONS["bitfield_attention"] is interface.bitfield_attention_forward
+
+
+def test_cornstarch_package_leaves_other_subpackages_to_a_checkout_further_down_the_path(tmp_path):
+    # a stand-in for a Cornstarch checkout: a `cornstarch` package with a subpackage of its own and a kernel
+    # package that must NOT win
+    import subprocess
+    import sys
+
+    pkg = tmp_path / "site" / "cornstarch"
+    (pkg / "shardformer").mkdir(parents=True)
+    (pkg / "kernel").mkdir()
+    (pkg / "__init__.py").write_text("")
+    (pkg / "shardformer" / "__init__.py").write_text("from cornstarch.kernel.bitfield_attention import BitfieldUtils\n")
+    (pkg / "kernel" / "__init__.py").write_text("")
+    (pkg / "kernel" / "bitfield_attention.py").write_text("BitfieldUtils = 'theirs'\n")
+    code = (
+        "import sys; sys.path[:0] = [%r, %r]\n"
+        "import cornstarch.shardformer as s, cornstarch_amd.kernel.bitfield_attention as ours\n"
+        "assert s.__file__.startswith(%r), s.__file__\n"
+        "assert s.BitfieldUtils is ours.BitfieldUtils\n"
+    ) % (ROOT, str(tmp_path / "site"), str(tmp_path))
+    subprocess.run([sys.executable, "-c", code], check=True)
 
 
 # histogram / pair counts of the synthetic workloads quoted by the baseline document
