@@ -353,3 +353,28 @@ def sdpa_forward_backward(q, k, v, bitfield, do=None, softmax_scale=None, row_ch
                 grads[1][b] += gk.transpose(1, 2)[0]
                 grads[2][b] += gv.transpose(1, 2)[0]
     return (o, *grads) if grads is not None else o
+
+
+def decode_step(query, key, value, scaling=None, sliding_window=None, softcap=None):
+    """Single-token decode step of the HF adapter (cornstarch/kernel/interface.py:71-83): the reference forwards it
+    to flash-attn through transformers' ``flash_attention_forward`` with ``attention_mask=None``.  flash-attn is not
+    part of the reference tree; its published semantics for ONE query at the last position are restated here in
+    fp32: scores ``scaling * q.k`` (default 1/sqrt(D)); ``softcap``: ``softcap * tanh(score / softcap)``;
+    ``sliding_window`` w (transformers passes ``window_size=(w - 1, w - 1)`` when the cache is longer than w):
+    keys ``j >= Sk - w``; softmax; times V.  Grouped kv heads: kv head of q head h is ``h // (Hq // Hkv)``.
+
+    query (B, Hq, 1, D), key / value (B, Hkv, Sk, D) -> (B, 1, Hq, D) fp32."""
+    B, Hq, one, D = query.shape
+    Hkv, Sk = key.shape[1], key.shape[2]
+    g = Hq // Hkv
+    qf = query.float()[:, :, 0]                              # (B, Hq, D)
+    kf = key.float().repeat_interleave(g, dim=1)             # (B, Hq, Sk, D)
+    vf = value.float().repeat_interleave(g, dim=1)
+    scale = scaling if scaling is not None else 1.0 / math.sqrt(D)
+    s = torch.einsum("bhd,bhjd->bhj", qf, kf) * scale
+    if softcap:
+        s = softcap * torch.tanh(s / softcap)
+    if sliding_window is not None and Sk > sliding_window:
+        s[:, :, : Sk - sliding_window] = -math.inf
+    p = torch.softmax(s, dim=-1)
+    return torch.einsum("bhj,bhjd->bhd", p, vf)[:, None]

@@ -396,3 +396,74 @@ def test_bias_closed_forms():
     ww = allow[None] * w[0, :, 0][:, None, :]  # (H, S, S)
     want = torch.einsum("hij,jhd->ihd", ww / ww.sum(-1, keepdim=True), v[0])
     assert torch.allclose(o2[0], want, atol=1e-12, rtol=0)
+
+
+# ------------------------------------------------------------------ the routine the CPU baseline times
+@pytest.mark.parametrize("row_chunk", [128, 77, 4096])
+def test_chunked_sdpa_routine_matches_the_attention_oracle(row_chunk):
+    # grouped kv heads, padding rows (bitfield 0) and a chunk that does not divide the sequence
+    B, S, Hq, Hkv, D = 2, 300, 4, 2, 32
+    g = torch.Generator().manual_seed(11)
+    q = torch.randn(B, S, Hq, D, generator=g)
+    k = torch.randn(B, S, Hkv, D, generator=g)
+    v = torch.randn(B, S, Hkv, D, generator=g)
+    do = torch.randn(B, S, Hq, D, generator=g)
+    bf = random_bitfield(B, S, seed=5, pad=9)
+    o, dq, dk, dv = O.sdpa_forward_backward(q, k, v, bf, do, row_chunk=row_chunk)
+    o_ref, _ = O.attention_forward(q, k, v, bf)
+    assert (o - o_ref).abs().max().item() <= 1e-5
+    assert torch.equal(O.sdpa_forward_backward(q, k, v, bf, row_chunk=row_chunk), o)  # forward-only form
+    for got, want in zip((dq, dk, dv), O.attention_backward(q, k, v, bf, do)):
+        assert rel_l2(got, want) <= 1e-5
+    # padding rows: zero output, zero gradient, finite everywhere
+    assert (o[:, S - 9 :] == 0).all() and (dq[:, S - 9 :] == 0).all()
+    assert all(torch.isfinite(t).all() for t in (o, dq, dk, dv))
+
+
+# ------------------------------------------------------------------ single-token decode step
+def _decode_inputs(B=2, Hq=4, Hkv=2, Sk=37, D=16, seed=3):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(B, Hq, 1, D, generator=g), torch.randn(B, Hkv, Sk, D, generator=g),
+            torch.randn(B, Hkv, Sk, D, generator=g))
+
+
+def test_decode_step_plain_is_library_sdpa():
+    q, k, v = _decode_inputs()
+    want = F.scaled_dot_product_attention(q, k, v, enable_gqa=True).transpose(1, 2)
+    assert torch.allclose(O.decode_step(q, k, v), want, atol=1e-6)
+    want = F.scaled_dot_product_attention(q, k, v, enable_gqa=True, scale=0.3).transpose(1, 2)
+    assert torch.allclose(O.decode_step(q, k, v, scaling=0.3), want, atol=1e-6)
+
+
+def test_decode_step_window_and_softcap_closed_forms():
+    q, k, v = _decode_inputs()
+    Sk = k.shape[2]
+    plain = O.decode_step(q, k, v)
+    # a window at least as long as the cache, or a cap far above every score, changes nothing
+    assert torch.equal(O.decode_step(q, k, v, sliding_window=Sk), plain)
+    assert torch.equal(O.decode_step(q, k, v, sliding_window=Sk + 5), plain)
+    assert torch.allclose(O.decode_step(q, k, v, softcap=1e6), plain, atol=1e-5)
+    # a window of w keys == attention over the last w keys of the cache
+    for w in (1, 5, Sk - 1):
+        want = F.scaled_dot_product_attention(q, k[:, :, Sk - w :], v[:, :, Sk - w :], enable_gqa=True).transpose(1, 2)
+        assert torch.allclose(O.decode_step(q, k, v, sliding_window=w), want, atol=1e-6)
+    assert torch.allclose(O.decode_step(q, k, v, sliding_window=1)[:, 0], v[:, :, -1].repeat_interleave(2, 1), atol=1e-6)
+    # a tiny cap flattens the scores: softmax of (almost) equal logits is the mean of V
+    mean_v = v.mean(dim=2).repeat_interleave(2, 1)
+    assert torch.allclose(O.decode_step(q, k, v, softcap=1e-4)[:, 0], mean_v, atol=1e-3)
+
+
+def test_decode_step_brute_force_with_both():
+    q, k, v = _decode_inputs(B=1, Hq=2, Hkv=1, Sk=9, D=4, seed=8)
+    cap, w, scale = 0.7, 4, 0.9
+    got = O.decode_step(q, k, v, scaling=scale, sliding_window=w, softcap=cap)
+    for h in range(2):
+        logits = []
+        for j in range(9 - w, 9):
+            s = scale * sum(float(q[0, h, 0, d]) * float(k[0, 0, j, d]) for d in range(4))
+            logits.append(cap * math.tanh(s / cap))
+        mx = max(logits)
+        e = [math.exp(x - mx) for x in logits]
+        for d in range(4):
+            want = sum(e[i] * float(v[0, 0, 9 - w + i, d]) for i in range(w)) / sum(e)
+            assert abs(float(got[0, 0, h, d]) - want) <= 1e-5
