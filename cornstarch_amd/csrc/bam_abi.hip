@@ -16,6 +16,9 @@ namespace {
 
 constexpr int kMaxDevices = 64;
 void* g_static_plan_ptr[kMaxDevices] = {};  // per device, resolved on first use
+// Every bam_tile_plan_static call on a device starts a new generation of that device's array; the plan it returns
+// carries the number, and a plan of an older generation (its arrays have been overwritten since) is refused.
+int32_t g_static_plan_generation[kMaxDevices] = {};
 
 thread_local char g_error[512] = "";
 
@@ -126,13 +129,21 @@ int fill_bias(bam::AttnParams& p, const char* who, const bam_bias* bias, int Sk)
     return BAM_OK;
 }
 
-// plan may be null.  It must have been built for this very (B, S).
-int fill_plan(bam::AttnParams& p, const char* who, const bam_plan* plan, int B, int S) {
+// plan may be null.  It must have been built for this very (B, Sq, Sk).
+int fill_plan(bam::AttnParams& p, const char* who, const bam_plan* plan, int B, int Sq, int Sk) {
     if (plan == nullptr) return BAM_OK;  // p.fine stays null
     if (plan->fine == nullptr || plan->order == nullptr) return fail(BAM_ERR_INVALID_ARGUMENT, "%s: plan: null array", who);
-    if (plan->B != B || plan->S != S)
-        return fail(BAM_ERR_INVALID_ARGUMENT, "%s: plan was built for B = %d, S = %d, not B = %d, S = %d", who, plan->B,
-                    plan->S, B, S);
+    if (plan->B != B || plan->Sq != Sq || plan->Sk != Sk)
+        return fail(BAM_ERR_INVALID_ARGUMENT, "%s: plan was built for B = %d, Sq = %d, Sk = %d, not B = %d, Sq = %d, Sk = %d",
+                    who, plan->B, plan->Sq, plan->Sk, B, Sq, Sk);
+    if (plan->generation != 0) {  // laid out in the built-in array of bam_tile_plan_static
+        int dev = -1;
+        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices ||
+            plan->fine != (const uint8_t*)g_static_plan_ptr[dev] || plan->generation != g_static_plan_generation[dev])
+            return fail(BAM_ERR_INVALID_ARGUMENT,
+                        "%s: plan of bam_tile_plan_static is stale (a later call on this GPU has reused the built-in array)",
+                        who);
+    }
     if (reinterpret_cast<uintptr_t>(plan->order) & 3u) return fail(BAM_ERR_INVALID_ARGUMENT, "%s: plan: misaligned order", who);
     p.fine = plan->fine;
     p.fine_sb = plan->fine_stride_b;
@@ -204,7 +215,7 @@ int fwd_impl(const char* who, const void* q, const void* k, const void* v, void*
     p.flags_sm = flags_stride_m;
     fill_sizes(p, m, B, Hq, Hkv, D, scale);
     BAM_TRY(fill_bias(p, who, bias, m.Sk));
-    BAM_TRY(fill_plan(p, who, plan, B, m.Sq));
+    BAM_TRY(fill_plan(p, who, plan, B, m.Sq, m.Sk));
     return launched(bam::launch_fwd(p, dtype, (hipStream_t)stream), who);
 }
 
@@ -249,7 +260,7 @@ int bwd_params(bam::AttnParams& p, const char* who, const void* q, const void* k
     p.flags_sb = st[21];
     p.flags_sm = st[22];
     fill_sizes(p, m, B, Hq, Hkv, D, scale);
-    BAM_TRY(fill_plan(p, who, plan, B, m.Sq));
+    BAM_TRY(fill_plan(p, who, plan, B, m.Sq, m.Sk));
     return fill_bias(p, who, bias, m.Sk);
 }
 
@@ -259,7 +270,7 @@ extern "C" {
 
 const char* bam_last_error(void) { return g_error; }
 
-int bam_abi_version(void) { return 6; }
+int bam_abi_version(void) { return 7; }
 
 int bam_tile_flags(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int64_t flags_stride_b,
                    int64_t flags_stride_m, int B, int S, void* stream) {
@@ -277,8 +288,8 @@ namespace {
 struct PlanLayout {
     int64_t fine_ss, fine_sb, order_sb, fine_off, order_off, bytes;
 };
-PlanLayout plan_layout(int B, int S) {
-    const int64_t num_m = (S + 127) / 128, num_n = (S + 31) / 32, slots = 4 * num_m;
+PlanLayout plan_layout(int B, int Sq, int Sk) {
+    const int64_t num_m = (Sq + 127) / 128, num_n = (Sk + 31) / 32, slots = 4 * num_m;
     auto up = [](int64_t x, int64_t a) { return (x + a - 1) / a * a; };
     PlanLayout l;
     l.fine_ss = up(num_n, 16);
@@ -291,10 +302,39 @@ PlanLayout plan_layout(int B, int S) {
 }
 }  // namespace
 
-int64_t bam_plan_workspace_bytes(int B, int S) {
-    if (B <= 0 || S <= 0 || (S + 31) / 32 > bam::MAX_PLAN_SLICES) return 0;
-    return plan_layout(B, S).bytes;
+int64_t bam_plan_workspace_bytes_rect(int B, int Sq, int Sk) {
+    if (B <= 0 || Sq <= 0 || Sk <= 0 || (Sq + 31) / 32 > bam::MAX_PLAN_SLICES || Sk > BAM_MAX_SEQLEN) return 0;
+    return plan_layout(B, Sq, Sk).bytes;
 }
+
+int64_t bam_plan_workspace_bytes(int B, int S) { return bam_plan_workspace_bytes_rect(B, S, S); }
+
+namespace {
+// Checks the workspace and lays the plan's arrays out in it.
+int place_plan(const char* who, void* workspace, int64_t workspace_bytes, int B, int Sq, int Sk, bam_plan* plan,
+               PlanLayout& l) {
+    if (workspace == nullptr || plan == nullptr) return fail(BAM_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
+    const int64_t need = bam_plan_workspace_bytes_rect(B, Sq, Sk);
+    if (need == 0) return fail(BAM_ERR_UNSUPPORTED, "%s: no plan is built for Sq = %d, Sk = %d", who, Sq, Sk);
+    if (workspace_bytes < need)
+        return fail(BAM_ERR_INVALID_ARGUMENT, "%s: workspace of %lld bytes, %lld needed", who, (long long)workspace_bytes,
+                    (long long)need);
+    if (reinterpret_cast<uintptr_t>(workspace) & 255u)
+        return fail(BAM_ERR_INVALID_ARGUMENT, "%s: workspace is not 256-byte aligned", who);
+    l = plan_layout(B, Sq, Sk);
+    char* w = (char*)workspace;
+    plan->fine = (const uint8_t*)(w + l.fine_off);
+    plan->fine_stride_b = l.fine_sb;
+    plan->fine_stride_s = l.fine_ss;
+    plan->order = (const int32_t*)(w + l.order_off);
+    plan->order_stride_b = l.order_sb;
+    plan->B = B;
+    plan->Sq = Sq;
+    plan->Sk = Sk;
+    plan->generation = 0;
+    return BAM_OK;
+}
+}  // namespace
 
 int bam_tile_plan(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int64_t flags_stride_b,
                   int64_t flags_stride_m, void* workspace, int64_t workspace_bytes, int B, int S, bam_plan* plan,
@@ -304,22 +344,9 @@ int bam_tile_plan(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int64_t
     if (B <= 0 || S <= 0) return fail(BAM_ERR_INVALID_ARGUMENT, "bam_tile_plan: B and S must be positive");
     if (B > 65535 || (S + 127) / 128 > 65535)
         return fail(BAM_ERR_UNSUPPORTED, "bam_tile_plan: grid too large (B = %d, S = %d)", B, S);
-    const int64_t need = bam_plan_workspace_bytes(B, S);
-    if (need == 0) return fail(BAM_ERR_UNSUPPORTED, "bam_tile_plan: no plan is built for S = %d (use bam_tile_flags)", S);
-    if (workspace_bytes < need)
-        return fail(BAM_ERR_INVALID_ARGUMENT, "bam_tile_plan: workspace of %lld bytes, %lld needed", (long long)workspace_bytes,
-                    (long long)need);
-    if (reinterpret_cast<uintptr_t>(workspace) & 255u)
-        return fail(BAM_ERR_INVALID_ARGUMENT, "bam_tile_plan: workspace is not 256-byte aligned");
-    const PlanLayout l = plan_layout(B, S);
+    PlanLayout l;
+    BAM_TRY(place_plan("bam_tile_plan", workspace, workspace_bytes, B, S, S, plan, l));
     char* w = (char*)workspace;
-    plan->fine = (const uint8_t*)(w + l.fine_off);
-    plan->fine_stride_b = l.fine_sb;
-    plan->fine_stride_s = l.fine_ss;
-    plan->order = (const int32_t*)(w + l.order_off);
-    plan->order_stride_b = l.order_sb;
-    plan->B = B;
-    plan->S = S;
     return launched(bam::launch_tile_plan(bf, bf_stride_b, flags, flags_stride_b, flags_stride_m, (uint8_t*)(w + l.fine_off),
                                           l.fine_sb, l.fine_ss, (int*)(w + l.order_off), l.order_sb, B, S,
                                           (hipStream_t)stream),
@@ -346,8 +373,41 @@ int bam_tile_plan_static(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, 
             return fail(BAM_ERR_LAUNCH, "bam_tile_plan_static: hipGetSymbolAddress failed: %s", hipGetErrorString(e));
         g_static_plan_ptr[dev] = ptr;
     }
-    return bam_tile_plan(bf, bf_stride_b, flags, flags_stride_b, flags_stride_m, g_static_plan_ptr[dev],
-                         BAM_STATIC_PLAN_BYTES, B, S, plan, stream);
+    BAM_TRY(bam_tile_plan(bf, bf_stride_b, flags, flags_stride_b, flags_stride_m, g_static_plan_ptr[dev],
+                          BAM_STATIC_PLAN_BYTES, B, S, plan, stream));
+    if (++g_static_plan_generation[dev] <= 0) g_static_plan_generation[dev] = 1;
+    plan->generation = g_static_plan_generation[dev];
+    return BAM_OK;
+}
+
+int bam_plan_indexed(const bam_index_view* iv, void* workspace, int64_t workspace_bytes, int B, bam_plan* plan,
+                     void* stream) {
+    MaskSource m;
+    BAM_TRY(indexed_source(iv, m));
+    if (B <= 0 || m.Sq <= 0 || m.Sk <= 0) return fail(BAM_ERR_INVALID_ARGUMENT, "bam_plan_indexed: B, Sq and Sk must be positive");
+    if (B > 65535) return fail(BAM_ERR_UNSUPPORTED, "bam_plan_indexed: B is limited to 65535 (got %d)", B);
+    PlanLayout l;
+    BAM_TRY(place_plan("bam_plan_indexed", workspace, workspace_bytes, B, m.Sq, m.Sk, plan, l));
+    char* w = (char*)workspace;
+    return launched(bam::launch_indexed_plan(m.bfq, m.bfq_sb, m.bfk, m.bfk_sb, m.posq, m.posk, m.Sq, m.Sk,
+                                             (uint8_t*)(w + l.fine_off), l.fine_sb, l.fine_ss, (int*)(w + l.order_off),
+                                             l.order_sb, B, (hipStream_t)stream),
+                    "bam_plan_indexed");
+}
+
+int bam_mask_tile_plan(const uint8_t* mask, int8_t* flags, int64_t flags_stride_b, int64_t flags_stride_m, void* workspace,
+                       int64_t workspace_bytes, int B, int Sq, int Sk, bam_plan* plan, void* stream) {
+    if (mask == nullptr || flags == nullptr) return fail(BAM_ERR_INVALID_ARGUMENT, "bam_mask_tile_plan: null pointer");
+    if (B <= 0 || Sq <= 0 || Sk <= 0) return fail(BAM_ERR_INVALID_ARGUMENT, "bam_mask_tile_plan: B, Sq and Sk must be positive");
+    if (B > 65535 || (Sq + 127) / 128 > 65535)
+        return fail(BAM_ERR_UNSUPPORTED, "bam_mask_tile_plan: grid too large (B = %d, Sq = %d)", B, Sq);
+    PlanLayout l;
+    BAM_TRY(place_plan("bam_mask_tile_plan", workspace, workspace_bytes, B, Sq, Sk, plan, l));
+    char* w = (char*)workspace;
+    return launched(bam::launch_mask_tile_plan(mask, flags, flags_stride_b, flags_stride_m, (uint8_t*)(w + l.fine_off),
+                                               l.fine_sb, l.fine_ss, (int*)(w + l.order_off), l.order_sb, B, Sq, Sk,
+                                               (hipStream_t)stream),
+                    "bam_mask_tile_plan");
 }
 
 int bam_materialize_mask(const int64_t* bf, int64_t bf_stride_b, uint8_t* out, int B, int S, void* stream) {
@@ -401,12 +461,13 @@ int bam_fwd_indexed(const void* q, const void* k, const void* v, void* o, float*
                     int64_t k_stride_b, int64_t k_stride_s, int64_t k_stride_h, int64_t v_stride_b,
                     int64_t v_stride_s, int64_t v_stride_h, int64_t o_stride_b, int64_t o_stride_s,
                     int64_t o_stride_h, int64_t flags_stride_b, int64_t flags_stride_m, int B, int Hq, int Hkv,
-                    int D, float scale, int dtype, const bam_bias* bias, void* stream) {
+                    int D, float scale, int dtype, const bam_bias* bias, const bam_plan* plan,
+        void* stream) {
     MaskSource m;
     BAM_TRY(indexed_source(iv, m));
     const int64_t st[12] = BAM_FWD_STRIDES;
     return fwd_impl("bam_fwd_indexed", q, k, v, o, lse, m, flags, st, flags_stride_b, flags_stride_m, B, Hq, Hkv, D,
-                    scale, dtype, bias, nullptr, stream);
+                    scale, dtype, bias, plan, stream);
 }
 
 int bam_bwd_preprocess(const void* o, const void* dout, float* delta, int64_t o_stride_b, int64_t o_stride_s,
@@ -489,7 +550,8 @@ int bam_bwd_dkdv_indexed(const void* q, const void* k, const void* v, const void
                          int64_t v_stride_h, int64_t do_stride_b, int64_t do_stride_s, int64_t do_stride_h,
                          int64_t dk_stride_b, int64_t dk_stride_s, int64_t dk_stride_h, int64_t dv_stride_b,
                          int64_t dv_stride_s, int64_t dv_stride_h, int64_t flags_stride_b, int64_t flags_stride_m,
-                         int B, int Hq, int Hkv, int D, float scale, int dtype, int accumulate, const bam_bias* bias, void* stream) {
+                         int B, int Hq, int Hkv, int D, float scale, int dtype, int accumulate, const bam_bias* bias, const bam_plan* plan,
+        void* stream) {
     MaskSource m;
     BAM_TRY(indexed_source(iv, m));
     void* dq = nullptr;
@@ -497,7 +559,7 @@ int bam_bwd_dkdv_indexed(const void* q, const void* k, const void* v, const void
     const int64_t st[23] = BAM_BWD_STRIDES;
     bam::AttnParams p = {};
     BAM_TRY(bwd_params(p, "bam_bwd_dkdv_indexed", q, k, v, dout, lse, delta, dq, dk, dv, m, flags, st, B, Hq, Hkv, D, scale,
-                       dtype, accumulate, false, true, bias, nullptr));
+                       dtype, accumulate, false, true, bias, plan));
     return launched(bam::launch_bwd_dkdv(p, dtype, (hipStream_t)stream), "bam_bwd_dkdv_indexed");
 }
 
@@ -508,7 +570,8 @@ int bam_bwd_dq_indexed(const void* q, const void* k, const void* v, const void* 
                        int64_t v_stride_h, int64_t do_stride_b, int64_t do_stride_s, int64_t do_stride_h,
                        int64_t dq_stride_b, int64_t dq_stride_s, int64_t dq_stride_h, int64_t flags_stride_b,
                        int64_t flags_stride_m, int B, int Hq, int Hkv, int D, float scale, int dtype,
-                       int accumulate, const bam_bias* bias, void* stream) {
+                       int accumulate, const bam_bias* bias, const bam_plan* plan,
+        void* stream) {
     MaskSource m;
     BAM_TRY(indexed_source(iv, m));
     void *dk = nullptr, *dv = nullptr;
@@ -516,8 +579,48 @@ int bam_bwd_dq_indexed(const void* q, const void* k, const void* v, const void* 
     const int64_t st[23] = BAM_BWD_STRIDES;
     bam::AttnParams p = {};
     BAM_TRY(bwd_params(p, "bam_bwd_dq_indexed", q, k, v, dout, lse, delta, dq, dk, dv, m, flags, st, B, Hq, Hkv, D, scale,
-                       dtype, accumulate, true, false, bias, nullptr));
+                       dtype, accumulate, true, false, bias, plan));
     return launched(bam::launch_bwd_dq(p, dtype, (hipStream_t)stream), "bam_bwd_dq_indexed");
+}
+
+int bam_decode(const void* q, const void* k, const void* v, void* o, int64_t q_stride_b, int64_t q_stride_h,
+               int64_t k_stride_b, int64_t k_stride_s, int64_t k_stride_h, int64_t v_stride_b, int64_t v_stride_s,
+               int64_t v_stride_h, int64_t o_stride_b, int64_t o_stride_h, int B, int Sk, int Hq, int Hkv, int D, float scale,
+               int dtype, int window, float softcap, void* stream) {
+    BAM_TRY(check_problem(B, 1, Sk, Hq, Hkv, D, dtype));
+    BAM_TRY(check_half_tensor("k", k, k_stride_b, k_stride_s, k_stride_h));
+    BAM_TRY(check_half_tensor("v", v, v_stride_b, v_stride_s, v_stride_h));
+    if (q == nullptr || o == nullptr) return fail(BAM_ERR_INVALID_ARGUMENT, "bam_decode: null pointer");
+    if ((reinterpret_cast<uintptr_t>(q) & 1u) || (reinterpret_cast<uintptr_t>(o) & 1u))
+        return fail(BAM_ERR_INVALID_ARGUMENT, "bam_decode: q / o are not 2-byte aligned");
+    if (!(scale > 0.f)) return fail(BAM_ERR_INVALID_ARGUMENT, "bam_decode: softmax scale must be > 0 (got %g)", scale);
+    if (window < 0) return fail(BAM_ERR_INVALID_ARGUMENT, "bam_decode: window must be >= 0 (0 = none), got %d", window);
+    if (!(softcap >= 0.f)) return fail(BAM_ERR_INVALID_ARGUMENT, "bam_decode: softcap must be >= 0 (0 = none), got %g", softcap);
+    if ((int64_t)B * Hq > 0x7FFFFFFFll) return fail(BAM_ERR_UNSUPPORTED, "bam_decode: grid too large");
+    bam::DecodeParams p = {};
+    p.q = q;
+    p.k = k;
+    p.v = v;
+    p.o = o;
+    p.q_sb = q_stride_b;
+    p.q_sh = q_stride_h;
+    p.k_sb = k_stride_b;
+    p.k_ss = k_stride_s;
+    p.k_sh = k_stride_h;
+    p.v_sb = v_stride_b;
+    p.v_ss = v_stride_s;
+    p.v_sh = v_stride_h;
+    p.o_sb = o_stride_b;
+    p.o_sh = o_stride_h;
+    p.B = B;
+    p.Sk = Sk;
+    p.Hq = Hq;
+    p.Hkv = Hkv;
+    p.D = D;
+    p.window = window;
+    p.scale = scale;
+    p.softcap = softcap;
+    return launched(bam::launch_decode(p, dtype, (hipStream_t)stream), "bam_decode");
 }
 
 int bam_mask_tile_flags(const uint8_t* mask, int8_t* flags, int64_t flags_stride_b, int64_t flags_stride_m, int B,
@@ -535,11 +638,12 @@ int bam_fwd_masked(const void* q, const void* k, const void* v, void* o, float* 
                    int64_t k_stride_b, int64_t k_stride_s, int64_t k_stride_h, int64_t v_stride_b,
                    int64_t v_stride_s, int64_t v_stride_h, int64_t o_stride_b, int64_t o_stride_s,
                    int64_t o_stride_h, int64_t flags_stride_b, int64_t flags_stride_m, int B, int Sq, int Sk, int Hq,
-                   int Hkv, int D, float scale, int dtype, const bam_bias* bias, void* stream) {
+                   int Hkv, int D, float scale, int dtype, const bam_bias* bias, const bam_plan* plan,
+        void* stream) {
     BAM_TRY(check_mask("bam_fwd_masked", mask));
     const int64_t st[12] = BAM_FWD_STRIDES;
     return fwd_impl("bam_fwd_masked", q, k, v, o, lse, dense_source(mask, Sq, Sk), flags, st, flags_stride_b,
-                    flags_stride_m, B, Hq, Hkv, D, scale, dtype, bias, nullptr, stream);
+                    flags_stride_m, B, Hq, Hkv, D, scale, dtype, bias, plan, stream);
 }
 
 int bam_bwd_dkdv_masked(const void* q, const void* k, const void* v, const void* dout, const float* lse,
@@ -550,14 +654,15 @@ int bam_bwd_dkdv_masked(const void* q, const void* k, const void* v, const void*
                         int64_t dk_stride_b, int64_t dk_stride_s, int64_t dk_stride_h, int64_t dv_stride_b,
                         int64_t dv_stride_s, int64_t dv_stride_h, int64_t flags_stride_b, int64_t flags_stride_m,
                         int B, int Sq, int Sk, int Hq, int Hkv, int D, float scale, int dtype, int accumulate,
-                        const bam_bias* bias, void* stream) {
+                        const bam_bias* bias, const bam_plan* plan,
+        void* stream) {
     BAM_TRY(check_mask("bam_bwd_dkdv_masked", mask));
     void* dq = nullptr;
     const int64_t dq_stride_b = 0, dq_stride_s = 0, dq_stride_h = 0;
     const int64_t st[23] = BAM_BWD_STRIDES;
     bam::AttnParams p = {};
     BAM_TRY(bwd_params(p, "bam_bwd_dkdv_masked", q, k, v, dout, lse, delta, dq, dk, dv, dense_source(mask, Sq, Sk), flags,
-                       st, B, Hq, Hkv, D, scale, dtype, accumulate, false, true, bias, nullptr));
+                       st, B, Hq, Hkv, D, scale, dtype, accumulate, false, true, bias, plan));
     return launched(bam::launch_bwd_dkdv(p, dtype, (hipStream_t)stream), "bam_bwd_dkdv_masked");
 }
 
@@ -567,14 +672,15 @@ int bam_bwd_dq_masked(const void* q, const void* k, const void* v, const void* d
                       int64_t k_stride_h, int64_t v_stride_b, int64_t v_stride_s, int64_t v_stride_h,
                       int64_t do_stride_b, int64_t do_stride_s, int64_t do_stride_h, int64_t dq_stride_b,
                       int64_t dq_stride_s, int64_t dq_stride_h, int64_t flags_stride_b, int64_t flags_stride_m, int B,
-                      int Sq, int Sk, int Hq, int Hkv, int D, float scale, int dtype, int accumulate, const bam_bias* bias, void* stream) {
+                      int Sq, int Sk, int Hq, int Hkv, int D, float scale, int dtype, int accumulate, const bam_bias* bias, const bam_plan* plan,
+        void* stream) {
     BAM_TRY(check_mask("bam_bwd_dq_masked", mask));
     void *dk = nullptr, *dv = nullptr;
     const int64_t dk_stride_b = 0, dk_stride_s = 0, dk_stride_h = 0, dv_stride_b = 0, dv_stride_s = 0, dv_stride_h = 0;
     const int64_t st[23] = BAM_BWD_STRIDES;
     bam::AttnParams p = {};
     BAM_TRY(bwd_params(p, "bam_bwd_dq_masked", q, k, v, dout, lse, delta, dq, dk, dv, dense_source(mask, Sq, Sk), flags, st,
-                       B, Hq, Hkv, D, scale, dtype, accumulate, true, false, bias, nullptr));
+                       B, Hq, Hkv, D, scale, dtype, accumulate, true, false, bias, plan));
     return launched(bam::launch_bwd_dq(p, dtype, (hipStream_t)stream), "bam_bwd_dq_masked");
 }
 

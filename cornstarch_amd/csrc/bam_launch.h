@@ -63,6 +63,16 @@ struct AttnParams {
     float scale;
 };
 
+// Single-token decode step (one query row per batch element and head, no mask); strides in elements.
+struct DecodeParams {
+    const void *q, *k, *v;         // q (B, Hq, D): q_sb, q_sh; k / v (B, Sk, Hkv, D): *_sb, *_ss, *_sh
+    void* o;                       // (B, Hq, D) in the dtype of q
+    int64_t q_sb, q_sh, k_sb, k_ss, k_sh, v_sb, v_ss, v_sh, o_sb, o_sh;
+    int B, Sk, Hq, Hkv, D;
+    int window;                    // > 0: only the last `window` keys are attended to
+    float scale, softcap;          // softcap > 0: scores become softcap * tanh(score / softcap)
+};
+
 int launch_tile_flags(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int64_t flags_stride_b,
                       int64_t flags_stride_m, int B, int S, hipStream_t stream);
 // Flags plus plan in one launch: fine (B, 4 * num_m, fine_ss) bytes, order (B, 4 * num_m) ints.
@@ -77,9 +87,18 @@ int launch_mask_tile_flags(const uint8_t* mask, int8_t* flags, int64_t flags_str
                            int Sq, int Sk, hipStream_t stream);
 int launch_gather_bitfields(const int64_t* bf, int64_t bf_stride_b, int L, const int64_t* idx, int n, int64_t* out_bits,
                             int64_t out_stride_b, int* out_pos, int B, hipStream_t stream);
+// Plan (fine classes + slice order) of index-tensor attention, from the gathered bitfields and positions.
+int launch_indexed_plan(const int64_t* qbits, int64_t qbits_sb, const int64_t* kbits, int64_t kbits_sb, const int* qpos,
+                        const int* kpos, int Sq, int Sk, uint8_t* fine, int64_t fine_sb, int64_t fine_ss, int* order,
+                        int64_t order_sb, int B, hipStream_t stream);
+// Flags plus plan of a materialized bool mask.
+int launch_mask_tile_plan(const uint8_t* mask, int8_t* flags, int64_t flags_stride_b, int64_t flags_stride_m,
+                          uint8_t* fine, int64_t fine_sb, int64_t fine_ss, int* order, int64_t order_sb, int B, int Sq,
+                          int Sk, hipStream_t stream);
 int launch_fwd(const AttnParams& p, int dtype, hipStream_t stream);
 int launch_bwd_preprocess(const AttnParams& p, int dtype, hipStream_t stream);
 int launch_bwd_dkdv(const AttnParams& p, int dtype, hipStream_t stream);
 int launch_bwd_dq(const AttnParams& p, int dtype, hipStream_t stream);
+int launch_decode(const DecodeParams& p, int dtype, hipStream_t stream);
 
 }  // namespace bam

@@ -59,7 +59,8 @@ __global__ __launch_bounds__(FWD_THREADS, D == 128 ? 2 : 3) void fwd_kernel(cons
     const int ub = unit / p.Hkv;
     const int b = ub % p.B;
     const int h = hk * G + g;
-    const WaveSlices ws = pick_wave_slices(p, b, ub / p.B);  // group 0 is the heaviest
+    const int grp = ub / p.B;
+    const WaveSlices ws = pick_wave_slices(p, b, grp);  // group 0 is the heaviest
 
     if (wave == 0) build_key_tile_list(ws, p.num_n, Sk, lane, 0, sList, &sCount);  // first pass (usually the only one)
 
@@ -386,6 +387,10 @@ __global__ __launch_bounds__(FWD_THREADS, D == 128 ? 2 : 3) void fwd_kernel(cons
     if (hi == 0 && slice >= 0)
         p.lse[((int64_t)b * p.Hq + h) * p.Sq_rounded + qrow] =
             ltot > 0.f ? (m_i * c2 + __builtin_amdgcn_logf(ltot)) * LN2 : -INFINITY;
+    // A wave without a slice (plan: slot 4 grp + wave of the order lies past the last slice) owns the 32 padding rows
+    // of that slot, so that every row of the rounded lse is written whether or not a plan is given.
+    if (hi == 0 && slice < 0 && 32 * (4 * grp + wave) + 31 < p.Sq_rounded)
+        p.lse[((int64_t)b * p.Hq + h) * p.Sq_rounded + 32 * (4 * grp + wave) + l32] = -INFINITY;
     if (qvalid) {
         char* op = (char*)p.o.ptr + 2 * ((int64_t)b * p.o.sb + (int64_t)qrow * p.o.ss + (int64_t)h * p.o.sh);
 #pragma unroll

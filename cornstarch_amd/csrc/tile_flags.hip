@@ -45,13 +45,15 @@ __device__ __forceinline__ void slice_sort_key(const int64_t* __restrict__ row, 
     k2 = text ? (unsigned long long)(ns - 1 - s) : (unsigned long long)s;
 }
 
-__device__ __forceinline__ void slice_order_part(const int64_t* __restrict__ row, int S, int part,
-                                                 int* __restrict__ order_row) {
+// Ranks the slices [256 part, +256) of one sequence among all `ns` slices by the two-word keys `key(s, k1, k2)`
+// delivers (distinct for distinct slices; slices >= ns get the largest key) and writes order_row[rank] = slice;
+// the slots past the last slice are set to -1.
+template <typename KeyFn>
+__device__ __forceinline__ void slice_order_ranked(KeyFn key, int ns, int slots, int part, int* __restrict__ order_row) {
     __shared__ unsigned long long sk[2 * 256];
-    const int ns = (S + 31) / 32, slots = 4 * ((S + BLOCK_M - 1) / BLOCK_M);
     const int tid = threadIdx.x, s = part * 256 + tid;
     unsigned long long my1, my2;
-    slice_sort_key(row, S, ns, s, my1, my2);
+    key(s, my1, my2);
     int rank = 0;
     for (int base = 0; base < ns; base += 256) {
         __syncthreads();
@@ -59,7 +61,7 @@ __device__ __forceinline__ void slice_order_part(const int64_t* __restrict__ row
             sk[2 * tid] = my1;
             sk[2 * tid + 1] = my2;
         } else {
-            slice_sort_key(row, S, ns, base + tid, sk[2 * tid], sk[2 * tid + 1]);
+            key(base + tid, sk[2 * tid], sk[2 * tid + 1]);
         }
         __syncthreads();
         const int cnt = min(256, ns - base);
@@ -72,6 +74,42 @@ __device__ __forceinline__ void slice_order_part(const int64_t* __restrict__ row
         order_row[rank] = s;
     else if (s < slots)
         order_row[s] = -1;
+}
+
+__device__ __forceinline__ void slice_order_part(const int64_t* __restrict__ row, int S, int part,
+                                                 int* __restrict__ order_row) {
+    const int ns = (S + 31) / 32, slots = 4 * ((S + BLOCK_M - 1) / BLOCK_M);
+    slice_order_ranked([&](int s, unsigned long long& k1, unsigned long long& k2) { slice_sort_key(row, S, ns, s, k1, k2); },
+                       ns, slots, part, order_row);
+}
+
+// The same ordering idea for index-tensor attention, where a local row's position is pos[row]: slices holding a
+// text row first, by descending largest position; then modality-only slices grouped by the OR of their bitfields,
+// by ascending smallest position.  The slice number in the low bits keeps the keys distinct whatever the positions.
+__device__ __forceinline__ void slice_sort_key_indexed(const int64_t* __restrict__ bits, const int* __restrict__ pos,
+                                                       int S, int ns, int s, unsigned long long& k1,
+                                                       unsigned long long& k2) {
+    k1 = ~0ull;
+    k2 = ~0ull;
+    if (s >= ns) return;
+    const int64_t M = (((int64_t)1) << 62) - 1;
+    int64_t sig = 0;
+    bool text = false;
+    int pmax = 0, pmin = 0x7FFFFFFF;
+#pragma unroll
+    for (int r = 0; r < 32; ++r) {
+        const int i = s * 32 + r;
+        const int64_t f = i < S ? bits[i] : 0;
+        const int q = i < S ? pos[i] : 0;
+        sig |= f & M;
+        text |= (f & 1) != 0;
+        if (i < S) {
+            pmax = max(pmax, q);
+            pmin = min(pmin, q);
+        }
+    }
+    k1 = text ? 0ull : (1ull << 62) | (unsigned long long)sig;
+    k2 = ((unsigned long long)(text ? 0x7FFFFFFF - pmax : pmin) << 20) | (unsigned long long)s;
 }
 
 // FINE: also write the class of every 32-row x 32-column tile (the four row slices of each flag tile) to
@@ -285,6 +323,144 @@ int launch_flag_row_workloads(const int8_t* flags, int64_t flags_stride_b, int64
                               int num_n, int* out, hipStream_t stream) {
     hipLaunchKernelGGL(flag_row_workloads_kernel, dim3(num_m), dim3(256), 0, stream, flags, flags_stride_b,
                        flags_stride_m, B, num_n, out);
+    return (int)hipGetLastError();
+}
+
+// Plan for index-tensor attention: the class of every 32-row x 32-key tile of the LOCAL score matrix (rows and keys
+// are gathered subsets of a global sequence: bits / positions per local row and key, as bam_gather_bitfields
+// delivers them) and a slice order.  Brute force over the pairs of each tile, same wave layout as the flag kernel:
+// lane = key column (lane & 31) x 64-row half (lane >> 5).  The extra column of workgroups ranks the slices.
+__global__ __launch_bounds__(FLAG_WAVES * 64) void indexed_plan_kernel(
+    const int64_t* __restrict__ qbits, int64_t qbits_sb, const int64_t* __restrict__ kbits, int64_t kbits_sb,
+    const int* __restrict__ qpos, const int* __restrict__ kpos, int Sq, int Sk, int num_n, uint8_t* __restrict__ fine,
+    int64_t fine_sb, int64_t fine_ss, int* __restrict__ order, int64_t order_sb, int flag_blocks_x) {
+    const int b = blockIdx.z;
+    const int64_t* qrow = qbits + (int64_t)b * qbits_sb;
+    if ((int)blockIdx.x >= flag_blocks_x) {
+        const int part = blockIdx.y;
+        const int ns = (Sq + 31) / 32, slots = 4 * (int)gridDim.y;
+        if (part * 256 < slots)
+            slice_order_ranked([&](int s, unsigned long long& k1,
+                                   unsigned long long& k2) { slice_sort_key_indexed(qrow, qpos, Sq, ns, s, k1, k2); },
+                               ns, slots, part, order + (int64_t)b * order_sb);
+        return;
+    }
+    __shared__ int64_t q_bits[BLOCK_M];
+    __shared__ int q_pos[BLOCK_M];
+    __shared__ __attribute__((aligned(8))) uint8_t s_out[4][FLAG_COLS_PER_BLOCK];
+    const int m = blockIdx.y;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5;
+    if (tid < 4 * FLAG_COLS_PER_BLOCK) s_out[0][tid] = 0;
+    if (tid < BLOCK_M) {
+        const int i = m * BLOCK_M + tid;
+        q_bits[tid] = (i < Sq) ? qrow[i] : 0;
+        q_pos[tid] = (i < Sq) ? qpos[i] : 0;
+    }
+    __syncthreads();
+    const int64_t* krow = kbits + (int64_t)b * kbits_sb;
+#pragma unroll
+    for (int t = 0; t < FLAG_TILES_PER_WAVE; ++t) {
+        const int n = blockIdx.x * FLAG_COLS_PER_BLOCK + wave * FLAG_TILES_PER_WAVE + t;
+        if (n >= num_n) break;  // wave-uniform
+        const int j = n * BLOCK_N + (lane & 31);
+        const int64_t kf = (j < Sk) ? krow[j] : 0;
+        const int64_t kp = (j < Sk) ? kpos[j] : 0;
+        int cnt_a = 0, cnt_b = 0;  // rows [64 half, +32) and [64 half + 32, +32)
+#pragma unroll 8
+        for (int r = 0; r < 32; ++r) {
+            const int ri = half * 64 + r;
+            cnt_a += allow_rule(q_bits[ri], kf, q_pos[ri], kp) ? 1 : 0;
+            cnt_b += allow_rule(q_bits[ri + 32], kf, q_pos[ri + 32], kp) ? 1 : 0;
+        }
+#pragma unroll
+        for (int off = 16; off > 0; off >>= 1) {
+            cnt_a += __shfl_xor(cnt_a, off);
+            cnt_b += __shfl_xor(cnt_b, off);
+        }
+        const int cols_in_range = min(BLOCK_N, Sk - n * BLOCK_N);
+        const int col = wave * FLAG_TILES_PER_WAVE + t;
+        if ((lane & 31) == 0) {
+#pragma unroll
+            for (int x = 0; x < 2; ++x) {
+                const int w = 2 * half + x, c = x ? cnt_b : cnt_a;
+                const int rows = max(0, min(32, Sq - (m * BLOCK_M + 32 * w)));
+                s_out[w][col] = (uint8_t)(c == 0 ? 0 : c == rows * cols_in_range ? 2 : 1);
+            }
+        }
+    }
+    __syncthreads();
+    const int n0 = blockIdx.x * FLAG_COLS_PER_BLOCK;
+    if (tid < 4) {
+        static_assert(FLAG_COLS_PER_BLOCK == 8, "one 64-bit word per row");
+        *(unsigned long long*)(fine + (int64_t)b * fine_sb + (int64_t)(4 * m + tid) * fine_ss + n0) =
+            *(const unsigned long long*)s_out[tid];
+    }
+}
+
+int launch_indexed_plan(const int64_t* qbits, int64_t qbits_sb, const int64_t* kbits, int64_t kbits_sb, const int* qpos,
+                        const int* kpos, int Sq, int Sk, uint8_t* fine, int64_t fine_sb, int64_t fine_ss, int* order,
+                        int64_t order_sb, int B, hipStream_t stream) {
+    const int num_m = (Sq + BLOCK_M - 1) / BLOCK_M, num_n = (Sk + BLOCK_N - 1) / BLOCK_N;
+    const int flag_blocks_x = (num_n + FLAG_COLS_PER_BLOCK - 1) / FLAG_COLS_PER_BLOCK;
+    dim3 grid(flag_blocks_x + 1, num_m, B);
+    hipLaunchKernelGGL(indexed_plan_kernel, grid, dim3(FLAG_WAVES * 64), 0, stream, qbits, qbits_sb, kbits, kbits_sb, qpos,
+                       kpos, Sq, Sk, num_n, fine, fine_sb, fine_ss, order, order_sb, flag_blocks_x);
+    return (int)hipGetLastError();
+}
+
+// Flags and plan of a materialized bool mask in one launch: as mask_tile_flags_kernel, with the count kept per
+// 32-row slice, so that the four slice classes of every flag tile come out of the same pass over the mask.  The
+// slice order is simply "last slice first" (under a causal-like mask the late rows see the most keys); it is
+// written by the workgroups of column 0.
+__global__ __launch_bounds__(256) void mask_tile_plan_kernel(const uint8_t* __restrict__ mask, int8_t* __restrict__ flags,
+                                                             int64_t flags_stride_b, int64_t flags_stride_m, int Sq,
+                                                             int Sk, int num_n, uint8_t* __restrict__ fine,
+                                                             int64_t fine_sb, int64_t fine_ss, int* __restrict__ order,
+                                                             int64_t order_sb) {
+    const int b = blockIdx.z, m = blockIdx.y, tid = threadIdx.x;
+    if (blockIdx.x == 0 && tid < 4) {
+        const int ns = (Sq + 31) / 32, slot = 4 * m + tid;
+        order[(int64_t)b * order_sb + slot] = slot < ns ? ns - 1 - slot : -1;
+    }
+    const int col = blockIdx.x * 256 + tid;
+    const int r0 = m * BLOCK_M;
+    int count[4] = {0, 0, 0, 0};
+    if (col < Sk) {
+        const uint8_t* pcol = mask + (int64_t)b * Sq * Sk + col;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            const int ra = r0 + 32 * w, rb = min(ra + 32, Sq);
+            for (int r = ra; r < rb; ++r) count[w] += pcol[(int64_t)r * Sk] != 0;
+        }
+    }
+#pragma unroll
+    for (int off = 16; off > 0; off >>= 1) {  // over the 32 columns of a tile
+#pragma unroll
+        for (int w = 0; w < 4; ++w) count[w] += __shfl_xor(count[w], off);
+    }
+    const int n = blockIdx.x * 8 + (tid >> 5);
+    if ((tid & 31) == 0 && n < num_n) {
+        const int cols = min(BLOCK_N, Sk - n * BLOCK_N);
+        int total = 0, cells = 0;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            const int rows = max(0, min(32, Sq - (r0 + 32 * w)));
+            fine[(int64_t)b * fine_sb + (int64_t)(4 * m + w) * fine_ss + n] =
+                (uint8_t)(count[w] == 0 ? 0 : count[w] == rows * cols ? 2 : 1);
+            total += count[w];
+            cells += rows * cols;
+        }
+        flags[(int64_t)b * flags_stride_b + (int64_t)m * flags_stride_m + n] = total == 0 ? 0 : total == cells ? 2 : 1;
+    }
+}
+
+int launch_mask_tile_plan(const uint8_t* mask, int8_t* flags, int64_t flags_stride_b, int64_t flags_stride_m,
+                          uint8_t* fine, int64_t fine_sb, int64_t fine_ss, int* order, int64_t order_sb, int B, int Sq,
+                          int Sk, hipStream_t stream) {
+    const int num_m = (Sq + BLOCK_M - 1) / BLOCK_M, num_n = (Sk + BLOCK_N - 1) / BLOCK_N;
+    dim3 grid((num_n + 7) / 8, num_m, B);
+    hipLaunchKernelGGL(mask_tile_plan_kernel, grid, dim3(256), 0, stream, mask, flags, flags_stride_b, flags_stride_m, Sq,
+                       Sk, num_n, fine, fine_sb, fine_ss, order, order_sb);
     return (int)hipGetLastError();
 }
 

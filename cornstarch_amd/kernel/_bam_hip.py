@@ -15,7 +15,7 @@ BAM_DTYPE_F16 = 0
 BAM_DTYPE_BF16 = 1
 BAM_MAX_SEQLEN = 4194304
 BAM_STATIC_PLAN_BYTES = 8 << 20
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 _i64 = ctypes.c_int64
 _int = ctypes.c_int
@@ -59,7 +59,9 @@ class Plan(ctypes.Structure):
         ("order", ctypes.c_void_p),
         ("order_stride_b", ctypes.c_int64),
         ("B", ctypes.c_int32),
-        ("S", ctypes.c_int32),
+        ("Sq", ctypes.c_int32),
+        ("Sk", ctypes.c_int32),
+        ("generation", ctypes.c_int32),
     ]
 
 
@@ -79,14 +81,17 @@ SIGNATURES = {
     "bam_bwd_dkdv": [_ptr] * 10 + [_i64] * 21 + [_int] * 5 + [_f32, _int, _int, _bias, _plan, _ptr],
     "bam_bwd_dq": [_ptr] * 9 + [_i64] * 18 + [_int] * 5 + [_f32, _int, _int, _bias, _plan, _ptr],
     "bam_mask_tile_flags": [_ptr, _ptr, _i64, _i64, _int, _int, _int, _ptr],
-    "bam_fwd_masked": [_ptr] * 7 + [_i64] * 14 + [_int] * 6 + [_f32, _int, _bias, _ptr],
-    "bam_bwd_dkdv_masked": [_ptr] * 10 + [_i64] * 20 + [_int] * 6 + [_f32, _int, _int, _bias, _ptr],
-    "bam_bwd_dq_masked": [_ptr] * 9 + [_i64] * 17 + [_int] * 6 + [_f32, _int, _int, _bias, _ptr],
+    "bam_mask_tile_plan": [_ptr, _ptr, _i64, _i64, _ptr, _i64, _int, _int, _int, _plan, _ptr],
+    "bam_fwd_masked": [_ptr] * 7 + [_i64] * 14 + [_int] * 6 + [_f32, _int, _bias, _plan, _ptr],
+    "bam_bwd_dkdv_masked": [_ptr] * 10 + [_i64] * 20 + [_int] * 6 + [_f32, _int, _int, _bias, _plan, _ptr],
+    "bam_bwd_dq_masked": [_ptr] * 9 + [_i64] * 17 + [_int] * 6 + [_f32, _int, _int, _bias, _plan, _ptr],
     "bam_flag_row_workloads": [_ptr, _i64, _i64, _int, _int, _int, _ptr, _ptr],
     "bam_gather_bitfields": [_ptr, _i64, _int, _ptr, _int, _ptr, _i64, _ptr, _int, _ptr],
-    "bam_fwd_indexed": [_ptr] * 5 + [_view, _ptr] + [_i64] * 14 + [_int] * 4 + [_f32, _int, _bias, _ptr],
-    "bam_bwd_dkdv_indexed": [_ptr] * 8 + [_view, _ptr] + [_i64] * 20 + [_int] * 4 + [_f32, _int, _int, _bias, _ptr],
-    "bam_bwd_dq_indexed": [_ptr] * 7 + [_view, _ptr] + [_i64] * 17 + [_int] * 4 + [_f32, _int, _int, _bias, _ptr],
+    "bam_plan_indexed": [_view, _ptr, _i64, _int, _plan, _ptr],
+    "bam_fwd_indexed": [_ptr] * 5 + [_view, _ptr] + [_i64] * 14 + [_int] * 4 + [_f32, _int, _bias, _plan, _ptr],
+    "bam_bwd_dkdv_indexed": [_ptr] * 8 + [_view, _ptr] + [_i64] * 20 + [_int] * 4 + [_f32, _int, _int, _bias, _plan, _ptr],
+    "bam_bwd_dq_indexed": [_ptr] * 7 + [_view, _ptr] + [_i64] * 17 + [_int] * 4 + [_f32, _int, _int, _bias, _plan, _ptr],
+    "bam_decode": [_ptr] * 4 + [_i64] * 10 + [_int] * 5 + [_f32, _int, _int, _f32, _ptr],
 }
 
 _lib = None
@@ -113,6 +118,8 @@ def load() -> ctypes.CDLL:
     lib.bam_abi_version.argtypes = []
     lib.bam_plan_workspace_bytes.restype = _i64
     lib.bam_plan_workspace_bytes.argtypes = [_int, _int]
+    lib.bam_plan_workspace_bytes_rect.restype = _i64
+    lib.bam_plan_workspace_bytes_rect.argtypes = [_int, _int, _int]
     for name, argtypes in SIGNATURES.items():
         fn = getattr(lib, name)
         fn.argtypes = argtypes

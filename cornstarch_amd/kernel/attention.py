@@ -22,6 +22,8 @@ from . import _bam_hip
 from .bitfield_attention import (
     _bias_arg,
     _BiasView,
+    _plan_arg,
+    _TilePlan,
     _dtype_code,
     _is_kernel_ready,
     _kernel_ready,
@@ -48,6 +50,46 @@ def mask_tile_flags(mask: Optional[torch.Tensor], batch: int, seqlen_q: int, seq
             batch, seqlen_q, seqlen_k, _stream_ptr(device),
         )
     return flags
+
+
+class _MaskPlan:
+    """Flags and plan (classes of the 32 x 32 tiles, slice order) of a bool mask, from one pass over it.  The forward
+    and, later, the backward of one call bring the same mask tensor: the last result is kept, together with the mask
+    it was computed from (so its address cannot be handed to another tensor meanwhile), and reused while that is
+    unchanged."""
+
+    _last = None
+
+    @classmethod
+    def get(cls, mask: Optional[torch.Tensor], batch: int, seqlen_q: int, seqlen_k: int, device):
+        """-> (flags int8 (B, ceil(Sq/128), ceil(Sk/32)), plan or None)"""
+        if mask is None:
+            return mask_tile_flags(None, batch, seqlen_q, seqlen_k, device), None
+        key = (mask.data_ptr(), tuple(mask.shape), tuple(mask.stride()), mask._version, mask.device)
+        if cls._last is not None and cls._last[0] == key:
+            return cls._last[1], cls._last[2]
+        import ctypes
+
+        num_m, num_n = -(-seqlen_q // BLOCK_M), -(-seqlen_k // BLOCK_N)
+        with torch.cuda.device(device):
+            ws_bytes = _bam_hip.load().bam_plan_workspace_bytes_rect(batch, seqlen_q, seqlen_k)
+            if ws_bytes > 0:
+                flags = torch.empty((batch, num_m, num_n), dtype=torch.int8, device=device)
+                workspace = torch.empty((ws_bytes,), dtype=torch.uint8, device=device)
+                struct = _bam_hip.Plan()
+                _bam_hip.call(
+                    "bam_mask_tile_plan", mask.data_ptr(), flags.data_ptr(), flags.stride(0), flags.stride(1),
+                    workspace.data_ptr(), ws_bytes, batch, seqlen_q, seqlen_k, ctypes.byref(struct), _stream_ptr(device),
+                )
+                plan = _TilePlan(workspace, struct, flags)
+            else:
+                flags, plan = mask_tile_flags(mask, batch, seqlen_q, seqlen_k, device), None
+        cls._last = (key, flags, plan, mask)
+        return flags, plan
+
+    @classmethod
+    def forget(cls):
+        cls._last = None
 
 
 def _checked_mask(mask, batch, seqlen_q, seqlen_k):
@@ -90,7 +132,7 @@ def _flash_attn_forward(
     if dp != d:  # zero columns change neither q.k nor the first d columns of p.v
         q, k, v = (F.pad(x, (0, dp - d)) for x in (q, k, v))
     qk, kk, vk = (_kernel_ready(x, 8) for x in (q, k, v))
-    flags = mask_tile_flags(mask, batch, seqlen_q, seqlen_k, q.device)
+    flags, plan = _MaskPlan.get(mask, batch, seqlen_q, seqlen_k, q.device)
     lse = torch.empty((batch, nheads, flags.shape[1] * BLOCK_M), device=q.device, dtype=torch.float32)
     o = torch.empty_like(qk)
     with torch.cuda.device(q.device):
@@ -100,7 +142,7 @@ def _flash_attn_forward(
             mask.data_ptr() if mask is not None else None, flags.data_ptr(),
             *_strides3(qk, kk, vk, o), flags.stride(0), flags.stride(1),
             batch, seqlen_q, seqlen_k, nheads, nheads_k, dp, float(softmax_scale), _dtype_code(q.dtype),
-            _bias_arg(bias_view), _stream_ptr(q.device),
+            _bias_arg(bias_view), _plan_arg(plan), _stream_ptr(q.device),
         )
     if dp != d:
         o = o[..., :d].contiguous()
@@ -137,7 +179,7 @@ def _flash_attn_backward(
     # the reference asserts the unit stride here instead of copying (attention.py:1002-1019)
     bias_view = _BiasView(bias, q, batch, nheads, seqlen_q, seqlen_k, may_copy=False) if bias is not None else None
     mask = _checked_mask(mask, batch, seqlen_q, seqlen_k)
-    flags = mask_tile_flags(mask, batch, seqlen_q, seqlen_k, q.device)
+    flags, plan = _MaskPlan.get(mask, batch, seqlen_q, seqlen_k, q.device)
 
     dp = _padded_head_dim(d)
     outs = (dq, dk, dv)
@@ -158,7 +200,7 @@ def _flash_attn_backward(
             wk.data_ptr(), wv.data_ptr(), mask_ptr, flags.data_ptr(),
             *_strides3(qk, kk, vk, gk, wk, wv), flags.stride(0), flags.stride(1),
             batch, seqlen_q, seqlen_k, nheads, nheads_k, dp, float(softmax_scale), _dtype_code(q.dtype), 0,
-            _bias_arg(bias_view), _stream_ptr(q.device),
+            _bias_arg(bias_view), _plan_arg(plan), _stream_ptr(q.device),
         )
         _bam_hip.call(
             "bam_bwd_dq_masked",
@@ -166,7 +208,7 @@ def _flash_attn_backward(
             wq.data_ptr(), mask_ptr, flags.data_ptr(),
             *_strides3(qk, kk, vk, gk, wq), flags.stride(0), flags.stride(1),
             batch, seqlen_q, seqlen_k, nheads, nheads_k, dp, float(softmax_scale), _dtype_code(q.dtype), 0,
-            _bias_arg(bias_view), _stream_ptr(q.device),
+            _bias_arg(bias_view), _plan_arg(plan), _stream_ptr(q.device),
         )
     if not direct:
         for dst, w in zip(outs, work):

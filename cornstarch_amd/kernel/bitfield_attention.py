@@ -75,10 +75,10 @@ class _TilePlan:
     the class of every 32-row x 32-key tile and an order of the 32-row slices in which neighbours need the same
     keys.  Built together with the flags, lives in one workspace tensor, and belongs to exactly one flags tensor."""
 
-    def __init__(self, workspace: torch.Tensor, struct: "_bam_hip.Plan", flags: torch.Tensor):
+    def __init__(self, workspace: torch.Tensor, struct: "_bam_hip.Plan", flags: Optional[torch.Tensor]):
         self.workspace = workspace  # keeps the device memory alive
         self.struct = struct
-        self.flags = flags
+        self.flags = flags  # None for plans that are not tied to a flags tensor (index-tensor attention)
 
     def byref(self):
         import ctypes
@@ -88,13 +88,13 @@ class _TilePlan:
     def fine_classes(self) -> torch.Tensor:
         """uint8 (B, 4 * ceil(S/128), ceil(S/32)) view: class 0 / 1 / 2 of every 32-row x 32-key tile."""
         st, ws = self.struct, self.workspace
-        slots, num_n = 4 * self.flags.shape[1], self.flags.shape[2]
+        slots, num_n = 4 * (-(-st.Sq // BLOCK_M)), -(-st.Sk // BLOCK_N)
         return torch.as_strided(ws, (st.B, slots, num_n), (st.fine_stride_b, st.fine_stride_s, 1), st.fine - ws.data_ptr())
 
     def slice_order(self) -> torch.Tensor:
         """int32 (B, 4 * ceil(S/128)) view: the 32-row slices in the order the forward / dQ kernels take them."""
         st, ws = self.struct, self.workspace
-        return torch.as_strided(ws.view(torch.int32), (st.B, 4 * self.flags.shape[1]), (st.order_stride_b, 1),
+        return torch.as_strided(ws.view(torch.int32), (st.B, 4 * (-(-st.Sq // BLOCK_M))), (st.order_stride_b, 1),
                                 (st.order - ws.data_ptr()) // 4)
 
 
@@ -285,6 +285,20 @@ class _IndexView:
             self.q_bits.data_ptr(), self.k_bits.data_ptr(), self.q_pos.data_ptr(), self.k_pos.data_ptr(),
             self.q_bits.stride(0), self.k_bits.stride(0), self.seqlen_q, self.seqlen_k,
         )
+        # the plan of the shard (classes of its 32 x 32 tiles, slice order), from the gathered arrays
+        self.plan = None
+        with torch.cuda.device(dev):
+            ws_bytes = _bam_hip.load().bam_plan_workspace_bytes_rect(batch, self.seqlen_q, self.seqlen_k)
+            if ws_bytes > 0:
+                import ctypes
+
+                workspace = torch.empty((ws_bytes,), dtype=torch.uint8, device=dev)
+                struct = _bam_hip.Plan()
+                _bam_hip.call(
+                    "bam_plan_indexed", ctypes.byref(self.struct), workspace.data_ptr(), ws_bytes, batch,
+                    ctypes.byref(struct), _stream_ptr(dev),
+                )
+                self.plan = _TilePlan(workspace, struct, None)
 
     def byref(self):
         import ctypes
@@ -380,7 +394,7 @@ def _bitfield_attn_forward(
                 flags.data_ptr(), *_strides3(qk, kk, vk, o),
                 flags.stride(0), flags.stride(1),
                 batch, nheads, nheads_k, dp, float(softmax_scale), _dtype_code(q.dtype),
-                _bias_arg(bias_view), _stream_ptr(q.device),
+                _bias_arg(bias_view), _plan_arg(view.plan), _stream_ptr(q.device),
             )
     if dp != d:
         o = o[..., :d].contiguous()
@@ -417,7 +431,7 @@ def _launch_bwd_dkdv(q, k, v, do, lse, delta, dk, dv, bf, flags, softmax_scale, 
                 dk.data_ptr(), dv.data_ptr(), bf.byref(), flags.data_ptr(),
                 *_strides3(q, k, v, do, dk, dv), flags.stride(0), flags.stride(1),
                 B, Hq, k.shape[2], D, float(softmax_scale), _dtype_code(q.dtype), int(accumulate),
-                _bias_arg(bias), _stream_ptr(q.device),
+                _bias_arg(bias), _plan_arg(bf.plan), _stream_ptr(q.device),
             )
             return
         _bam_hip.call(
@@ -440,7 +454,7 @@ def _launch_bwd_dq(q, k, v, do, lse, delta, dq, bf, flags, softmax_scale, accumu
                 dq.data_ptr(), bf.byref(), flags.data_ptr(),
                 *_strides3(q, k, v, do, dq), flags.stride(0), flags.stride(1),
                 B, Hq, k.shape[2], D, float(softmax_scale), _dtype_code(q.dtype), int(accumulate),
-                _bias_arg(bias), _stream_ptr(q.device),
+                _bias_arg(bias), _plan_arg(bf.plan), _stream_ptr(q.device),
             )
             return
         _bam_hip.call(

@@ -85,8 +85,9 @@ typedef struct bam_bias {
  *   order: int32 (B, 4 * ceil(S/128)) -- the row slices of each sequence sorted so that four neighbours need
  *          about the same keys (slices holding text rows first, latest first; then modality-only slices grouped
  *          by modality), -1 in the unused tail.
- * bam_tile_plan fills the arrays (inside a caller-provided device workspace) and this host struct; the plain
- * bitfield entry points (bam_fwd, bam_bwd, bam_bwd_dkdv, bam_bwd_dq) take a `const bam_plan*` that may be null.
+ * bam_tile_plan fills the arrays (inside a caller-provided device workspace) and this host struct; bam_plan_indexed
+ * and bam_mask_tile_plan do the same for index-tensor attention and for a materialized mask (rows and keys may then
+ * differ in number).  Every attention entry point takes a `const bam_plan*` that may be null.
  * With a plan, the forward and dQ kernels build their workgroups from four slices of `order` and every wave skips
  * the key tiles its own slice does not need; dK/dV walks the slices that have work for its keys, two at a time.
  * Results do not depend on whether a plan is given (same pairs, same arithmetic per pair; only the order in which
@@ -99,7 +100,9 @@ typedef struct bam_plan {
     const int32_t* order;
     int64_t order_stride_b;
     int32_t B;
-    int32_t S;
+    int32_t Sq;         /* query rows and keys the plan was built for (equal for plain bitfield attention) */
+    int32_t Sk;
+    int32_t generation; /* 0: caller-provided workspace; otherwise the call of bam_tile_plan_static that wrote it */
 } bam_plan;
 
 const char* bam_last_error(void);
@@ -124,6 +127,8 @@ int bam_tile_flags(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int64_
  * (S above 131072); bam_tile_plan then refuses, and the caller uses bam_tile_flags and passes no plan.
  */
 int64_t bam_plan_workspace_bytes(int B, int S);
+/* The same for Sq query rows against Sk keys (index-tensor attention, materialized masks); 0 above 131072 rows. */
+int64_t bam_plan_workspace_bytes_rect(int B, int Sq, int Sk);
 int bam_tile_plan(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int64_t flags_stride_b,
                   int64_t flags_stride_m, void* workspace, int64_t workspace_bytes, int B, int S, bam_plan* plan,
                   void* stream);
@@ -137,10 +142,24 @@ int bam_tile_plan(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int64_t
  * with BAM_ERR_UNSUPPORTED.  Every call on a GPU reuses that GPU's array: the plan it returns is valid until the
  * next call of this function on the same GPU, and calls whose work overlaps on one GPU (two streams, two threads)
  * race.  Nothing in the array has to start at zero: every byte a later kernel reads is rewritten by each call.
+ * A plan of an earlier call is refused by the attention entry points once a later call has reused the array
+ * (bam_plan.generation).  The first call on a GPU resolves the array's address (hipGetSymbolAddress, which may load
+ * the library's code onto that GPU): make one call outside graph capture before relying on "allocates nothing".
  */
 #define BAM_STATIC_PLAN_BYTES (8 << 20)
 int bam_tile_plan_static(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int64_t flags_stride_b,
                          int64_t flags_stride_m, int B, int S, bam_plan* plan, void* stream);
+
+/*
+ * Plan for index-tensor attention: classes of the 32 x 32 tiles of the LOCAL score matrix (iv->Sq rows against
+ * iv->Sk keys, bitfields and positions as bam_gather_bitfields delivers them) and a slice order, laid out in
+ * `workspace` (at least bam_plan_workspace_bytes_rect(B, iv->Sq, iv->Sk) bytes, 256-byte aligned).  No counterpart
+ * in the reference, whose context-parallel shards work from the re-indexed 128 x 32 flags alone
+ * (shardformer/layers/utils.py:331-353); with this plan a shard skips masked work at 32-row granularity like the
+ * unsharded path.  The flags the caller passes to the attention entry points are then not consulted.
+ */
+int bam_plan_indexed(const bam_index_view* iv, void* workspace, int64_t workspace_bytes, int B, bam_plan* plan,
+                     void* stream);
 
 /*
  * Dense bool mask, uint8 (B, S, S) contiguous: the allow rule for every pair
@@ -195,7 +214,8 @@ int bam_fwd_indexed(const void* q, const void* k, const void* v, void* o, float*
                     int64_t k_stride_b, int64_t k_stride_s, int64_t k_stride_h, int64_t v_stride_b,
                     int64_t v_stride_s, int64_t v_stride_h, int64_t o_stride_b, int64_t o_stride_s,
                     int64_t o_stride_h, int64_t flags_stride_b, int64_t flags_stride_m, int B, int Hq, int Hkv,
-                    int D, float scale, int dtype, const bam_bias* bias, void* stream);
+                    int D, float scale, int dtype, const bam_bias* bias, const bam_plan* plan,
+        void* stream);
 
 /*
  * delta[b,h,i] = sum_d o[b,i,h,d] * do[b,i,h,d] in fp32.  Replaces
@@ -266,7 +286,8 @@ int bam_bwd_dkdv_indexed(const void* q, const void* k, const void* v, const void
                          int64_t v_stride_h, int64_t do_stride_b, int64_t do_stride_s, int64_t do_stride_h,
                          int64_t dk_stride_b, int64_t dk_stride_s, int64_t dk_stride_h, int64_t dv_stride_b,
                          int64_t dv_stride_s, int64_t dv_stride_h, int64_t flags_stride_b, int64_t flags_stride_m,
-                         int B, int Hq, int Hkv, int D, float scale, int dtype, int accumulate, const bam_bias* bias, void* stream);
+                         int B, int Hq, int Hkv, int D, float scale, int dtype, int accumulate, const bam_bias* bias, const bam_plan* plan,
+        void* stream);
 
 int bam_bwd_dq_indexed(const void* q, const void* k, const void* v, const void* dout, const float* lse,
                        const float* delta, void* dq, const bam_index_view* iv, const int8_t* flags,
@@ -275,7 +296,8 @@ int bam_bwd_dq_indexed(const void* q, const void* k, const void* v, const void* 
                        int64_t v_stride_h, int64_t do_stride_b, int64_t do_stride_s, int64_t do_stride_h,
                        int64_t dq_stride_b, int64_t dq_stride_s, int64_t dq_stride_h, int64_t flags_stride_b,
                        int64_t flags_stride_m, int B, int Hq, int Hkv, int D, float scale, int dtype,
-                       int accumulate, const bam_bias* bias, void* stream);
+                       int accumulate, const bam_bias* bias, const bam_plan* plan,
+        void* stream);
 
 /*
  * Materialized-mask attention: the sibling path of the reference,
@@ -296,7 +318,8 @@ int bam_fwd_masked(const void* q, const void* k, const void* v, void* o, float* 
                    int64_t k_stride_b, int64_t k_stride_s, int64_t k_stride_h, int64_t v_stride_b,
                    int64_t v_stride_s, int64_t v_stride_h, int64_t o_stride_b, int64_t o_stride_s,
                    int64_t o_stride_h, int64_t flags_stride_b, int64_t flags_stride_m, int B, int Sq, int Sk, int Hq,
-                   int Hkv, int D, float scale, int dtype, const bam_bias* bias, void* stream);
+                   int Hkv, int D, float scale, int dtype, const bam_bias* bias, const bam_plan* plan,
+        void* stream);
 
 int bam_bwd_dkdv_masked(const void* q, const void* k, const void* v, const void* dout, const float* lse,
                         const float* delta, void* dk, void* dv, const uint8_t* mask, const int8_t* flags,
@@ -306,7 +329,8 @@ int bam_bwd_dkdv_masked(const void* q, const void* k, const void* v, const void*
                         int64_t dk_stride_b, int64_t dk_stride_s, int64_t dk_stride_h, int64_t dv_stride_b,
                         int64_t dv_stride_s, int64_t dv_stride_h, int64_t flags_stride_b, int64_t flags_stride_m,
                         int B, int Sq, int Sk, int Hq, int Hkv, int D, float scale, int dtype, int accumulate,
-                        const bam_bias* bias, void* stream);
+                        const bam_bias* bias, const bam_plan* plan,
+        void* stream);
 
 int bam_bwd_dq_masked(const void* q, const void* k, const void* v, const void* dout, const float* lse,
                       const float* delta, void* dq, const uint8_t* mask, const int8_t* flags, int64_t q_stride_b,
@@ -314,7 +338,32 @@ int bam_bwd_dq_masked(const void* q, const void* k, const void* v, const void* d
                       int64_t k_stride_h, int64_t v_stride_b, int64_t v_stride_s, int64_t v_stride_h,
                       int64_t do_stride_b, int64_t do_stride_s, int64_t do_stride_h, int64_t dq_stride_b,
                       int64_t dq_stride_s, int64_t dq_stride_h, int64_t flags_stride_b, int64_t flags_stride_m, int B,
-                      int Sq, int Sk, int Hq, int Hkv, int D, float scale, int dtype, int accumulate, const bam_bias* bias, void* stream);
+                      int Sq, int Sk, int Hq, int Hkv, int D, float scale, int dtype, int accumulate, const bam_bias* bias, const bam_plan* plan,
+        void* stream);
+
+/*
+ * bam_mask_tile_flags plus a plan, in one pass over the mask: the four 32-row classes of every flag tile and a slice
+ * order (last slice first).  workspace: at least bam_plan_workspace_bytes_rect(B, Sq, Sk) bytes, 256-byte aligned.
+ * Serves `_flash_attn_forward` / `_flash_attn_backward` of the reference's cornstarch/kernel/attention.py:855-1146,
+ * whose kernels decide per 128 x 32 tile inside the attention loop (:188-200).
+ */
+int bam_mask_tile_plan(const uint8_t* mask, int8_t* flags, int64_t flags_stride_b, int64_t flags_stride_m, void* workspace,
+                       int64_t workspace_bytes, int B, int Sq, int Sk, bam_plan* plan, void* stream);
+
+/*
+ * Single-token decode step of a model in eval mode: one query row per batch element and head against the whole
+ * key / value cache, no bitfield consulted.  The reference hands this case to flash-attn through transformers'
+ * `flash_attention_forward(module, q, k, v, attention_mask=None, dropout=, scaling=, sliding_window=, softcap=)`
+ * (cornstarch/kernel/interface.py:71-83); with one query at the last position that is
+ *   s_j = scale * q . k_j ;  s_j = softcap * tanh(s_j / softcap) when softcap > 0 ;
+ *   keys j < Sk - window are dropped when 0 < window < Sk ;  o = softmax(s) v.
+ * q, o: (B, Hq, D) with element strides for batch and head, unit stride along D, 2-byte aligned; k, v: (B, Sk, Hkv, D)
+ * under the common layout rules.  window = 0 / softcap = 0 mean "none".
+ */
+int bam_decode(const void* q, const void* k, const void* v, void* o, int64_t q_stride_b, int64_t q_stride_h,
+               int64_t k_stride_b, int64_t k_stride_s, int64_t k_stride_h, int64_t v_stride_b, int64_t v_stride_s,
+               int64_t v_stride_h, int64_t o_stride_b, int64_t o_stride_h, int B, int Sk, int Hq, int Hkv, int D, float scale,
+               int dtype, int window, float softcap, void* stream);
 
 #ifdef __cplusplus
 }

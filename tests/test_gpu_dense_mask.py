@@ -133,3 +133,53 @@ def test_full_size_mask_materialized_from_bitfields_gives_the_bitfield_result_bi
         else:
             assert rel_l2(a.float(), b.float()) <= 2e-3, name
     BA.BitfieldUtils.clear_cache()
+
+
+# ------------------------------------------------- flags + plan of a mask in one pass
+@pytest.mark.parametrize("Sq,Sk,D", [(300, 170, 64), (517, 517, 128), (1024, 2000, 32), (33, 700, 64)])
+def test_mask_plan_classes_and_results_do_not_depend_on_the_plan(Sq, Sk, D, monkeypatch):
+    d = dev()
+    g = torch.Generator().manual_seed(Sq + Sk)
+    mask = torch.rand(2, Sq, Sk, generator=g) < 0.5
+    mask[:, : Sq // 2, : Sk // 3] = True           # full tiles
+    mask[:, Sq // 3 :, Sk // 2 :] = False          # empty tiles
+    mask[0, 40:70, :] = False                      # one empty and two partly empty row slices
+    mask[:, -1, :] = False
+    mg = mask.to(d)
+    A._MaskPlan.forget()
+    flags, plan = A._MaskPlan.get(mg, 2, Sq, Sk, d)
+    assert plan is not None and torch.equal(flags.cpu(), O.mask_tile_flags(mask))
+    assert A._MaskPlan.get(mg, 2, Sq, Sk, d)[1] is plan          # kept for the backward of the same mask
+    n_q, n_k = -(-Sq // 32), -(-Sk // 32)
+    pad = torch.nn.functional.pad(mask, (0, n_k * 32 - Sk, 0, n_q * 32 - Sq))
+    cells = torch.nn.functional.pad(torch.ones_like(mask), (0, n_k * 32 - Sk, 0, n_q * 32 - Sq))
+    cnt = pad.view(2, n_q, 32, n_k, 32).sum(dim=(2, 4))
+    tot = cells.view(2, n_q, 32, n_k, 32).sum(dim=(2, 4))
+    want = torch.where(cnt == 0, 0, torch.where(cnt == tot, 2, 1)).to(torch.uint8)
+    fine = plan.fine_classes().cpu()
+    assert torch.equal(fine[:, :n_q], want) and (fine[:, n_q:] == 0).all()
+    for b in range(2):
+        order = plan.slice_order()[b].cpu().tolist()
+        assert order[:n_q] == list(range(n_q - 1, -1, -1)) and all(x == -1 for x in order[n_q:])
+
+    q, k, v, do = (t.to(d) for t in inputs(2, Sq, Sk, 4, 2, D, torch.bfloat16, seed=Sq))
+
+    def run():
+        o, lse, scale = A._flash_attn_forward(q, k, v, mask=mg)
+        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        A._flash_attn_backward(do, q, k, v, o, lse, dq, dk, dv, mask=mg, softmax_scale=scale)
+        torch.cuda.synchronize()
+        return o, lse[:, :, :Sq], dq, dk, dv
+
+    with_plan = run()
+    real_get = A._MaskPlan.get.__func__
+    monkeypatch.setattr(A._MaskPlan, "get", classmethod(lambda cls, *a: (real_get(cls, *a)[0], None)))
+    without = run()
+    for name, a, b in zip(("o", "lse", "dq", "dk", "dv"), with_plan, without):
+        if name in ("dk", "dv"):  # fp32 partial sums of the two row streams meet in another order
+            assert rel_l2(a.float(), b.float()) <= 2e-3, name
+        else:
+            assert torch.equal(a, b), name
+    o_ref, _ = O.masked_attention_forward(q.cpu(), k.cpu(), v.cpu(), mask)
+    torch.testing.assert_close(with_plan[0].float().cpu(), o_ref, atol=1e-2, rtol=1e-2)
+    A._MaskPlan.forget()

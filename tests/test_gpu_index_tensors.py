@@ -174,3 +174,56 @@ def test_index_view_is_gathered_once_per_forward_backward_pair():
     assert (o2.float().cpu() - o_ref).abs().max().item() <= O_MAX_ABS
     BA.BitfieldUtils.clear_cache()
     assert BA._IndexView._last is None
+
+
+# ------------------------------------------------- the plan of a shard (classes of its 32 x 32 tiles, slice order)
+def _rank_with_and_without_plan(q, k, v, do, bf, idx_q, idx_k, flags, use_plan):
+    d = dev()
+    ql, dol = q[:, idx_q].contiguous().to(d), do[:, idx_q].contiguous().to(d)
+    kl, vl = k[:, idx_k].contiguous().to(d), v[:, idx_k].contiguous().to(d)
+    bfg, fl = bf.to(d), flags.to(d)
+    oq, ok = idx_q.to(d), idx_k.to(d)
+    BA.BitfieldUtils.clear_cache()
+    view = BA._IndexView.get(bfg, oq, ok)
+    assert view.plan is not None
+    if not use_plan:
+        view.plan = None  # the kernels then work from the caller's 128 x 32 flags alone
+    o, lse, scale = BA._bitfield_attn_forward(ql, kl, vl, bfg, fl, oq, ok)
+    dq, dk, dv = (torch.zeros_like(t, dtype=torch.float32) for t in (ql, kl, vl))
+    BA._bitfield_attn_backward(dol, ql, kl, vl, o, bfg, fl, lse, dq, dk, dv, offsets_q=oq, offsets_k=ok, softmax_scale=scale)
+    torch.cuda.synchronize()
+    assert BA._IndexView._last[1] is view
+    return o.cpu(), lse[:, :, : idx_q.numel()].cpu(), dq.cpu(), dk.cpu(), dv.cpu(), view
+
+
+@pytest.mark.parametrize("kind", ["zigzag", "blocks", "scattered"])
+@pytest.mark.parametrize("S,D,Hq,Hkv", [(777, 64, 4, 2), (1024, 128, 4, 1)])
+def test_shard_results_do_not_depend_on_the_plan(kind, S, D, Hq, Hkv):
+    bf = random_bitfield(2, S, seed=S + 3, pad=5)
+    q, k, v, do = inputs(2, S, Hq, Hkv, D, torch.bfloat16, seed=S)
+    ranks = splits(S, kind)
+    idx_k = torch.cat(ranks)
+    for idx_q in ranks:
+        flags = O.tile_flags_indexed(bf, idx_q, idx_k)
+        without = _rank_with_and_without_plan(q, k, v, do, bf, idx_q, idx_k, flags, False)
+        with_plan = _rank_with_and_without_plan(q, k, v, do, bf, idx_q, idx_k, flags, True)
+        for name, a, b in zip(("o", "lse", "dq", "dk", "dv"), with_plan, without):
+            if name in ("dk", "dv"):  # fp32 partial sums of the two row streams meet in another order
+                assert rel_l2(a, b) <= 2e-3, name
+            else:
+                assert torch.equal(a, b), name
+        # the classes are those of the shard's own score matrix, at 32 x 32
+        view = with_plan[5]
+        n_q, n_k = -(-idx_q.numel() // 32), -(-idx_k.numel() // 32)
+        for b in range(2):
+            allow = O.allow_rows(bf[b], 0, idx_q.numel(), idx_q, idx_k)
+            pad = torch.nn.functional.pad(allow, (0, n_k * 32 - idx_k.numel(), 0, n_q * 32 - idx_q.numel()))
+            cells = torch.nn.functional.pad(torch.ones_like(allow), (0, n_k * 32 - idx_k.numel(), 0, n_q * 32 - idx_q.numel()))
+            cnt = pad.view(n_q, 32, n_k, 32).sum(dim=(1, 3))
+            tot = cells.view(n_q, 32, n_k, 32).sum(dim=(1, 3))
+            want = torch.where(cnt == 0, 0, torch.where(cnt == tot, 2, 1)).to(torch.uint8)
+            fine = view.plan.fine_classes()[b].cpu()
+            assert torch.equal(fine[:n_q], want) and (fine[n_q:] == 0).all()
+            order = view.plan.slice_order()[b].cpu().tolist()
+            assert sorted(order[:n_q]) == list(range(n_q)) and all(x == -1 for x in order[n_q:])
+    BA.BitfieldUtils.clear_cache()

@@ -56,6 +56,7 @@ def test_plan_in_the_built_in_array_equals_the_plan_in_a_caller_workspace():
     d = torch.device("cuda:0")
     lib = _bam_hip.load()
     stream = BA._stream_ptr(d)
+    earlier = []
     for B, S, seed in ((2, 1000, 5), (1, 283, 6)):  # the second call is smaller: stale bytes of the first stay behind it
         bf = random_bitfield(B, S, seed=seed, pad=3).to(d)
         num_m, num_n = -(-S // 128), -(-S // 32)
@@ -72,7 +73,8 @@ def test_plan_in_the_built_in_array_equals_the_plan_in_a_caller_workspace():
         plan_b = _bam_hip.Plan()
         _bam_hip.call("bam_tile_plan_static", bf.data_ptr(), bf.stride(0), flags_b.data_ptr(), flags_b.stride(0),
                       flags_b.stride(1), B, S, ctypes.byref(plan_b), stream)
-        assert plan_b.fine != plan_a.fine and (plan_b.B, plan_b.S) == (B, S)
+        assert plan_b.fine != plan_a.fine and (plan_b.B, plan_b.Sq, plan_b.Sk) == (B, S, S)
+        assert plan_a.generation == 0 and plan_b.generation > 0
         assert torch.equal(flags_a, flags_b) and torch.equal(flags_a.cpu(), O.tile_flags(bf.cpu()))
         fine_a, order_a = _views(plan_a, B, S)
         fine_b, order_b = _views(plan_b, B, S)
@@ -87,6 +89,42 @@ def test_plan_in_the_built_in_array_equals_the_plan_in_a_caller_workspace():
         assert torch.equal(o_a, o_b) and torch.equal(lse_a, lse_b)
         o_ref, _ = O.attention_forward(q, k, v, bf)
         assert (o_b.float() - o_ref).abs().max().item() <= 2e-2
+        earlier.append((q, k, v, bf, flags_b, plan_b))
+    # the plan of the first call lives in the array the second call has rewritten: it is refused, not used
+    q, k, v, bf, flags_b, plan_b = earlier[0]
+    with pytest.raises(_bam_hip.BamError, match="stale"):
+        _fwd(q, k, v, bf, flags_b, ctypes.byref(plan_b), 0.125)
+
+
+def test_the_static_entry_point_allocates_no_device_memory():
+    # after one warm-up call (which resolves the array's address on this GPU), a call changes neither the
+    # free device memory the driver reports nor what torch's allocator holds
+    d = torch.device("cuda:0")
+    hip = ctypes.CDLL("libamdhip64.so")
+    hip.hipMemGetInfo.argtypes = [ctypes.POINTER(ctypes.c_size_t), ctypes.POINTER(ctypes.c_size_t)]
+    hip.hipMemGetInfo.restype = ctypes.c_int
+    B, S = 2, 777
+    bf = random_bitfield(B, S, seed=2).to(d)
+    flags = torch.empty((B, -(-S // 128), -(-S // 32)), dtype=torch.int8, device=d)
+    plan = _bam_hip.Plan()
+
+    def call():
+        _bam_hip.call("bam_tile_plan_static", bf.data_ptr(), bf.stride(0), flags.data_ptr(), flags.stride(0),
+                      flags.stride(1), B, S, ctypes.byref(plan), BA._stream_ptr(d))
+
+    def free_bytes():
+        free, total = ctypes.c_size_t(), ctypes.c_size_t()
+        assert hip.hipMemGetInfo(ctypes.byref(free), ctypes.byref(total)) == 0
+        return free.value
+
+    call()
+    torch.cuda.synchronize()
+    before = (free_bytes(), torch.cuda.memory_allocated(d), torch.cuda.memory_reserved(d))
+    for _ in range(3):
+        call()
+    torch.cuda.synchronize()
+    assert (free_bytes(), torch.cuda.memory_allocated(d), torch.cuda.memory_reserved(d)) == before
+    assert torch.equal(flags.cpu(), O.tile_flags(bf.cpu()))
 
 
 def test_sizes_beyond_the_built_in_array_are_refused():
