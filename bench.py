@@ -27,6 +27,26 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 PEAK_BF16_DENSE_TFLOPS = 2500.0  # MI355X published dense bf16 MFMA peak
+PEAK_HBM_GBPS = 8000.0           # MI355X published HBM3E bandwidth
+
+
+def library_gemm_tflops(dev, n=8192, reps=10):
+    """bf16 GEMM of the vendor library (torch.matmul) on n x n x n, TFLOP/s: a reference point for what the MFMA
+    units of this box sustain, measured next to the attention kernels."""
+    import torch
+
+    a = torch.randn(n, n, device=dev, dtype=torch.bfloat16)
+    b = torch.randn(n, n, device=dev, dtype=torch.bfloat16)
+    for _ in range(3):
+        torch.matmul(a, b)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(reps):
+        torch.matmul(a, b)
+    e1.record()
+    torch.cuda.synchronize()
+    return round(2 * n ** 3 * reps / (e0.elapsed_time(e1) * 1e-3) / 1e12, 1)
 
 
 def parse():
@@ -102,11 +122,12 @@ def measured_traffic(workload, kernel):
     return None
 
 
-def issued_flops(flags, plan, w):
+def issued_flops(flags, plan, w, handover=False):
     """MFMA FLOPs the three attention kernels issue, from the tile lists they build: a wave of the forward
     and dQ kernels computes a 32-row slice against every 64-key tile in which the slice has a non-empty class
     (4 resp. 6 D-deep products per pair), a wave of dK/dV a 32-row slice against a 32-key group (8).  Partial
-    tiles count in full.  Without a plan a slice inherits the classes of its 128-row block."""
+    tiles count in full.  Without a plan a slice inherits the classes of its 128-row block.  With the dS hand-over
+    the dQ kernel runs one product per pair of the 32 x 32 blocks that have work (2)."""
     import torch.nn.functional as F
 
     cls = plan.fine_classes() if plan is not None else flags.repeat_interleave(4, dim=1)
@@ -119,7 +140,7 @@ def issued_flops(flags, plan, w):
     return {
         "fwd": 4 * per_pair * tiles64 * 32 * 64,
         "dkdv": 8 * per_pair * tiles32 * 32 * 32,
-        "dq": 6 * per_pair * tiles64 * 32 * 64,
+        "dq": 2 * per_pair * tiles32 * 32 * 32 if handover else 6 * per_pair * tiles64 * 32 * 64,
     }
 
 
@@ -145,6 +166,7 @@ def run_workload(name, steps, warmup, dev):
 
     stages = ["flags", "fwd", "alloc", "delta", "dkdv", "dq"]
     n_ev = len(stages) + 1
+    handover = [False]  # did the last step hand dS from dK/dV to dQ through a workspace?
 
     def step(ev=None):
         def mark(i):
@@ -164,6 +186,9 @@ def run_workload(name, steps, warmup, dev):
             return o, None
         dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
         delta = torch.empty_like(lse)
+        # the dS workspace of the backward (head dim 128), sized from the plan's pair count, as the autograd path does
+        ds_ws = plan.attach_ds_workspace(w.Hq, w.D, w.S) if plan is not None else None
+        handover[0] = ds_ws is not None
         mark(3)
         BA._launch_bwd_preprocess(o, do, delta)
         mark(4)
@@ -171,6 +196,8 @@ def run_workload(name, steps, warmup, dev):
         mark(5)
         BA._launch_bwd_dq(q, k, v, do, lse, delta, dq, bf, flags, scale, accumulate=False, plan=plan)
         mark(6)
+        if plan is not None:
+            plan.detach_ds_workspace()
         return o, (dq, dk, dv)
 
     for _ in range(warmup):
@@ -219,15 +246,114 @@ def run_workload(name, steps, warmup, dev):
 
     BA.BitfieldUtils.clear_cache()
     flags = BA.BitfieldUtils.materialize_compressed_mask_from_bitfield_mask(bf)
-    issued = issued_flops(flags, BA.BitfieldUtils.plan_for(flags, bf), w)
+    the_plan = BA.BitfieldUtils.plan_for(flags, bf)
+    issued = issued_flops(flags, the_plan, w, handover[0])
+    ds_bytes = the_plan.ds_pairs() * w.Hq * 8192 if (handover[0] and the_plan is not None) else 0
     BA.BitfieldUtils.clear_cache()
     return {
-        "w": w, "pairs": pairs, "f_fwd": f_fwd, "f_bwd": f_bwd,
+        "w": w, "pairs": pairs, "f_fwd": f_fwd, "f_bwd": f_bwd, "handover": handover[0], "ds_workspace_bytes": ds_bytes,
         "ms_per_step": ms_per_step, "median_ms_per_step": statistics.median(per_step),
         "stage_ms": stage_ms, "stage_median_ms": stage_med,
         "api_ms_per_step": api_wall * 1e3 / steps, "api_median_ms_per_step": statistics.median(api_times),
         "issued": issued,
     }
+
+
+def run_neighbouring_entry_points(dev, steps):
+    """C2-shaped records for the entry points either side of plain bitfield attention, forward + backward each:
+    a context-parallel shard (index tensors: rank 0 of a two-rank zigzag split, 4096 rows against all 8192 keys,
+    through `_bitfield_attn_forward` / `_bitfield_attn_backward`), the materialized C2 mask through `flash_attn_func`,
+    and an ALiBi-like bias vector through `bitfield_attn_func`.  Effective TFLOP/s over each case's unmasked pairs."""
+    import torch
+
+    from cornstarch_amd import workloads as W
+    from cornstarch_amd.kernel import attention as A
+    from cornstarch_amd.kernel import bitfield_attention as BA
+    from oracle import bam_oracle as O  # pair counts only (setup, untimed)
+
+    w = W.WORKLOADS["C2"]
+    q, k, v, do = (t.to(dev) for t in W.make_tensors("C2"))
+    bf = W.make_bitfields("C2").to(dev)
+    per_pair = 14 * w.D * w.Hq
+
+    def timed(fn):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / steps
+
+    def issued_ratio(plan, pairs, handover):
+        nz = plan.fine_classes() > 0
+        if nz.shape[-1] % 2:
+            nz = torch.nn.functional.pad(nz, (0, 1))
+        t64, t32 = int((nz[..., 0::2] | nz[..., 1::2]).sum()), int(nz.sum())
+        issued = 4 * t64 * 2048 + 8 * t32 * 1024 + (2 * t32 * 1024 if handover else 6 * t64 * 2048)
+        return round(issued / ((14 if handover else 18) * pairs), 4)
+
+    out = {}
+    # --- context-parallel shard
+    chunks = torch.arange(w.S, device=dev).chunk(4)
+    idx_q = torch.cat([chunks[0], chunks[3]])
+    idx_k = torch.cat([chunks[0], chunks[3], chunks[1], chunks[2]])
+    pairs = sum(int(O.allow_rows(bf[0], r0, min(r0 + 1024, idx_q.numel()), idx_q, idx_k).sum())
+                for r0 in range(0, idx_q.numel(), 1024))
+    ql, dol = q[:, idx_q].contiguous(), do[:, idx_q].contiguous()
+    kl, vl = k[:, idx_k].contiguous(), v[:, idx_k].contiguous()
+    BA.BitfieldUtils.clear_cache()
+    glob = BA.BitfieldUtils.materialize_compressed_mask_from_bitfield_mask(bf)
+    # the caller's recipe for the shard's 128 x 32 flags (reference shardformer/layers/utils.py:331-353)
+    flags = glob[:, idx_q[::128] // 128][:, :, idx_k[::32] // 32].contiguous()
+    grads = [torch.zeros_like(t, dtype=torch.float32) for t in (ql, kl, vl)]
+
+    def shard_step():
+        o, lse, sc = BA._bitfield_attn_forward(ql, kl, vl, bf, flags, idx_q, idx_k)
+        BA._bitfield_attn_backward(dol, ql, kl, vl, o, bf, flags, lse, *grads, offsets_q=idx_q, offsets_k=idx_k, softmax_scale=sc)
+
+    ms = timed(shard_step)
+    view = BA._IndexView.get(bf, idx_q, idx_k)
+    out["index_tensors_zigzag_rank0"] = {
+        "ms_per_step": round(ms, 4), "tflops": round(per_pair * pairs / (ms * 1e-3) / 1e12, 3), "unmasked_pairs": pairs,
+        "issued_over_unmasked": issued_ratio(view.plan, pairs, True), "steps": steps,
+    }
+    BA.BitfieldUtils.clear_cache()
+    # --- materialized mask
+    mask = BA.materialize_bitfield_mask(bf)
+    pairs = int(mask.sum())
+    qg, kg, vg = (t.detach().requires_grad_(True) for t in (q, k, v))
+
+    def mask_step():
+        A._MaskPlan.forget()  # flags and plan of the mask are rebuilt every step, like the bitfield flags in the headline
+        o = A.flash_attn_func(qg, kg, vg, mask=mask)
+        torch.autograd.grad(o, (qg, kg, vg), do)
+
+    ms = timed(mask_step)
+    _, mplan = A._MaskPlan.get(mask, w.B, w.S, w.S, dev)
+    out["materialized_mask"] = {
+        "ms_per_step": round(ms, 4), "tflops": round(per_pair * pairs / (ms * 1e-3) / 1e12, 3), "unmasked_pairs": pairs,
+        "issued_over_unmasked": issued_ratio(mplan, pairs, True), "steps": steps,
+    }
+    A._MaskPlan.forget()
+    del mask
+    # --- bias vector
+    slopes = torch.tensor([2.0 ** (-8.0 * (i + 1) / w.Hq) for i in range(w.Hq)], device=dev)
+    bias = (-torch.arange(w.S, device=dev, dtype=torch.float32))[None, None, None, :] * slopes[None, :, None, None] * 1e-3
+
+    def bias_step():
+        BA.BitfieldUtils.clear_cache()
+        o = BA.bitfield_attn_func(qg, kg, vg, bf, bias)
+        torch.autograd.grad(o, (qg, kg, vg), do)
+
+    ms = timed(bias_step)
+    out["alibi_bias_vector"] = {
+        "ms_per_step": round(ms, 4), "tflops": round(per_pair * pairs / (ms * 1e-3) / 1e12, 3), "unmasked_pairs": pairs,
+        "steps": steps,
+    }
+    BA.BitfieldUtils.clear_cache()
+    return out
 
 
 def main():
@@ -257,15 +383,38 @@ def main():
     fwd_ms = stage_ms["flags"] + stage_ms["fwd"]
     bwd_ms = stage_ms["alloc"] + stage_ms["delta"] + stage_ms["dkdv"] + stage_ms["dq"]
 
-    # dominant kernel and its algorithmic FLOPs per launch (5-GEMM accounting of the
-    # backward: the dK/dV kernel owns S, dP, dV, dK; the dQ kernel owns dQ)
+    # Per kernel: algorithmic FLOPs (5-GEMM accounting of the backward: the dK/dV kernel owns S, dP, dV, dK; the dQ
+    # kernel owns dQ) and algorithmic HBM bytes (every operand and result once; with the dS hand-over the workspace
+    # is written once by dK/dV and read once by dQ).
+    esz = 2
+    t_q, t_kv, t_row = w.B * w.S * w.Hq * w.D * esz, w.B * w.S * w.Hkv * w.D * esz, w.B * w.Hq * w.S * 4
+    ds_bytes = r["ds_workspace_bytes"]
     algo = {"fwd": f_fwd, "dkdv": 8 * w.D * w.Hq * pairs, "dq": 2 * w.D * w.Hq * pairs}
-    kname = {"fwd": "fwd_kernel", "dkdv": "bwd_dkdv_kernel", "dq": "bwd_dq_kernel"}
-    dom = max(algo, key=lambda s: stage_ms[s])
-    achieved = algo[dom] / (stage_ms[dom] * 1e-3) / 1e12
+    algo_bytes = {
+        "fwd": 2 * t_q + 2 * t_kv + t_row,
+        "dkdv": 2 * t_q + 4 * t_kv + 2 * t_row + ds_bytes,
+        "dq": (ds_bytes + t_kv + t_q) if r["handover"] else (3 * t_q + 2 * t_kv + 2 * t_row),
+    }
+    kname = {"fwd": "fwd_kernel", "dkdv": "bwd_dkdv_kernel", "dq": "bwd_dq_saved_kernel" if r["handover"] else "bwd_dq_kernel"}
+    kernels = {}
+    for s_ in algo:
+        sec = stage_ms[s_] * 1e-3
+        kernels[kname[s_]] = {
+            "avg_launch_ms": round(stage_ms[s_], 4),
+            "algorithmic_tflops": round(algo[s_] / sec / 1e12, 3),
+            "mfma_frac": round(algo[s_] / sec / 1e12 / PEAK_BF16_DENSE_TFLOPS, 4),
+            "algorithmic_gbytes_per_s": round(algo_bytes[s_] / sec / 1e9, 1),
+            "hbm_frac": round(algo_bytes[s_] / sec / 1e9 / PEAK_HBM_GBPS, 4),
+            "issued_tflops": round(r["issued"][s_] / sec / 1e12, 3),
+        }
+    dom = max(algo, key=lambda s_: stage_ms[s_])
+    dk = kernels[kname[dom]]
+    # the roof the dominant kernel sits closer to, by its own measured fractions
+    bound = "mfma" if dk["mfma_frac"] >= dk["hbm_frac"] else "hbm"
     traffic = measured_traffic(name, kname[dom])
 
     value = (f_fwd + f_bwd) / (ms_per_step * 1e-3) / 1e12
+    dq_gemms = 2 if r["handover"] else 6
     result = {
         "metric": "bitfield attention fwd+bwd effective TFLOP/s over unmasked pairs (S=8192 GQA bf16)"
         if name == "C2"
@@ -295,33 +444,35 @@ def main():
         "bwd_ms": round(bwd_ms, 4),
         "fwd_tflops": round(f_fwd / (fwd_ms * 1e-3) / 1e12, 3),
         "mfma_util_unmasked": round(value / PEAK_BF16_DENSE_TFLOPS, 4),
-        "stage_ms": {s: round(x, 4) for s, x in stage_ms.items()},
-        "stage_median_ms": {s: round(x, 4) for s, x in r["stage_median_ms"].items()},
+        "stage_ms": {s_: round(x, 4) for s_, x in stage_ms.items()},
+        "stage_median_ms": {s_: round(x, 4) for s_, x in r["stage_median_ms"].items()},
+        # backward decomposition in use: with the hand-over the dK/dV kernel stores its dS blocks (8 KiB per q head and
+        # (32-row slice, 128-key tile) pair) and the dQ kernel is one GEMM over them; without, dQ recomputes S and dP
+        "ds_handover": r["handover"],
+        "ds_workspace_bytes": ds_bytes,
         # MFMA FLOPs issued according to the tile lists, and their ratio to the algorithmic (unmasked-pair) FLOPs of
-        # the GEMMs each kernel runs (forward 2, dK/dV 4, dQ 3: dQ recomputes S and dP)
+        # the GEMMs each kernel runs (forward 2, dK/dV 4, dQ 1 with the hand-over, 3 without)
         "issued_mfma_flops": r["issued"],
         "issued_over_unmasked": {
             "fwd": round(r["issued"]["fwd"] / f_fwd, 4),
             "dkdv": round(r["issued"]["dkdv"] / (8 * w.D * w.Hq * pairs), 4),
-            "dq": round(r["issued"]["dq"] / (6 * w.D * w.Hq * pairs), 4),
+            "dq": round(r["issued"]["dq"] / (dq_gemms * w.D * w.Hq * pairs), 4),
         },
-        # what the measurements say holds the dominant kernel back: no single saturated unit -- MFMA pipe 43-54 %
-        # busy, ~30 % of wave time at s_waitcnt / barriers, 4-5 other vector instructions per MFMA
-        # (profiles/bam_kernels_C2_counters.txt); dK/dV reads 1.5 KB of LDS operands per MFMA (2 KB in its S / dP
-        # phase): at the MFMA peak that is 75 % (100 %) of the 256 B per clock a compute unit's LDS delivers
-        "limiter": "latency / instruction mix, not a saturated unit (dK/dV: LDS operand traffic = 75 % of LDS peak at MFMA peak)",
+        "kernels": kernels,
+        # the library's bf16 GEMM on this very box, same process: what a pure MFMA kernel sustains here
+        "library_gemm_tflops": library_gemm_tflops(dev),
         "roofline": {
             "kernel": kname[dom],
-            "bound": "mfma",
-            "achieved": round(achieved, 3),
-            "peak": PEAK_BF16_DENSE_TFLOPS,
-            "unit": "TFLOP/s",
-            "frac": round(achieved / PEAK_BF16_DENSE_TFLOPS, 4),
+            "bound": bound,
+            "achieved": dk["algorithmic_tflops"] if bound == "mfma" else dk["algorithmic_gbytes_per_s"],
+            "peak": PEAK_BF16_DENSE_TFLOPS if bound == "mfma" else PEAK_HBM_GBPS,
+            "unit": "TFLOP/s" if bound == "mfma" else "GB/s",
+            "frac": dk["mfma_frac"] if bound == "mfma" else dk["hbm_frac"],
             "traffic": traffic,
             "traffic_source": "profiles/hbm_traffic.txt (rocprofv3 --pmc run of this command on another box)"
             if traffic is not None else None,
-            "avg_launch_ms": round(stage_ms[dom], 4),
-            "issued_tflops": round(r["issued"][dom] / (stage_ms[dom] * 1e-3) / 1e12, 3),
+            "avg_launch_ms": dk["avg_launch_ms"],
+            "issued_tflops": dk["issued_tflops"],
         },
     }
     if name == "C2" and not args.no_other_workloads:
@@ -339,9 +490,12 @@ def main():
                 "steps": other_steps,
                 "unmasked_pairs": ro["pairs"],
                 "stage_ms": {s: round(x, 4) for s, x in ro["stage_ms"].items()},
-                "issued_over_unmasked": round(sum(ro["issued"].values()) / (18 * ro["w"].D * ro["w"].Hq * ro["pairs"]), 4),
+                "ds_handover": ro["handover"],
+                "issued_over_unmasked": round(sum(ro["issued"].values()) /
+                                              ((14 if ro["handover"] else 18) * ro["w"].D * ro["w"].Hq * ro["pairs"]), 4),
             }
         result["other_workloads"] = others
+        result["neighbouring_entry_points"] = run_neighbouring_entry_points(dev, args.other_steps * 2)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(name)
     print(json.dumps(result))

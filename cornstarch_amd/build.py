@@ -17,7 +17,7 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_PATH = os.path.join(PKG_DIR, "libbam_hip.so")
 # the longest compilations first: they are spread over the workers
-SOURCES = ["bwd_long.hip", "bwd_dkdv.hip", "bwd_dq.hip", "fwd_long.hip", "fwd.hip", "tile_flags.hip", "decode.hip", "bam_abi.hip"]
+SOURCES = ["bwd_long.hip", "bwd_dkdv.hip", "bwd_dkdv_save.hip", "bwd_dq_saved.hip", "bwd_dq.hip", "fwd_long.hip", "fwd.hip", "tile_flags.hip", "decode.hip", "bam_abi.hip"]
 ARCH = "gfx950"
 FLAGS = [
     f"--offload-arch={ARCH}",

@@ -150,6 +150,21 @@ int fill_plan(bam::AttnParams& p, const char* who, const bam_plan* plan, int B, 
     p.fine_ss = plan->fine_stride_s;
     p.order = plan->order;
     p.order_sb = plan->order_stride_b;
+    // hand-over of dS from dK/dV to dQ: only with a workspace, for the head dim and lengths its kernels cover
+    if (plan->ds_workspace != nullptr && plan->ds_entry != nullptr && plan->ds_tile_base != nullptr && p.D == 128 &&
+        Sk <= bam::MAX_LIST * 64) {
+        if (reinterpret_cast<uintptr_t>(plan->ds_workspace) & 15u)
+            return fail(BAM_ERR_INVALID_ARGUMENT, "%s: plan: dS workspace is not 16-byte aligned", who);
+        if (plan->ds_capacity <= 0) return fail(BAM_ERR_INVALID_ARGUMENT, "%s: plan: dS workspace without a capacity", who);
+        if ((int64_t)p.Hq * plan->ds_capacity > 0x7FFFFFFFll)  // record numbers are 32-bit in the kernels
+            return fail(BAM_ERR_UNSUPPORTED, "%s: plan: dS workspace of %lld pairs x %d heads has too many records", who,
+                        (long long)plan->ds_capacity, p.Hq);
+        p.ds_entry = plan->ds_entry;
+        p.ds_entry_sb = plan->ds_entry_stride_b;
+        p.ds_tile_base = plan->ds_tile_base;
+        p.ds_ws = plan->ds_workspace;
+        p.ds_capacity = plan->ds_capacity;
+    }
     return BAM_OK;
 }
 
@@ -264,6 +279,16 @@ int bwd_params(bam::AttnParams& p, const char* who, const void* q, const void* k
     return fill_bias(p, who, bias, m.Sk);
 }
 
+// with a dS workspace in the plan, dK/dV stores its dS blocks and dQ is computed from them
+int launch_dkdv(const bam::AttnParams& p, int dtype, void* stream) {
+    return p.ds_ws != nullptr ? bam::launch_bwd_dkdv_save(p, dtype, (hipStream_t)stream)
+                              : bam::launch_bwd_dkdv(p, dtype, (hipStream_t)stream);
+}
+int launch_dq(const bam::AttnParams& p, int dtype, void* stream) {
+    return p.ds_ws != nullptr ? bam::launch_bwd_dq_saved(p, dtype, (hipStream_t)stream)
+                              : bam::launch_bwd_dq(p, dtype, (hipStream_t)stream);
+}
+
 }  // namespace
 
 extern "C" {
@@ -286,7 +311,7 @@ int bam_tile_flags(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int64_
 namespace {
 // workspace layout: fine | order, each part 256-byte aligned
 struct PlanLayout {
-    int64_t fine_ss, fine_sb, order_sb, fine_off, order_off, bytes;
+    int64_t fine_ss, fine_sb, order_sb, entry_sb, fine_off, order_off, entry_off, base_off, count_off, bytes;
 };
 PlanLayout plan_layout(int B, int Sq, int Sk) {
     const int64_t num_m = (Sq + 127) / 128, num_n = (Sk + 31) / 32, slots = 4 * num_m;
@@ -297,7 +322,11 @@ PlanLayout plan_layout(int B, int Sq, int Sk) {
     l.order_sb = slots;
     l.fine_off = 0;
     l.order_off = up(B * l.fine_sb, 256);
-    l.bytes = l.order_off + up(B * slots * 4, 256);
+    l.entry_sb = slots * ((Sk + 127) / 128);
+    l.entry_off = l.order_off + up(B * slots * 4, 256);
+    l.base_off = l.entry_off + up(B * l.entry_sb * 4, 256);
+    l.count_off = l.base_off + up(B * ((Sk + 127) / 128) * 4, 256);
+    l.bytes = l.count_off + 256;
     return l;
 }
 }  // namespace
@@ -328,11 +357,26 @@ int place_plan(const char* who, void* workspace, int64_t workspace_bytes, int B,
     plan->fine_stride_s = l.fine_ss;
     plan->order = (const int32_t*)(w + l.order_off);
     plan->order_stride_b = l.order_sb;
+    plan->ds_entry = (const int32_t*)(w + l.entry_off);
+    plan->ds_entry_stride_b = l.entry_sb;
+    plan->ds_tile_base = (const int32_t*)(w + l.base_off);
+    plan->ds_count = (const int32_t*)(w + l.count_off);
+    plan->ds_workspace = nullptr;
+    plan->ds_capacity = 0;
     plan->B = B;
     plan->Sq = Sq;
     plan->Sk = Sk;
     plan->generation = 0;
     return BAM_OK;
+}
+
+// second launch of every plan builder: numbers the (slice, 128-key tile) pairs that have work
+int number_pairs(const char* who, const bam_plan* plan, void* stream) {
+    return launched(bam::launch_ds_entries(plan->fine, plan->fine_stride_b, plan->fine_stride_s, plan->B, plan->Sq, plan->Sk,
+                                           const_cast<int*>(plan->ds_entry), const_cast<int*>(plan->ds_tile_base),
+                                           const_cast<int*>(plan->ds_count),
+                                           (hipStream_t)stream),
+                    who);
 }
 }  // namespace
 
@@ -347,10 +391,11 @@ int bam_tile_plan(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int64_t
     PlanLayout l;
     BAM_TRY(place_plan("bam_tile_plan", workspace, workspace_bytes, B, S, S, plan, l));
     char* w = (char*)workspace;
-    return launched(bam::launch_tile_plan(bf, bf_stride_b, flags, flags_stride_b, flags_stride_m, (uint8_t*)(w + l.fine_off),
-                                          l.fine_sb, l.fine_ss, (int*)(w + l.order_off), l.order_sb, B, S,
-                                          (hipStream_t)stream),
-                    "bam_tile_plan");
+    BAM_TRY(launched(bam::launch_tile_plan(bf, bf_stride_b, flags, flags_stride_b, flags_stride_m, (uint8_t*)(w + l.fine_off),
+                                           l.fine_sb, l.fine_ss, (int*)(w + l.order_off), l.order_sb, B, S,
+                                           (hipStream_t)stream),
+                     "bam_tile_plan"));
+    return number_pairs("bam_tile_plan", plan, stream);
 }
 
 int bam_tile_plan_static(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int64_t flags_stride_b,
@@ -389,10 +434,11 @@ int bam_plan_indexed(const bam_index_view* iv, void* workspace, int64_t workspac
     PlanLayout l;
     BAM_TRY(place_plan("bam_plan_indexed", workspace, workspace_bytes, B, m.Sq, m.Sk, plan, l));
     char* w = (char*)workspace;
-    return launched(bam::launch_indexed_plan(m.bfq, m.bfq_sb, m.bfk, m.bfk_sb, m.posq, m.posk, m.Sq, m.Sk,
-                                             (uint8_t*)(w + l.fine_off), l.fine_sb, l.fine_ss, (int*)(w + l.order_off),
-                                             l.order_sb, B, (hipStream_t)stream),
-                    "bam_plan_indexed");
+    BAM_TRY(launched(bam::launch_indexed_plan(m.bfq, m.bfq_sb, m.bfk, m.bfk_sb, m.posq, m.posk, m.Sq, m.Sk,
+                                              (uint8_t*)(w + l.fine_off), l.fine_sb, l.fine_ss, (int*)(w + l.order_off),
+                                              l.order_sb, B, (hipStream_t)stream),
+                     "bam_plan_indexed"));
+    return number_pairs("bam_plan_indexed", plan, stream);
 }
 
 int bam_mask_tile_plan(const uint8_t* mask, int8_t* flags, int64_t flags_stride_b, int64_t flags_stride_m, void* workspace,
@@ -404,10 +450,16 @@ int bam_mask_tile_plan(const uint8_t* mask, int8_t* flags, int64_t flags_stride_
     PlanLayout l;
     BAM_TRY(place_plan("bam_mask_tile_plan", workspace, workspace_bytes, B, Sq, Sk, plan, l));
     char* w = (char*)workspace;
-    return launched(bam::launch_mask_tile_plan(mask, flags, flags_stride_b, flags_stride_m, (uint8_t*)(w + l.fine_off),
-                                               l.fine_sb, l.fine_ss, (int*)(w + l.order_off), l.order_sb, B, Sq, Sk,
-                                               (hipStream_t)stream),
-                    "bam_mask_tile_plan");
+    BAM_TRY(launched(bam::launch_mask_tile_plan(mask, flags, flags_stride_b, flags_stride_m, (uint8_t*)(w + l.fine_off),
+                                                l.fine_sb, l.fine_ss, (int*)(w + l.order_off), l.order_sb, B, Sq, Sk,
+                                                (hipStream_t)stream),
+                     "bam_mask_tile_plan"));
+    return number_pairs("bam_mask_tile_plan", plan, stream);
+}
+
+int64_t bam_ds_workspace_bytes(int Hq, int64_t pairs) {
+    if (Hq <= 0 || pairs <= 0) return 0;
+    return (int64_t)Hq * pairs * 8192;
 }
 
 int bam_materialize_mask(const int64_t* bf, int64_t bf_stride_b, uint8_t* out, int B, int S, void* stream) {
@@ -504,8 +556,8 @@ int bam_bwd(const void* q, const void* k, const void* v, const void* dout, const
     bam::AttnParams p = {};
     BAM_TRY(bwd_params(p, "bam_bwd", q, k, v, dout, lse, delta, dq, dk, dv, plain_source(bf, bf_stride_b, S), flags, st, B,
                        Hq, Hkv, D, scale, dtype, accumulate, true, true, bias, plan));
-    BAM_TRY(launched(bam::launch_bwd_dkdv(p, dtype, (hipStream_t)stream), "bam_bwd (dk/dv)"));
-    return launched(bam::launch_bwd_dq(p, dtype, (hipStream_t)stream), "bam_bwd (dq)");
+    BAM_TRY(launched(launch_dkdv(p, dtype, stream), "bam_bwd (dk/dv)"));
+    return launched(launch_dq(p, dtype, stream), "bam_bwd (dq)");
 }
 
 int bam_bwd_dkdv(const void* q, const void* k, const void* v, const void* dout, const float* lse,
@@ -523,7 +575,7 @@ int bam_bwd_dkdv(const void* q, const void* k, const void* v, const void* dout, 
     bam::AttnParams p = {};
     BAM_TRY(bwd_params(p, "bam_bwd_dkdv", q, k, v, dout, lse, delta, dq, dk, dv, plain_source(bf, bf_stride_b, S), flags,
                        st, B, Hq, Hkv, D, scale, dtype, accumulate, false, true, bias, plan));
-    return launched(bam::launch_bwd_dkdv(p, dtype, (hipStream_t)stream), "bam_bwd_dkdv");
+    return launched(launch_dkdv(p, dtype, stream), "bam_bwd_dkdv");
 }
 
 int bam_bwd_dq(const void* q, const void* k, const void* v, const void* dout, const float* lse,
@@ -540,7 +592,7 @@ int bam_bwd_dq(const void* q, const void* k, const void* v, const void* dout, co
     bam::AttnParams p = {};
     BAM_TRY(bwd_params(p, "bam_bwd_dq", q, k, v, dout, lse, delta, dq, dk, dv, plain_source(bf, bf_stride_b, S), flags, st,
                        B, Hq, Hkv, D, scale, dtype, accumulate, true, false, bias, plan));
-    return launched(bam::launch_bwd_dq(p, dtype, (hipStream_t)stream), "bam_bwd_dq");
+    return launched(launch_dq(p, dtype, stream), "bam_bwd_dq");
 }
 
 int bam_bwd_dkdv_indexed(const void* q, const void* k, const void* v, const void* dout, const float* lse,
@@ -560,7 +612,7 @@ int bam_bwd_dkdv_indexed(const void* q, const void* k, const void* v, const void
     bam::AttnParams p = {};
     BAM_TRY(bwd_params(p, "bam_bwd_dkdv_indexed", q, k, v, dout, lse, delta, dq, dk, dv, m, flags, st, B, Hq, Hkv, D, scale,
                        dtype, accumulate, false, true, bias, plan));
-    return launched(bam::launch_bwd_dkdv(p, dtype, (hipStream_t)stream), "bam_bwd_dkdv_indexed");
+    return launched(launch_dkdv(p, dtype, stream), "bam_bwd_dkdv_indexed");
 }
 
 int bam_bwd_dq_indexed(const void* q, const void* k, const void* v, const void* dout, const float* lse,
@@ -580,7 +632,7 @@ int bam_bwd_dq_indexed(const void* q, const void* k, const void* v, const void* 
     bam::AttnParams p = {};
     BAM_TRY(bwd_params(p, "bam_bwd_dq_indexed", q, k, v, dout, lse, delta, dq, dk, dv, m, flags, st, B, Hq, Hkv, D, scale,
                        dtype, accumulate, true, false, bias, plan));
-    return launched(bam::launch_bwd_dq(p, dtype, (hipStream_t)stream), "bam_bwd_dq_indexed");
+    return launched(launch_dq(p, dtype, stream), "bam_bwd_dq_indexed");
 }
 
 int bam_decode(const void* q, const void* k, const void* v, void* o, int64_t q_stride_b, int64_t q_stride_h,
@@ -663,7 +715,7 @@ int bam_bwd_dkdv_masked(const void* q, const void* k, const void* v, const void*
     bam::AttnParams p = {};
     BAM_TRY(bwd_params(p, "bam_bwd_dkdv_masked", q, k, v, dout, lse, delta, dq, dk, dv, dense_source(mask, Sq, Sk), flags,
                        st, B, Hq, Hkv, D, scale, dtype, accumulate, false, true, bias, plan));
-    return launched(bam::launch_bwd_dkdv(p, dtype, (hipStream_t)stream), "bam_bwd_dkdv_masked");
+    return launched(launch_dkdv(p, dtype, stream), "bam_bwd_dkdv_masked");
 }
 
 int bam_bwd_dq_masked(const void* q, const void* k, const void* v, const void* dout, const float* lse,
@@ -681,7 +733,7 @@ int bam_bwd_dq_masked(const void* q, const void* k, const void* v, const void* d
     bam::AttnParams p = {};
     BAM_TRY(bwd_params(p, "bam_bwd_dq_masked", q, k, v, dout, lse, delta, dq, dk, dv, dense_source(mask, Sq, Sk), flags, st,
                        B, Hq, Hkv, D, scale, dtype, accumulate, true, false, bias, plan));
-    return launched(bam::launch_bwd_dq(p, dtype, (hipStream_t)stream), "bam_bwd_dq_masked");
+    return launched(launch_dq(p, dtype, stream), "bam_bwd_dq_masked");
 }
 
 }  // extern "C"

@@ -58,6 +58,16 @@ struct AttnParams {
     int64_t fine_sb, fine_ss;
     const int* order;
     int64_t order_sb;
+    // Optional hand-over of dS from the dK/dV kernel to the dQ kernel (needs the plan; null = none).  ds_entry:
+    // number of every (slice, 128-key tile) pair that has work, (B, 4 * num_m, num_kt) ints, -1 = none.  ds_ws: one
+    // 8 KiB record per (q head, pair), record (h, e) at ((h * ds_capacity + e) * 8 KiB); inside it four 2 KiB blocks,
+    // one per 32-key group; a block holds, for each of its 32 keys, 32 values of -dS / scale in the input dtype.
+    const int* ds_entry;
+    int64_t ds_entry_sb;
+    const int* ds_tile_base;   // (B, num_kt): number of the first pair of each 128-key tile; the pairs of a tile are
+                               // numbered consecutively, by ascending slice
+    void* ds_ws;
+    int64_t ds_capacity;
     int B, Sq, Sk, Hq, Hkv, D;
     int Sq_rounded, num_m, num_n, num_kt;  // ceil(Sq/128)*128, ceil(Sq/128), ceil(Sk/32), ceil(Sk/128)
     float scale;
@@ -95,10 +105,17 @@ int launch_indexed_plan(const int64_t* qbits, int64_t qbits_sb, const int64_t* k
 int launch_mask_tile_plan(const uint8_t* mask, int8_t* flags, int64_t flags_stride_b, int64_t flags_stride_m,
                           uint8_t* fine, int64_t fine_sb, int64_t fine_ss, int* order, int64_t order_sb, int B, int Sq,
                           int Sk, hipStream_t stream);
+// Numbers the (slice, 128-key tile) pairs that have work: entry (B, 4 * num_m, ceil(Sk/128)) ints, -1 = none.
+// tile_base (B, ceil(Sk/128)) ints: number of the first pair of each key tile (pairs are numbered tile by tile).
+int launch_ds_entries(const uint8_t* fine, int64_t fine_sb, int64_t fine_ss, int B, int Sq, int Sk, int* entry,
+                      int* tile_base, int* count, hipStream_t stream);
 int launch_fwd(const AttnParams& p, int dtype, hipStream_t stream);
 int launch_bwd_preprocess(const AttnParams& p, int dtype, hipStream_t stream);
 int launch_bwd_dkdv(const AttnParams& p, int dtype, hipStream_t stream);
 int launch_bwd_dq(const AttnParams& p, int dtype, hipStream_t stream);
 int launch_decode(const DecodeParams& p, int dtype, hipStream_t stream);
+// dK/dV that also stores dS (p.ds_ws), and the dQ kernel that consumes it; D = 128, plan required
+int launch_bwd_dkdv_save(const AttnParams& p, int dtype, hipStream_t stream);
+int launch_bwd_dq_saved(const AttnParams& p, int dtype, hipStream_t stream);
 
 }  // namespace bam

@@ -70,7 +70,9 @@ constexpr int DKDV_THREADS = 512;
 // BIAS: the forward added p.bias to scale * q.k (reference bitfield_attention.py:815-835); P is recomputed with it.
 // LONG: sequences of more than MAX_SLICE_LIST 32-row slices (131072 rows), walked in several passes; the short form has
 // no pass loop at all (a loop around the main loop costs registers and a few per cent).
-template <typename T, int D, int MODE, bool BIAS, bool LONG>
+// SAVE: every wave also stores its 32 x 32 block of -dS / scale (the packed operand of the dK product) to p.ds_ws, where
+// the dQ kernel of bwd_dq_saved.h picks it up instead of recomputing S and dP.  Record and block layout: AttnParams.
+template <typename T, int D, int MODE, bool BIAS, bool LONG, bool SAVE = false>
 __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnParams p) {
     constexpr bool IDX = MODE == MASK_INDEXED, DENSE = MODE == MASK_DENSE;
     constexpr int NCH = D / 8, KK = D / 16, DB = D / 32;
@@ -254,15 +256,24 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
     // condition the compiler can prove wave-uniform makes it restructure the loop around that branch, and the
     // result needs far more registers than a wave has.
     const int kg_lane = (tid >> 6) & 3;
-    auto tile_step = [&](auto prefetch, int cur, int cls, int h_cur, int myrow0, const TileSource& next) {
+    // SAVE: where this lane's 32 bytes sit inside a 2 KiB block (key l32: 64 bytes, rows 4 hi + {0..3, 8..11, ...} first)
+    const unsigned ds_lane_off = (unsigned)(kg * 2048 + l32 * 64 + hi * 32);
+    // SAVE: the pairs (slice, this key tile) that have work are numbered consecutively from ds_base, by ascending slice,
+    // i.e. in the order of the slice list: pair number = ds_base + position in the list
+    int ds_base = 0;
+    if (SAVE) ds_base = __builtin_amdgcn_readfirstlane(p.ds_tile_base[(int64_t)b * p.num_kt + nt]);
+    // ds_pos: position of the wave's slice in the slice list.
+    // returns true when the wave has issued its two dS stores (they may stay in flight over the end of the iteration)
+    auto tile_step = [&](auto prefetch, int cur, int cls, int h_cur, int myrow0, int ds_pos, const TileSource& next) -> bool {
         constexpr bool PREFETCH = decltype(prefetch)::value;
         if (cls == 0) {
             if (PREFETCH) {
 #pragma unroll
                 for (int j = 0; j < NLOADS; ++j) issue_copy(j, next, cur ^ 1);
             }
-            return;
+            return false;
         }
+        const int ds_e = ds_base + ds_pos;
         const u32x4* tQ = sQ[cur];
         const u32x4* tG = sDO[cur];
         // ---- S = Q K^T and dP = dO V^T : 32 queries x 32 keys, two accumulator chains; both operands of
@@ -418,6 +429,20 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
                 }
             sched_pipeline_mfma_lds<4 * DB, 4, 2>();
         }
+        if (SAVE) {
+            // Issued after the MFMAs of the tile (in front of them they cost the kernel 2 % more).  Record number and
+            // record address are wave-uniform (kept in scalar registers); the two 16-byte stores are inline asm so that
+            // they take the scalar-base form and stay out of the compiler's load / store bookkeeping, like the tile
+            // copies (the caller waits with explicit counts); non-temporal: the blocks are read once, by another
+            // kernel, and should not push the Q / dO rows the other workgroups re-read out of L2
+            const unsigned rec_no = (unsigned)__builtin_amdgcn_readfirstlane(h_cur * (int)p.ds_capacity + ds_e);
+            const char* rec = (const char*)p.ds_ws + ((uint64_t)rec_no << 13);
+            asm volatile("global_store_dwordx4 %0, %1, %3 nt\n\tglobal_store_dwordx4 %0, %2, %3 offset:16 nt"
+                         :
+                         : "v"(ds_lane_off), "v"(dsb[0]), "v"(dsb[1]), "s"(rec)
+                         : "memory");
+        }
+        return SAVE;
     };
 
     // Sequences of more than MAX_SLICE_LIST slices are walked in several passes, from the end, each with a list
@@ -442,7 +467,7 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
             auto entry_lo = [&](int r) { return sList[n - 2 - 2 * r]; };  // entry -1 where the count is odd
             // current tile (g_cur, entries e_*), next tile (g_nxt, r_nxt, entries n_*, head base hb_nxt); past the
             // last tile "next" keeps walking through pairs of the last head, whose copies nobody reads
-            int g_cur = 0, g_nxt = 0, r_nxt = 0;
+            int g_cur = 0, g_nxt = 0, r_nxt = 0, r_cur = 0;
             HeadBase hb_nxt = head_base(hk * G);
             int e_lo = __builtin_amdgcn_readfirstlane(entry_lo(0)), e_hi = __builtin_amdgcn_readfirstlane(entry_hi(0));
             {
@@ -473,14 +498,20 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
                 const int a_lo = entry_lo(r_aft), a_hi = entry_hi(r_aft);
                 const TileSource next = tile_source(hb_nxt, (n_lo >> 8) * 32, (n_hi >> 8) * 32);
                 const int mine = st ? e_hi : e_lo;
-                tile_step(std::true_type{}, cur, (mine >> (2 * kg_lane)) & 3, hk * G + g_cur, (mine >> 8) * 32, next);
+                const bool stored = tile_step(std::true_type{}, cur, (mine >> (2 * kg_lane)) & 3, hk * G + g_cur,
+                                              (mine >> 8) * 32, n - 2 - 2 * r_cur + st, next);
                 g_cur = g_nxt;
+                r_cur = r_nxt;
                 e_lo = n_lo;
                 e_hi = n_hi;
                 advance();
                 n_lo = __builtin_amdgcn_readfirstlane(a_lo);
                 n_hi = __builtin_amdgcn_readfirstlane(a_hi);
-                wait_async();
+                // the copies of the next tile must have landed; the two dS stores, issued after them, may stay in flight
+                if (SAVE && stored)
+                    asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+                else
+                    wait_async();
                 __syncthreads();
             }
         }
@@ -510,7 +541,7 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
                 __syncthreads();
                 load_kv_operands();
                 // the slice sits in LDS rows 0..31: row stream 0 computes it, row stream 1 has nothing to do
-                tile_step(std::false_type{}, 0, st ? 0 : (entry >> (2 * kg_lane)) & 3, h, row0, TileSource{});
+                tile_step(std::false_type{}, 0, st ? 0 : (entry >> (2 * kg_lane)) & 3, h, row0, n_all - 1, TileSource{});
             }
         }
         if (!LONG) break;
@@ -926,6 +957,17 @@ static int launch_dkdv_b(const AttnParams& p, hipStream_t stream) {
         hipLaunchKernelGGL((bwd_dkdv_kernel<T, D, MASK_DENSE, BIAS, LONG>), dim3(blocks), dim3(DKDV_THREADS), 0, stream, p);
     else
         hipLaunchKernelGGL((bwd_dkdv_kernel<T, D, MASK_BITFIELD, BIAS, LONG>), dim3(blocks), dim3(DKDV_THREADS), 0, stream, p);
+    return (int)hipGetLastError();
+}
+template <typename T, int D, bool BIAS>
+static int launch_dkdv_save_b(const AttnParams& p, hipStream_t stream) {
+    const int blocks = p.num_kt * p.B * p.Hkv;
+    if (p.mask_mode == MASK_INDEXED)
+        hipLaunchKernelGGL((bwd_dkdv_kernel<T, D, MASK_INDEXED, BIAS, false, true>), dim3(blocks), dim3(DKDV_THREADS), 0, stream, p);
+    else if (p.mask_mode == MASK_DENSE)
+        hipLaunchKernelGGL((bwd_dkdv_kernel<T, D, MASK_DENSE, BIAS, false, true>), dim3(blocks), dim3(DKDV_THREADS), 0, stream, p);
+    else
+        hipLaunchKernelGGL((bwd_dkdv_kernel<T, D, MASK_BITFIELD, BIAS, false, true>), dim3(blocks), dim3(DKDV_THREADS), 0, stream, p);
     return (int)hipGetLastError();
 }
 template <typename T, int D, bool BIAS, bool LONG>

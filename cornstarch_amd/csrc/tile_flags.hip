@@ -464,6 +464,67 @@ int launch_mask_tile_plan(const uint8_t* mask, int8_t* flags, int64_t flags_stri
     return (int)hipGetLastError();
 }
 
+// Numbering of the (32-row slice, 128-key tile) pairs that have work, for the backward that hands dS from the dK/dV
+// kernel to the dQ kernel through memory.  Pairs are numbered in (batch, tile, slice) order, so the slices that have
+// work for one key tile -- exactly the list a dK/dV workgroup builds -- carry consecutive numbers:
+//   entry[b][s][t]  = number of pair (b, s, t), or -1 where its four classes are all "empty"  (what the dQ kernel looks up)
+//   tile_base[b][t] = number of the first pair of key tile (b, t)                             (what dK/dV starts from)
+//   *count          = how many pairs there are.
+// One workgroup: every thread counts a contiguous run of pairs, the counts are scanned, the run is numbered.
+constexpr int DS_SCAN_THREADS = 1024;
+__global__ __launch_bounds__(DS_SCAN_THREADS) void ds_entries_kernel(const uint8_t* __restrict__ fine, int64_t fine_sb,
+                                                                    int64_t fine_ss, int B, int slots, int nkt, int num_n,
+                                                                    int* __restrict__ entry, int* __restrict__ tile_base,
+                                                                    int* __restrict__ count) {
+    __shared__ int wave_total[DS_SCAN_THREADS / 64];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int64_t total = (int64_t)B * slots * nkt;
+    const int64_t per = (total + DS_SCAN_THREADS - 1) / DS_SCAN_THREADS;
+    const int64_t first = min(total, per * tid), last = min(total, first + per);
+    // position i of the scan = (b * nkt + t) * slots + s
+    auto has_work = [&](int64_t i) {
+        const int sl = (int)(i % slots);
+        const int64_t bt = i / slots;
+        const int t = (int)(bt % nkt);
+        const uint8_t* f = fine + (bt / nkt) * fine_sb + (int64_t)sl * fine_ss + 4 * t;
+        bool any = false;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) any |= (4 * t + w < num_n) && f[w] != 0;
+        return any;
+    };
+    int mine = 0;
+    for (int64_t i = first; i < last; ++i) mine += has_work(i) ? 1 : 0;
+    int incl = mine;  // inclusive scan inside the wave
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const int up = __shfl_up(incl, off);
+        if (lane >= off) incl += up;
+    }
+    if (lane == 63) wave_total[wave] = incl;
+    __syncthreads();
+    int base = 0, all = 0;
+    for (int w = 0; w < DS_SCAN_THREADS / 64; ++w) {
+        if (w < wave) base += wave_total[w];
+        all += wave_total[w];
+    }
+    int next = base + incl - mine;
+    for (int64_t i = first; i < last; ++i) {
+        const int sl = (int)(i % slots);
+        const int64_t bt = i / slots;
+        if (sl == 0) tile_base[bt] = next;
+        entry[((bt / nkt) * slots + sl) * nkt + (bt % nkt)] = has_work(i) ? next++ : -1;
+    }
+    if (tid == 0) *count = all;
+}
+
+int launch_ds_entries(const uint8_t* fine, int64_t fine_sb, int64_t fine_ss, int B, int Sq, int Sk, int* entry,
+                      int* tile_base, int* count, hipStream_t stream) {
+    const int slots = 4 * ((Sq + BLOCK_M - 1) / BLOCK_M), nkt = (Sk + 127) / 128, num_n = (Sk + BLOCK_N - 1) / BLOCK_N;
+    hipLaunchKernelGGL(ds_entries_kernel, dim3(1), dim3(DS_SCAN_THREADS), 0, stream, fine, fine_sb, fine_ss, B, slots, nkt,
+                       num_n, entry, tile_base, count);
+    return (int)hipGetLastError();
+}
+
 int launch_tile_flags(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int64_t flags_stride_b,
                       int64_t flags_stride_m, int B, int S, hipStream_t stream) {
     const int num_m = (S + BLOCK_M - 1) / BLOCK_M, num_n = (S + BLOCK_N - 1) / BLOCK_N;

@@ -58,6 +58,12 @@ class Plan(ctypes.Structure):
         ("fine_stride_s", ctypes.c_int64),
         ("order", ctypes.c_void_p),
         ("order_stride_b", ctypes.c_int64),
+        ("ds_entry", ctypes.c_void_p),
+        ("ds_entry_stride_b", ctypes.c_int64),
+        ("ds_tile_base", ctypes.c_void_p),
+        ("ds_count", ctypes.c_void_p),
+        ("ds_workspace", ctypes.c_void_p),
+        ("ds_capacity", ctypes.c_int64),
         ("B", ctypes.c_int32),
         ("Sq", ctypes.c_int32),
         ("Sk", ctypes.c_int32),
@@ -120,6 +126,8 @@ def load() -> ctypes.CDLL:
     lib.bam_plan_workspace_bytes.argtypes = [_int, _int]
     lib.bam_plan_workspace_bytes_rect.restype = _i64
     lib.bam_plan_workspace_bytes_rect.argtypes = [_int, _int, _int]
+    lib.bam_ds_workspace_bytes.restype = _i64
+    lib.bam_ds_workspace_bytes.argtypes = [_int, _i64]
     for name, argtypes in SIGNATURES.items():
         fn = getattr(lib, name)
         fn.argtypes = argtypes

@@ -193,6 +193,7 @@ def _flash_attn_backward(
     _launch_bwd_preprocess(ok, gk, delta)
     mask_ptr = mask.data_ptr() if mask is not None else None
     wq, wk, wv = work
+    ds_ws = plan.attach_ds_workspace(nheads, dp, seqlen_k) if plan is not None else None  # noqa: F841 (kept alive)
     with torch.cuda.device(q.device):
         _bam_hip.call(
             "bam_bwd_dkdv_masked",
@@ -210,6 +211,8 @@ def _flash_attn_backward(
             batch, seqlen_q, seqlen_k, nheads, nheads_k, dp, float(softmax_scale), _dtype_code(q.dtype), 0,
             _bias_arg(bias_view), _plan_arg(plan), _stream_ptr(q.device),
         )
+    if plan is not None:
+        plan.detach_ds_workspace()
     if not direct:
         for dst, w in zip(outs, work):
             dst.copy_(w[..., :d])

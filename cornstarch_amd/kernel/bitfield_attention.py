@@ -11,6 +11,7 @@ live on the GPU and the HIP library must be built.
 from __future__ import annotations
 
 import math
+import os
 from typing import Optional
 
 import torch
@@ -70,6 +71,34 @@ def materialize_bitfield_mask(bitfield_mask: torch.Tensor) -> torch.Tensor:
     return out.bool()
 
 
+# Largest dS workspace the backward allocates for the hand-over of dS from the dK/dV kernel to the dQ kernel; beyond it
+# the dQ kernel recomputes S and dP instead.  BAM_DS_WORKSPACE_LIMIT_GB overrides the default (a quarter of the
+# device's memory, at most 64 GiB); 0 switches the hand-over off.
+_DS_LIMIT_ENV = os.environ.get("BAM_DS_WORKSPACE_LIMIT_GB")
+
+
+def _ds_workspace_limit(device) -> int:
+    if _DS_LIMIT_ENV is not None:
+        return int(float(_DS_LIMIT_ENV) * (1 << 30))
+    return min(64 << 30, torch.cuda.get_device_properties(device).total_memory // 4)
+
+
+class _PinnedInts:
+    """A small pool of pinned host ints for asynchronous device-to-host copies of single counters."""
+
+    _buf: Optional[torch.Tensor] = None
+    _next = 0
+    _SLOTS = 256
+
+    @classmethod
+    def slot(cls) -> torch.Tensor:
+        if cls._buf is None:
+            cls._buf = torch.empty((cls._SLOTS,), dtype=torch.int32, pin_memory=True)
+        i = cls._next
+        cls._next = (i + 1) % cls._SLOTS
+        return cls._buf[i : i + 1]
+
+
 class _TilePlan:
     """What the kernels use beyond the 128 x 32 flags to skip masked work (``bam_plan`` of include/bam_hip.h):
     the class of every 32-row x 32-key tile and an order of the 32-row slices in which neighbours need the same
@@ -79,6 +108,41 @@ class _TilePlan:
         self.workspace = workspace  # keeps the device memory alive
         self.struct = struct
         self.flags = flags  # None for plans that are not tied to a flags tensor (index-tensor attention)
+        # The number of (slice, 128-key tile) pairs that have work is device data; it sizes the dS workspace of the
+        # backward.  Its copy to the host is enqueued here, right behind the kernels that compute it, and awaited
+        # only when a backward asks for it -- by then it has long arrived.
+        self._pairs: Optional[int] = None
+        self._pairs_host = _PinnedInts.slot()
+        count = torch.as_strided(workspace.view(torch.int32), (1,), (1,), (struct.ds_count - workspace.data_ptr()) // 4)
+        self._pairs_host.copy_(count, non_blocking=True)
+        self._pairs_event = torch.cuda.Event()
+        self._pairs_event.record(torch.cuda.current_stream(workspace.device))
+
+    def ds_pairs(self) -> int:
+        """How many (32-row slice, 128-key tile) pairs have work (waits for the asynchronous copy on first use)."""
+        if self._pairs is None:
+            self._pairs_event.synchronize()
+            self._pairs = int(self._pairs_host[0])
+        return self._pairs
+
+    def attach_ds_workspace(self, nheads: int, head_dim: int, seqlen_k: int) -> Optional[torch.Tensor]:
+        """Allocates the dS workspace of one backward call and names it in the plan struct; None (and nothing
+        attached) where the hand-over does not apply.  The caller detaches it after its launches."""
+        self.detach_ds_workspace()
+        if head_dim != 128 or seqlen_k > 131072:
+            return None
+        pairs = self.ds_pairs()
+        nbytes = _bam_hip.load().bam_ds_workspace_bytes(nheads, pairs)
+        if nbytes <= 0 or nbytes > _ds_workspace_limit(self.workspace.device) or nheads * pairs >= 1 << 31:
+            return None
+        ws = torch.empty((nbytes,), dtype=torch.uint8, device=self.workspace.device)
+        self.struct.ds_workspace = ws.data_ptr()
+        self.struct.ds_capacity = pairs
+        return ws
+
+    def detach_ds_workspace(self) -> None:
+        self.struct.ds_workspace = None
+        self.struct.ds_capacity = 0
 
     def byref(self):
         import ctypes
@@ -494,8 +558,13 @@ def _bitfield_attn_backward_overwrite(do, q, k, v, o, bitfield_mask, compressed_
     batch, seqlen_q, nheads, _ = q.shape
     bias_view = _BiasView(bias, q, batch, nheads, seqlen_q, k.shape[1], may_copy=False) if bias is not None else None
     _launch_bwd_preprocess(o, do, delta)
-    _launch_bwd_dkdv(q, k, v, do, lse, delta, dk, dv, bf, flags, softmax_scale, accumulate=False, bias=bias_view, plan=plan)
-    _launch_bwd_dq(q, k, v, do, lse, delta, dq, bf, flags, softmax_scale, accumulate=False, bias=bias_view, plan=plan)
+    ds_ws = plan.attach_ds_workspace(nheads, d, k.shape[1]) if plan is not None else None  # noqa: F841 (kept alive)
+    try:
+        _launch_bwd_dkdv(q, k, v, do, lse, delta, dk, dv, bf, flags, softmax_scale, accumulate=False, bias=bias_view, plan=plan)
+        _launch_bwd_dq(q, k, v, do, lse, delta, dq, bf, flags, softmax_scale, accumulate=False, bias=bias_view, plan=plan)
+    finally:
+        if plan is not None:
+            plan.detach_ds_workspace()
     return dq, dk, dv
 
 
@@ -556,8 +625,14 @@ def _bitfield_attn_backward(
     delta = torch.empty_like(lse)
     wq, wk, wv = work
     _launch_bwd_preprocess(ok, gk, delta)
-    _launch_bwd_dkdv(qk, kk, vk, gk, lse, delta, wk, wv, bf, flags, softmax_scale, bias=bias_view, plan=plan)
-    _launch_bwd_dq(qk, kk, vk, gk, lse, delta, wq, bf, flags, softmax_scale, bias=bias_view, plan=plan)
+    the_plan = plan if view is None else view.plan
+    ds_ws = the_plan.attach_ds_workspace(nheads, dp, seqlen_k) if the_plan is not None else None  # noqa: F841
+    try:
+        _launch_bwd_dkdv(qk, kk, vk, gk, lse, delta, wk, wv, bf, flags, softmax_scale, bias=bias_view, plan=plan)
+        _launch_bwd_dq(qk, kk, vk, gk, lse, delta, wq, bf, flags, softmax_scale, bias=bias_view, plan=plan)
+    finally:
+        if the_plan is not None:
+            the_plan.detach_ds_workspace()
     # the kernels accumulated into `work`; hand the sums back if those were copies
     for dst, mid, w in zip((dq, dk, dv), acc, work):
         if dp != d:

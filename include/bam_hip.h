@@ -92,6 +92,16 @@ typedef struct bam_bias {
  * the key tiles its own slice does not need; dK/dV walks the slices that have work for its keys, two at a time.
  * Results do not depend on whether a plan is given (same pairs, same arithmetic per pair; only the order in which
  * fp32 partial sums meet can differ in dK/dV).
+ *
+ * dS hand-over.  The reference's backward computes dS once per tile and adds dS k to dq with fp32 atomics
+ * (bitfield_attention.py:877-898); the atomic-free split used here (dK/dV kernel, dQ kernel) recomputes S and dP in
+ * the dQ kernel.  When the caller provides a workspace (plan->ds_workspace, plan->ds_capacity >= *plan->ds_count,
+ * head dim 128, at most 131072 keys), the dK/dV kernel also stores every 32 x 32 block of dS it computes
+ * (input dtype, as the reference rounds it, :877) and the dQ kernel becomes one GEMM over those blocks: 8 KiB per
+ * (q head, pair).  With bam_bwd both kernels run in that order; with the separate entry points bam_bwd_dkdv* must be
+ * called before bam_bwd_dq* with the same plan and workspace.  dq is then the sum of the very dS values that went
+ * into dk (instead of a recomputation that may differ in the last bit).  The count is device data: read it (for
+ * instance with an asynchronous copy enqueued right after the plan builder) before sizing the workspace.
  */
 typedef struct bam_plan {
     const uint8_t* fine;
@@ -99,6 +109,15 @@ typedef struct bam_plan {
     int64_t fine_stride_s;
     const int32_t* order;
     int64_t order_stride_b;
+    /* Hand-over of dS from the dK/dV kernel to the dQ kernel (see below).  ds_entry / ds_count are filled by the plan
+     * builders; ds_workspace / ds_capacity are the caller's to set before a backward call (null / 0 = not used). */
+    const int32_t* ds_entry;   /* device, (B, 4 * ceil(Sq/128), ceil(Sk/128)): number of each (slice, 128-key tile) pair
+                                  that has work, numbered in (batch, tile, slice) order; -1 = the pair has none */
+    int64_t ds_entry_stride_b;
+    const int32_t* ds_tile_base; /* device, (B, ceil(Sk/128)): number of the first pair of each key tile */
+    const int32_t* ds_count;   /* device, one int: how many such pairs there are */
+    void* ds_workspace;        /* device, at least bam_ds_workspace_bytes(Hq, pairs) bytes, 16-byte aligned */
+    int64_t ds_capacity;       /* pairs the workspace has room for: at least *ds_count */
     int32_t B;
     int32_t Sq;         /* query rows and keys the plan was built for (equal for plain bitfield attention) */
     int32_t Sk;
@@ -158,6 +177,9 @@ int bam_tile_plan_static(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, 
  * (shardformer/layers/utils.py:331-353); with this plan a shard skips masked work at 32-row granularity like the
  * unsharded path.  The flags the caller passes to the attention entry points are then not consulted.
  */
+/* Bytes of a dS workspace for Hq query heads and `pairs` (slice, 128-key tile) pairs. */
+int64_t bam_ds_workspace_bytes(int Hq, int64_t pairs);
+
 int bam_plan_indexed(const bam_index_view* iv, void* workspace, int64_t workspace_bytes, int B, bam_plan* plan,
                      void* stream);
 

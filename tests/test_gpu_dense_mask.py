@@ -176,7 +176,9 @@ def test_mask_plan_classes_and_results_do_not_depend_on_the_plan(Sq, Sk, D, monk
     monkeypatch.setattr(A._MaskPlan, "get", classmethod(lambda cls, *a: (real_get(cls, *a)[0], None)))
     without = run()
     for name, a, b in zip(("o", "lse", "dq", "dk", "dv"), with_plan, without):
-        if name in ("dk", "dv"):  # fp32 partial sums of the two row streams meet in another order
+        # dk, dv: fp32 partial sums of the two row streams meet in another order.  dq at head dim 128: with a plan
+        # the backward hands dS from dK/dV to the dQ kernel, without one dQ recomputes it.
+        if name in ("dk", "dv") or (name == "dq" and D == 128):
             assert rel_l2(a.float(), b.float()) <= 2e-3, name
         else:
             assert torch.equal(a, b), name

@@ -1,0 +1,181 @@
+"""The backward that hands dS from the dK/dV kernel to the dQ kernel through a workspace (head dim 128) against the
+backward that recomputes S and dP for dQ: same dk / dv bit for bit, dq to rounding (both sum the same rounded dS
+values, in another order), both within the gradient bar of the fp32 oracle.  The reference computes dS once per tile
+as well (bitfield_attention.py:877-898) and adds ds k to dq with atomics; here the sum has one owner per row."""
+
+import math
+
+import pytest
+import torch
+
+from cornstarch_amd.kernel import attention as A
+from cornstarch_amd.kernel import bitfield_attention as BA
+from oracle import bam_oracle as O
+from tests.helpers import random_bitfield, rel_l2
+
+pytestmark = pytest.mark.gpu
+
+GRAD_REL_L2 = 5e-2
+
+
+def dev():
+    return torch.device("cuda:0")
+
+
+def inputs(B, S, Hq, Hkv, D, dtype, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    q = (torch.randn(B, S, Hq, D, generator=g) * 0.5).to(dtype)
+    k = (torch.randn(B, S, Hkv, D, generator=g) * 0.5).to(dtype)
+    v = (torch.randn(B, S, Hkv, D, generator=g) * 0.5).to(dtype)
+    do = torch.randn(B, S, Hq, D, generator=g).to(dtype)
+    return q, k, v, do
+
+
+def build(bf):
+    BA.BitfieldUtils.clear_cache()
+    flags = BA.BitfieldUtils.materialize_compressed_mask_from_bitfield_mask(bf)
+    plan = BA.BitfieldUtils.plan_for(flags, bf)
+    assert plan is not None
+    return flags, plan
+
+
+@pytest.mark.parametrize("S", [1, 57, 283, 1000])
+def test_pair_numbering_against_the_fine_classes(S):
+    bf = random_bitfield(3, S, seed=S, pad=min(5, S - 1)).to(dev())
+    flags, plan = build(bf)
+    st, ws = plan.struct, plan.workspace
+    slots, nkt, num_n = 4 * flags.shape[1], -(-S // 128), -(-S // 32)
+    fine = torch.nn.functional.pad(plan.fine_classes().cpu(), (0, 4 * nkt - num_n))
+    has = (fine.view(3, slots, nkt, 4) != 0).any(dim=3)                          # (B, slots, nkt)
+    i32 = ws.view(torch.int32)
+    entry = torch.as_strided(i32, (3, slots, nkt), (st.ds_entry_stride_b, nkt, 1), (st.ds_entry - ws.data_ptr()) // 4).cpu()
+    base = torch.as_strided(i32, (3, nkt), (nkt, 1), (st.ds_tile_base - ws.data_ptr()) // 4).cpu()
+    # numbered in (batch, tile, slice) order
+    order = has.permute(0, 2, 1).reshape(-1)
+    numbers = torch.cumsum(order.to(torch.int64), 0) - 1
+    want = torch.where(order, numbers, torch.full_like(numbers, -1)).view(3, nkt, slots).permute(0, 2, 1)
+    assert torch.equal(entry.to(torch.int64), want)
+    first = (torch.cumsum(order.to(torch.int64), 0) - order.to(torch.int64)).view(3, nkt, slots)[:, :, 0]
+    assert torch.equal(base.to(torch.int64), first)
+    assert plan.ds_pairs() == int(has.sum())
+    BA.BitfieldUtils.clear_cache()
+
+
+def run_backward(q, k, v, do, bf, handover, monkeypatch, accumulate=False):
+    monkeypatch.setattr(BA, "_ds_workspace_limit", (lambda device: 1 << 40) if handover else (lambda device: 0))
+    flags, plan = build(bf)
+    o, lse, scale = BA._bitfield_attn_forward(q, k, v, bf, flags)
+    if accumulate:
+        grads = [torch.zeros_like(t, dtype=torch.float32) for t in (q, k, v)]
+        BA._bitfield_attn_backward(do, q, k, v, o, bf, flags, lse, *grads, softmax_scale=scale)
+    else:
+        grads = BA._bitfield_attn_backward_overwrite(do, q, k, v, o, bf, flags, lse, scale)
+    torch.cuda.synchronize()
+    assert plan.struct.ds_workspace is None  # detached after the launches
+    return [g.clone() for g in grads]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,S,Hq,Hkv", [(2, 57, 2, 1), (1, 283, 4, 4), (2, 517, 4, 2), (1, 1000, 8, 2), (1, 2048, 4, 1)])
+@pytest.mark.parametrize("accumulate", [False, True], ids=["typed", "fp32"])
+def test_handover_equals_recomputation(dtype, B, S, Hq, Hkv, accumulate, monkeypatch):
+    d = dev()
+    bf = random_bitfield(B, S, seed=S, pad=3).to(d)
+    q, k, v, do = (t.to(d) for t in inputs(B, S, Hq, Hkv, 128, dtype, seed=S))
+    with_ds = run_backward(q, k, v, do, bf, True, monkeypatch, accumulate)
+    recomputed = run_backward(q, k, v, do, bf, False, monkeypatch, accumulate)
+    assert torch.equal(with_ds[1], recomputed[1]) and torch.equal(with_ds[2], recomputed[2])  # dk, dv: same kernel
+    assert rel_l2(with_ds[0].float(), recomputed[0].float()) <= 2e-3
+    again = run_backward(q, k, v, do, bf, True, monkeypatch, accumulate)
+    assert all(torch.equal(a, b) for a, b in zip(with_ds, again))                            # no atomics: reruns agree
+    for got, want in zip(with_ds, O.attention_backward(q, k, v, bf, do)):
+        assert torch.isfinite(got).all() and rel_l2(got.float(), want) <= GRAD_REL_L2
+    BA.BitfieldUtils.clear_cache()
+
+
+def test_every_block_the_dq_kernel_reads_was_written(monkeypatch):
+    # the workspace starts as NaN bit patterns: a block read but never written would show up in dq
+    d = dev()
+    B, S, Hq, Hkv = 2, 777, 4, 2
+    bf = random_bitfield(B, S, seed=12, pad=9).to(d)
+    q, k, v, do = (t.to(d) for t in inputs(B, S, Hq, Hkv, 128, torch.bfloat16, seed=5))
+    flags, plan = build(bf)
+    o, lse, scale = BA._bitfield_attn_forward(q, k, v, bf, flags)
+    delta = torch.empty_like(lse)
+    BA._launch_bwd_preprocess(o, do, delta)
+    ws = plan.attach_ds_workspace(Hq, 128, S)
+    assert ws is not None and ws.numel() == plan.ds_pairs() * Hq * 8192
+    ws.fill_(0xFF)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    BA._launch_bwd_dkdv(q, k, v, do, lse, delta, dk, dv, bf, flags, scale, accumulate=False, plan=plan)
+    BA._launch_bwd_dq(q, k, v, do, lse, delta, dq, bf, flags, scale, accumulate=False, plan=plan)
+    plan.detach_ds_workspace()
+    torch.cuda.synchronize()
+    assert torch.isfinite(dq).all()
+    dq2 = torch.empty_like(q)
+    BA._launch_bwd_dq(q, k, v, do, lse, delta, dq2, bf, flags, scale, accumulate=False, plan=plan)  # recomputing kernel
+    assert rel_l2(dq.float(), dq2.float()) <= 2e-3
+    BA.BitfieldUtils.clear_cache()
+
+
+def test_handover_with_index_tensors_dense_masks_and_bias(monkeypatch):
+    d = dev()
+    B, S, Hq, Hkv = 2, 640, 4, 2
+    bf_cpu = random_bitfield(B, S, seed=3, pad=4)
+    q, k, v, do = inputs(B, S, Hq, Hkv, 128, torch.bfloat16, seed=9)
+
+    # index tensors: one zigzag "rank" (rows of chunks 0 and 3 of 4, keys of all chunks rank by rank)
+    chunks = torch.arange(S).chunk(4)
+    idx_q = torch.cat([chunks[0], chunks[3]])
+    idx_k = torch.cat([chunks[0], chunks[3], chunks[1], chunks[2]])
+    flags = O.tile_flags_indexed(bf_cpu, idx_q, idx_k).to(d)
+    results = []
+    for handover in (True, False):
+        monkeypatch.setattr(BA, "_ds_workspace_limit", (lambda device: 1 << 40) if handover else (lambda device: 0))
+        BA.BitfieldUtils.clear_cache()
+        ql, dol = q[:, idx_q].contiguous().to(d), do[:, idx_q].contiguous().to(d)
+        kl, vl = k[:, idx_k].contiguous().to(d), v[:, idx_k].contiguous().to(d)
+        bfg, oq, ok = bf_cpu.to(d), idx_q.to(d), idx_k.to(d)
+        o, lse, scale = BA._bitfield_attn_forward(ql, kl, vl, bfg, flags, oq, ok)
+        grads = [torch.zeros_like(t, dtype=torch.float32) for t in (ql, kl, vl)]
+        BA._bitfield_attn_backward(dol, ql, kl, vl, o, bfg, flags, lse, *grads, offsets_q=oq, offsets_k=ok, softmax_scale=scale)
+        torch.cuda.synchronize()
+        results.append(grads)
+    assert torch.equal(results[0][1], results[1][1]) and torch.equal(results[0][2], results[1][2])
+    assert rel_l2(results[0][0], results[1][0]) <= 2e-3
+    want = O.attention_backward(q[:, idx_q], k[:, idx_k], v[:, idx_k], bf_cpu, do[:, idx_q], idx_q=idx_q, idx_k=idx_k)
+    for got, w in zip(results[0], want):
+        assert rel_l2(got.cpu(), w) <= GRAD_REL_L2
+
+    # a materialized mask plus an ALiBi-like bias vector
+    mask = O.materialize_mask(bf_cpu).to(d)
+    bias = (-(torch.arange(S, dtype=torch.float32)[None, None, None, :]) * torch.tensor([0.01, 0.02, 0.04, 0.08])[None, :, None, None]).to(d)
+    qd, kd, vd, dod = (t.to(d) for t in (q, k, v, do))
+    results = []
+    for handover in (True, False):
+        monkeypatch.setattr(BA, "_ds_workspace_limit", (lambda device: 1 << 40) if handover else (lambda device: 0))
+        A._MaskPlan.forget()
+        o, lse, scale = A._flash_attn_forward(qd, kd, vd, bias=bias, mask=mask)
+        grads = [torch.empty_like(t) for t in (qd, kd, vd)]
+        A._flash_attn_backward(dod, qd, kd, vd, o, lse, *grads, bias=bias, mask=mask, softmax_scale=scale)
+        torch.cuda.synchronize()
+        results.append(grads)
+    assert torch.equal(results[0][1], results[1][1]) and torch.equal(results[0][2], results[1][2])
+    assert rel_l2(results[0][0].float(), results[1][0].float()) <= 2e-3
+    want = O.masked_attention_backward(q, k, v, mask.cpu(), do, bias=bias.cpu())
+    for got, w in zip(results[0], want):
+        assert rel_l2(got.float().cpu(), w) <= GRAD_REL_L2
+    A._MaskPlan.forget()
+    BA.BitfieldUtils.clear_cache()
+
+
+def test_head_dim_64_and_a_zero_limit_keep_the_recomputing_backward():
+    d = dev()
+    bf = random_bitfield(1, 300, seed=1).to(d)
+    flags, plan = build(bf)
+    assert plan.attach_ds_workspace(4, 64, 300) is None and plan.struct.ds_workspace is None
+    ws = plan.attach_ds_workspace(4, 128, 300)
+    assert ws is not None and plan.struct.ds_workspace == ws.data_ptr() and plan.struct.ds_capacity == plan.ds_pairs()
+    plan.detach_ds_workspace()
+    assert plan.struct.ds_workspace is None and plan.struct.ds_capacity == 0
+    BA.BitfieldUtils.clear_cache()

@@ -208,7 +208,9 @@ def test_shard_results_do_not_depend_on_the_plan(kind, S, D, Hq, Hkv):
         without = _rank_with_and_without_plan(q, k, v, do, bf, idx_q, idx_k, flags, False)
         with_plan = _rank_with_and_without_plan(q, k, v, do, bf, idx_q, idx_k, flags, True)
         for name, a, b in zip(("o", "lse", "dq", "dk", "dv"), with_plan, without):
-            if name in ("dk", "dv"):  # fp32 partial sums of the two row streams meet in another order
+            # dk, dv: fp32 partial sums of the two row streams meet in another order.  dq at head dim 128: with a
+            # plan the backward hands dS from dK/dV to the dQ kernel, without one dQ recomputes it.
+            if name in ("dk", "dv") or (name == "dq" and D == 128):
                 assert rel_l2(a, b) <= 2e-3, name
             else:
                 assert torch.equal(a, b), name

@@ -40,7 +40,8 @@ def test_library_exports_every_declared_symbol():
     assert _bam_hip.load().bam_abi_version() == _bam_hip.ABI_VERSION
     # the binding's prototypes cover every compute entry point of the header
     assert set(_bam_hip.SIGNATURES) == set(names) - {
-        "bam_last_error", "bam_abi_version", "bam_plan_workspace_bytes", "bam_plan_workspace_bytes_rect"}
+        "bam_last_error", "bam_abi_version", "bam_plan_workspace_bytes", "bam_plan_workspace_bytes_rect",
+        "bam_ds_workspace_bytes"}
     # plan workspace: sized without a GPU; no plan beyond 4096 row slices
     lib2 = _bam_hip.load()
     assert lib2.bam_plan_workspace_bytes(1, 8192) >= 256 * 256 + 256 * 4 and lib2.bam_plan_workspace_bytes(1, 8192) % 256 == 0
