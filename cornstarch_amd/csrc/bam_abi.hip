@@ -373,7 +373,8 @@ int place_plan(const char* who, void* workspace, int64_t workspace_bytes, int B,
 // second launch of every plan builder: numbers the (slice, 128-key tile) pairs that have work
 int number_pairs(const char* who, const bam_plan* plan, void* stream) {
     return launched(bam::launch_ds_entries(plan->fine, plan->fine_stride_b, plan->fine_stride_s, plan->B, plan->Sq, plan->Sk,
-                                           const_cast<int*>(plan->ds_entry), const_cast<int*>(plan->ds_tile_base),
+                                           const_cast<int*>(plan->ds_entry), plan->ds_entry_stride_b,
+                                           const_cast<int*>(plan->ds_tile_base),
                                            const_cast<int*>(plan->ds_count),
                                            (hipStream_t)stream),
                     who);
@@ -392,8 +393,8 @@ int bam_tile_plan(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int64_t
     BAM_TRY(place_plan("bam_tile_plan", workspace, workspace_bytes, B, S, S, plan, l));
     char* w = (char*)workspace;
     BAM_TRY(launched(bam::launch_tile_plan(bf, bf_stride_b, flags, flags_stride_b, flags_stride_m, (uint8_t*)(w + l.fine_off),
-                                           l.fine_sb, l.fine_ss, (int*)(w + l.order_off), l.order_sb, B, S,
-                                           (hipStream_t)stream),
+                                           l.fine_sb, l.fine_ss, (int*)(w + l.order_off), l.order_sb,
+                                           (int*)(w + l.count_off), B, S, (hipStream_t)stream),
                      "bam_tile_plan"));
     return number_pairs("bam_tile_plan", plan, stream);
 }
@@ -436,7 +437,7 @@ int bam_plan_indexed(const bam_index_view* iv, void* workspace, int64_t workspac
     char* w = (char*)workspace;
     BAM_TRY(launched(bam::launch_indexed_plan(m.bfq, m.bfq_sb, m.bfk, m.bfk_sb, m.posq, m.posk, m.Sq, m.Sk,
                                               (uint8_t*)(w + l.fine_off), l.fine_sb, l.fine_ss, (int*)(w + l.order_off),
-                                              l.order_sb, B, (hipStream_t)stream),
+                                              l.order_sb, (int*)(w + l.count_off), B, (hipStream_t)stream),
                      "bam_plan_indexed"));
     return number_pairs("bam_plan_indexed", plan, stream);
 }
@@ -451,8 +452,8 @@ int bam_mask_tile_plan(const uint8_t* mask, int8_t* flags, int64_t flags_stride_
     BAM_TRY(place_plan("bam_mask_tile_plan", workspace, workspace_bytes, B, Sq, Sk, plan, l));
     char* w = (char*)workspace;
     BAM_TRY(launched(bam::launch_mask_tile_plan(mask, flags, flags_stride_b, flags_stride_m, (uint8_t*)(w + l.fine_off),
-                                                l.fine_sb, l.fine_ss, (int*)(w + l.order_off), l.order_sb, B, Sq, Sk,
-                                                (hipStream_t)stream),
+                                                l.fine_sb, l.fine_ss, (int*)(w + l.order_off), l.order_sb,
+                                                (int*)(w + l.count_off), B, Sq, Sk, (hipStream_t)stream),
                      "bam_mask_tile_plan"));
     return number_pairs("bam_mask_tile_plan", plan, stream);
 }

@@ -86,9 +86,10 @@ struct DecodeParams {
 int launch_tile_flags(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int64_t flags_stride_b,
                       int64_t flags_stride_m, int B, int S, hipStream_t stream);
 // Flags plus plan in one launch: fine (B, 4 * num_m, fine_ss) bytes, order (B, 4 * num_m) ints.
+// (pair_count: the counter launch_ds_entries adds to, reset here)
 int launch_tile_plan(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int64_t flags_stride_b,
                      int64_t flags_stride_m, uint8_t* fine, int64_t fine_sb, int64_t fine_ss, int* order,
-                     int64_t order_sb, int B, int S, hipStream_t stream);
+                     int64_t order_sb, int* pair_count, int B, int S, hipStream_t stream);
 int launch_materialize_mask(const int64_t* bf, int64_t bf_stride_b, uint8_t* out, int B, int S,
                             hipStream_t stream);
 int launch_flag_row_workloads(const int8_t* flags, int64_t flags_stride_b, int64_t flags_stride_m, int B, int num_m,
@@ -100,15 +101,16 @@ int launch_gather_bitfields(const int64_t* bf, int64_t bf_stride_b, int L, const
 // Plan (fine classes + slice order) of index-tensor attention, from the gathered bitfields and positions.
 int launch_indexed_plan(const int64_t* qbits, int64_t qbits_sb, const int64_t* kbits, int64_t kbits_sb, const int* qpos,
                         const int* kpos, int Sq, int Sk, uint8_t* fine, int64_t fine_sb, int64_t fine_ss, int* order,
-                        int64_t order_sb, int B, hipStream_t stream);
+                        int64_t order_sb, int* pair_count, int B, hipStream_t stream);
 // Flags plus plan of a materialized bool mask.
 int launch_mask_tile_plan(const uint8_t* mask, int8_t* flags, int64_t flags_stride_b, int64_t flags_stride_m,
-                          uint8_t* fine, int64_t fine_sb, int64_t fine_ss, int* order, int64_t order_sb, int B, int Sq,
-                          int Sk, hipStream_t stream);
+                          uint8_t* fine, int64_t fine_sb, int64_t fine_ss, int* order, int64_t order_sb, int* pair_count,
+                          int B, int Sq, int Sk, hipStream_t stream);
 // Numbers the (slice, 128-key tile) pairs that have work: entry (B, 4 * num_m, ceil(Sk/128)) ints, -1 = none.
 // tile_base (B, ceil(Sk/128)) ints: number of the first pair of each key tile (pairs are numbered tile by tile).
+// *count must be zero when the kernel starts (the plan kernels reset it).
 int launch_ds_entries(const uint8_t* fine, int64_t fine_sb, int64_t fine_ss, int B, int Sq, int Sk, int* entry,
-                      int* tile_base, int* count, hipStream_t stream);
+                      int64_t entry_sb, int* tile_base, int* count, hipStream_t stream);
 int launch_fwd(const AttnParams& p, int dtype, hipStream_t stream);
 int launch_bwd_preprocess(const AttnParams& p, int dtype, hipStream_t stream);
 int launch_bwd_dkdv(const AttnParams& p, int dtype, hipStream_t stream);

@@ -122,7 +122,11 @@ __global__ __launch_bounds__(FLAG_WAVES * 64) void tile_flags_kernel(const int64
                                                                     int64_t flags_stride_m, int S, int num_n,
                                                                     uint8_t* __restrict__ fine, int64_t fine_sb,
                                                                     int64_t fine_ss, int* __restrict__ order,
-                                                                    int64_t order_sb, int flag_blocks_x) {
+                                                                    int64_t order_sb, int flag_blocks_x,
+                                                                    int* __restrict__ pair_count) {
+    // (the pair counter of the numbering kernel that follows in the stream starts from zero)
+    if (FINE && pair_count != nullptr && blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0 && threadIdx.x == 0)
+        *pair_count = 0;
     if (FINE && (int)blockIdx.x >= flag_blocks_x) {  // the workgroups that sort the slices (see slice_order_part)
         const int part = blockIdx.y;
         if (part * 256 < 4 * (int)gridDim.y)
@@ -333,9 +337,11 @@ int launch_flag_row_workloads(const int8_t* flags, int64_t flags_stride_b, int64
 __global__ __launch_bounds__(FLAG_WAVES * 64) void indexed_plan_kernel(
     const int64_t* __restrict__ qbits, int64_t qbits_sb, const int64_t* __restrict__ kbits, int64_t kbits_sb,
     const int* __restrict__ qpos, const int* __restrict__ kpos, int Sq, int Sk, int num_n, uint8_t* __restrict__ fine,
-    int64_t fine_sb, int64_t fine_ss, int* __restrict__ order, int64_t order_sb, int flag_blocks_x) {
+    int64_t fine_sb, int64_t fine_ss, int* __restrict__ order, int64_t order_sb, int flag_blocks_x,
+    int* __restrict__ pair_count) {
     const int b = blockIdx.z;
     const int64_t* qrow = qbits + (int64_t)b * qbits_sb;
+    if (pair_count != nullptr && blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0 && threadIdx.x == 0) *pair_count = 0;
     if ((int)blockIdx.x >= flag_blocks_x) {
         const int part = blockIdx.y;
         const int ns = (Sq + 31) / 32, slots = 4 * (int)gridDim.y;
@@ -399,12 +405,12 @@ __global__ __launch_bounds__(FLAG_WAVES * 64) void indexed_plan_kernel(
 
 int launch_indexed_plan(const int64_t* qbits, int64_t qbits_sb, const int64_t* kbits, int64_t kbits_sb, const int* qpos,
                         const int* kpos, int Sq, int Sk, uint8_t* fine, int64_t fine_sb, int64_t fine_ss, int* order,
-                        int64_t order_sb, int B, hipStream_t stream) {
+                        int64_t order_sb, int* pair_count, int B, hipStream_t stream) {
     const int num_m = (Sq + BLOCK_M - 1) / BLOCK_M, num_n = (Sk + BLOCK_N - 1) / BLOCK_N;
     const int flag_blocks_x = (num_n + FLAG_COLS_PER_BLOCK - 1) / FLAG_COLS_PER_BLOCK;
     dim3 grid(flag_blocks_x + 1, num_m, B);
     hipLaunchKernelGGL(indexed_plan_kernel, grid, dim3(FLAG_WAVES * 64), 0, stream, qbits, qbits_sb, kbits, kbits_sb, qpos,
-                       kpos, Sq, Sk, num_n, fine, fine_sb, fine_ss, order, order_sb, flag_blocks_x);
+                       kpos, Sq, Sk, num_n, fine, fine_sb, fine_ss, order, order_sb, flag_blocks_x, pair_count);
     return (int)hipGetLastError();
 }
 
@@ -416,8 +422,9 @@ __global__ __launch_bounds__(256) void mask_tile_plan_kernel(const uint8_t* __re
                                                              int64_t flags_stride_b, int64_t flags_stride_m, int Sq,
                                                              int Sk, int num_n, uint8_t* __restrict__ fine,
                                                              int64_t fine_sb, int64_t fine_ss, int* __restrict__ order,
-                                                             int64_t order_sb) {
+                                                             int64_t order_sb, int* __restrict__ pair_count) {
     const int b = blockIdx.z, m = blockIdx.y, tid = threadIdx.x;
+    if (pair_count != nullptr && blockIdx.x == 0 && m == 0 && b == 0 && tid == 0) *pair_count = 0;
     if (blockIdx.x == 0 && tid < 4) {
         const int ns = (Sq + 31) / 32, slot = 4 * m + tid;
         order[(int64_t)b * order_sb + slot] = slot < ns ? ns - 1 - slot : -1;
@@ -455,73 +462,77 @@ __global__ __launch_bounds__(256) void mask_tile_plan_kernel(const uint8_t* __re
 }
 
 int launch_mask_tile_plan(const uint8_t* mask, int8_t* flags, int64_t flags_stride_b, int64_t flags_stride_m,
-                          uint8_t* fine, int64_t fine_sb, int64_t fine_ss, int* order, int64_t order_sb, int B, int Sq,
-                          int Sk, hipStream_t stream) {
+                          uint8_t* fine, int64_t fine_sb, int64_t fine_ss, int* order, int64_t order_sb, int* pair_count,
+                          int B, int Sq, int Sk, hipStream_t stream) {
     const int num_m = (Sq + BLOCK_M - 1) / BLOCK_M, num_n = (Sk + BLOCK_N - 1) / BLOCK_N;
     dim3 grid((num_n + 7) / 8, num_m, B);
     hipLaunchKernelGGL(mask_tile_plan_kernel, grid, dim3(256), 0, stream, mask, flags, flags_stride_b, flags_stride_m, Sq,
-                       Sk, num_n, fine, fine_sb, fine_ss, order, order_sb);
+                       Sk, num_n, fine, fine_sb, fine_ss, order, order_sb, pair_count);
     return (int)hipGetLastError();
 }
 
 // Numbering of the (32-row slice, 128-key tile) pairs that have work, for the backward that hands dS from the dK/dV
-// kernel to the dQ kernel through memory.  Pairs are numbered in (batch, tile, slice) order, so the slices that have
-// work for one key tile -- exactly the list a dK/dV workgroup builds -- carry consecutive numbers:
+// kernel to the dQ kernel through memory.  The pairs of one key tile -- exactly the slices a dK/dV workgroup lists --
+// get consecutive numbers, by ascending slice; the tiles themselves take their blocks of numbers in the order their
+// workgroups arrive (one atomic add per tile on *count, which the plan kernels reset):
 //   entry[b][s][t]  = number of pair (b, s, t), or -1 where its four classes are all "empty"  (what the dQ kernel looks up)
 //   tile_base[b][t] = number of the first pair of key tile (b, t)                             (what dK/dV starts from)
 //   *count          = how many pairs there are.
-// One workgroup: every thread counts a contiguous run of pairs, the counts are scanned, the run is numbered.
-constexpr int DS_SCAN_THREADS = 1024;
-__global__ __launch_bounds__(DS_SCAN_THREADS) void ds_entries_kernel(const uint8_t* __restrict__ fine, int64_t fine_sb,
-                                                                    int64_t fine_ss, int B, int slots, int nkt, int num_n,
-                                                                    int* __restrict__ entry, int* __restrict__ tile_base,
-                                                                    int* __restrict__ count) {
-    __shared__ int wave_total[DS_SCAN_THREADS / 64];
+// Which tile gets which block of numbers only decides where a record sits in the workspace, never a result.
+// One workgroup per (key tile, batch); thread = slice, 256 slices per sweep.
+constexpr int DS_NUM_THREADS = 256;
+__global__ __launch_bounds__(DS_NUM_THREADS) void ds_entries_kernel(const uint8_t* __restrict__ fine, int64_t fine_sb,
+                                                                   int64_t fine_ss, int slots, int nkt, int num_n,
+                                                                   int* __restrict__ entry, int64_t entry_sb,
+                                                                   int* __restrict__ tile_base, int* __restrict__ count) {
+    __shared__ int wave_sum[DS_NUM_THREADS / 64];
+    __shared__ int s_base;
+    const int t = blockIdx.x, b = blockIdx.y;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int64_t total = (int64_t)B * slots * nkt;
-    const int64_t per = (total + DS_SCAN_THREADS - 1) / DS_SCAN_THREADS;
-    const int64_t first = min(total, per * tid), last = min(total, first + per);
-    // position i of the scan = (b * nkt + t) * slots + s
-    auto has_work = [&](int64_t i) {
-        const int sl = (int)(i % slots);
-        const int64_t bt = i / slots;
-        const int t = (int)(bt % nkt);
-        const uint8_t* f = fine + (bt / nkt) * fine_sb + (int64_t)sl * fine_ss + 4 * t;
-        bool any = false;
+    const uint8_t* col = fine + (int64_t)b * fine_sb + 4 * t;
+    unsigned valid = 0;  // which of the tile's four 32-key columns exist
 #pragma unroll
-        for (int w = 0; w < 4; ++w) any |= (4 * t + w < num_n) && f[w] != 0;
-        return any;
-    };
+    for (int w = 0; w < 4; ++w)
+        if (4 * t + w < num_n) valid |= 0xFFu << (8 * w);
+    auto has_work = [&](int sl) { return sl < slots && (*(const unsigned*)(col + (int64_t)sl * fine_ss) & valid) != 0; };
     int mine = 0;
-    for (int64_t i = first; i < last; ++i) mine += has_work(i) ? 1 : 0;
-    int incl = mine;  // inclusive scan inside the wave
+    for (int sl = tid; sl < slots; sl += DS_NUM_THREADS) mine += has_work(sl) ? 1 : 0;
 #pragma unroll
-    for (int off = 1; off < 64; off <<= 1) {
-        const int up = __shfl_up(incl, off);
-        if (lane >= off) incl += up;
-    }
-    if (lane == 63) wave_total[wave] = incl;
+    for (int off = 32; off > 0; off >>= 1) mine += __shfl_xor(mine, off);
+    if (lane == 0) wave_sum[wave] = mine;
     __syncthreads();
-    int base = 0, all = 0;
-    for (int w = 0; w < DS_SCAN_THREADS / 64; ++w) {
-        if (w < wave) base += wave_total[w];
-        all += wave_total[w];
+    if (tid == 0) {
+        int total = 0;
+        for (int w = 0; w < DS_NUM_THREADS / 64; ++w) total += wave_sum[w];
+        const int base = atomicAdd(count, total);
+        s_base = base;
+        tile_base[(int64_t)b * nkt + t] = base;
     }
-    int next = base + incl - mine;
-    for (int64_t i = first; i < last; ++i) {
-        const int sl = (int)(i % slots);
-        const int64_t bt = i / slots;
-        if (sl == 0) tile_base[bt] = next;
-        entry[((bt / nkt) * slots + sl) * nkt + (bt % nkt)] = has_work(i) ? next++ : -1;
+    __syncthreads();
+    int next = s_base;
+    int* out = entry + (int64_t)b * entry_sb + t;
+    for (int s0 = 0; s0 < slots; s0 += DS_NUM_THREADS) {
+        const int sl = s0 + tid;
+        const bool h = has_work(sl);
+        const unsigned long long bal = __ballot(h);
+        __syncthreads();  // wave_sum is free again
+        if (lane == 0) wave_sum[wave] = __popcll(bal);
+        __syncthreads();
+        int before = 0, all = 0;
+        for (int w = 0; w < DS_NUM_THREADS / 64; ++w) {
+            if (w < wave) before += wave_sum[w];
+            all += wave_sum[w];
+        }
+        if (sl < slots) out[(int64_t)sl * nkt] = h ? next + before + __popcll(bal & ((1ull << lane) - 1ull)) : -1;
+        next += all;
     }
-    if (tid == 0) *count = all;
 }
 
 int launch_ds_entries(const uint8_t* fine, int64_t fine_sb, int64_t fine_ss, int B, int Sq, int Sk, int* entry,
-                      int* tile_base, int* count, hipStream_t stream) {
+                      int64_t entry_sb, int* tile_base, int* count, hipStream_t stream) {
     const int slots = 4 * ((Sq + BLOCK_M - 1) / BLOCK_M), nkt = (Sk + 127) / 128, num_n = (Sk + BLOCK_N - 1) / BLOCK_N;
-    hipLaunchKernelGGL(ds_entries_kernel, dim3(1), dim3(DS_SCAN_THREADS), 0, stream, fine, fine_sb, fine_ss, B, slots, nkt,
-                       num_n, entry, tile_base, count);
+    hipLaunchKernelGGL(ds_entries_kernel, dim3(nkt, B), dim3(DS_NUM_THREADS), 0, stream, fine, fine_sb, fine_ss, slots, nkt,
+                       num_n, entry, entry_sb, tile_base, count);
     return (int)hipGetLastError();
 }
 
@@ -531,20 +542,21 @@ int launch_tile_flags(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int
     dim3 grid((num_n + FLAG_COLS_PER_BLOCK - 1) / FLAG_COLS_PER_BLOCK, num_m, B);
     hipLaunchKernelGGL(tile_flags_kernel<false>, grid, dim3(FLAG_WAVES * 64), 0, stream, bf, bf_stride_b, flags,
                        flags_stride_b, flags_stride_m, S, num_n, (uint8_t*)nullptr, (int64_t)0, (int64_t)0, (int*)nullptr,
-                       (int64_t)0, 0);
+                       (int64_t)0, 0, (int*)nullptr);
     return (int)hipGetLastError();
 }
 
 int launch_tile_plan(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int64_t flags_stride_b,
                      int64_t flags_stride_m, uint8_t* fine, int64_t fine_sb, int64_t fine_ss, int* order,
-                     int64_t order_sb, int B, int S, hipStream_t stream) {
+                     int64_t order_sb, int* pair_count, int B, int S, hipStream_t stream) {
     const int num_m = (S + BLOCK_M - 1) / BLOCK_M, num_n = (S + BLOCK_N - 1) / BLOCK_N;
     const int flag_blocks_x = (num_n + FLAG_COLS_PER_BLOCK - 1) / FLAG_COLS_PER_BLOCK;
     // one more column of workgroups: (flag_blocks_x, part, b) ranks 256 slices; 4 num_m slots need
     // ceil(4 num_m / 256) <= num_m parts
     dim3 grid(flag_blocks_x + 1, num_m, B);
     hipLaunchKernelGGL(tile_flags_kernel<true>, grid, dim3(FLAG_WAVES * 64), 0, stream, bf, bf_stride_b, flags,
-                       flags_stride_b, flags_stride_m, S, num_n, fine, fine_sb, fine_ss, order, order_sb, flag_blocks_x);
+                       flags_stride_b, flags_stride_m, S, num_n, fine, fine_sb, fine_ss, order, order_sb, flag_blocks_x,
+                       pair_count);
     return (int)hipGetLastError();
 }
 

@@ -98,6 +98,17 @@ class _PinnedInts:
         cls._next = (i + 1) % cls._SLOTS
         return cls._buf[i : i + 1]
 
+    _streams: dict = {}
+
+    @classmethod
+    def copy_stream(cls, device) -> "torch.cuda.Stream":
+        """One side stream per device for these copies, so that they never sit between two kernels of the caller's
+        stream."""
+        key = torch.device(device).index if torch.device(device).index is not None else torch.cuda.current_device()
+        if key not in cls._streams:
+            cls._streams[key] = torch.cuda.Stream(device=device)
+        return cls._streams[key]
+
 
 class _TilePlan:
     """What the kernels use beyond the 128 x 32 flags to skip masked work (``bam_plan`` of include/bam_hip.h):
@@ -114,9 +125,16 @@ class _TilePlan:
         self._pairs: Optional[int] = None
         self._pairs_host = _PinnedInts.slot()
         count = torch.as_strided(workspace.view(torch.int32), (1,), (1,), (struct.ds_count - workspace.data_ptr()) // 4)
-        self._pairs_host.copy_(count, non_blocking=True)
+        main = torch.cuda.current_stream(workspace.device)
+        side = _PinnedInts.copy_stream(workspace.device)
+        built = torch.cuda.Event()
+        built.record(main)
+        side.wait_event(built)
+        with torch.cuda.stream(side):
+            self._pairs_host.copy_(count, non_blocking=True)
+        workspace.record_stream(side)
         self._pairs_event = torch.cuda.Event()
-        self._pairs_event.record(torch.cuda.current_stream(workspace.device))
+        self._pairs_event.record(side)
 
     def ds_pairs(self) -> int:
         """How many (32-row slice, 128-key tile) pairs have work (waits for the asynchronous copy on first use)."""

@@ -50,13 +50,21 @@ def test_pair_numbering_against_the_fine_classes(S):
     i32 = ws.view(torch.int32)
     entry = torch.as_strided(i32, (3, slots, nkt), (st.ds_entry_stride_b, nkt, 1), (st.ds_entry - ws.data_ptr()) // 4).cpu()
     base = torch.as_strided(i32, (3, nkt), (nkt, 1), (st.ds_tile_base - ws.data_ptr()) // 4).cpu()
-    # numbered in (batch, tile, slice) order
-    order = has.permute(0, 2, 1).reshape(-1)
-    numbers = torch.cumsum(order.to(torch.int64), 0) - 1
-    want = torch.where(order, numbers, torch.full_like(numbers, -1)).view(3, nkt, slots).permute(0, 2, 1)
-    assert torch.equal(entry.to(torch.int64), want)
-    first = (torch.cumsum(order.to(torch.int64), 0) - order.to(torch.int64)).view(3, nkt, slots)[:, :, 0]
-    assert torch.equal(base.to(torch.int64), first)
+    # the pairs of a key tile carry consecutive numbers from the tile's base, by ascending slice; the tiles' blocks of
+    # numbers tile [0, total) without gaps or overlaps (which tile gets which block is not specified)
+    blocks = []
+    for bb in range(3):
+        for t in range(nkt):
+            col = has[bb, :, t]
+            n_t = int(col.sum())
+            start = int(base[bb, t])
+            assert entry[bb, :, t][col].tolist() == list(range(start, start + n_t))
+            assert (entry[bb, :, t][~col] == -1).all()
+            if n_t:
+                blocks.append((start, n_t))
+    blocks.sort()
+    assert all(blocks[i][0] + blocks[i][1] == blocks[i + 1][0] for i in range(len(blocks) - 1))
+    assert not blocks or (blocks[0][0] == 0 and blocks[-1][0] + blocks[-1][1] == int(has.sum()))
     assert plan.ds_pairs() == int(has.sum())
     BA.BitfieldUtils.clear_cache()
 
