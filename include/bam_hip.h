@@ -109,7 +109,7 @@ typedef struct bam_plan {
     int64_t fine_stride_s;
     const int32_t* order;
     int64_t order_stride_b;
-    /* Hand-over of dS from the dK/dV kernel to the dQ kernel (see below).  ds_entry / ds_count are filled by the plan
+    /* Hand-over of dS from the dK/dV kernel to the dQ kernel (described above).  ds_entry / ds_count are filled by the plan
      * builders; ds_workspace / ds_capacity are the caller's to set before a backward call (null / 0 = not used). */
     const int32_t* ds_entry;   /* device, (B, 4 * ceil(Sq/128), ceil(Sk/128)): number of each (slice, 128-key tile) pair
                                   that has work, numbered in (batch, tile, slice) order; -1 = the pair has none */
@@ -169,6 +169,9 @@ int bam_tile_plan(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int64_t
 int bam_tile_plan_static(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int64_t flags_stride_b,
                          int64_t flags_stride_m, int B, int S, bam_plan* plan, void* stream);
 
+/* Bytes of a dS workspace for Hq query heads and `pairs` (slice, 128-key tile) pairs: 8192 * Hq * pairs. */
+int64_t bam_ds_workspace_bytes(int Hq, int64_t pairs);
+
 /*
  * Plan for index-tensor attention: classes of the 32 x 32 tiles of the LOCAL score matrix (iv->Sq rows against
  * iv->Sk keys, bitfields and positions as bam_gather_bitfields delivers them) and a slice order, laid out in
@@ -177,9 +180,6 @@ int bam_tile_plan_static(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, 
  * (shardformer/layers/utils.py:331-353); with this plan a shard skips masked work at 32-row granularity like the
  * unsharded path.  The flags the caller passes to the attention entry points are then not consulted.
  */
-/* Bytes of a dS workspace for Hq query heads and `pairs` (slice, 128-key tile) pairs. */
-int64_t bam_ds_workspace_bytes(int Hq, int64_t pairs);
-
 int bam_plan_indexed(const bam_index_view* iv, void* workspace, int64_t workspace_bytes, int B, bam_plan* plan,
                      void* stream);
 
