@@ -165,6 +165,16 @@ int fill_plan(bam::AttnParams& p, const char* who, const bam_plan* plan, int B, 
         p.ds_ws = plan->ds_workspace;
         p.ds_capacity = plan->ds_capacity;
     }
+    if (p.mask_mode == bam::MASK_DENSE && plan->row_bits != nullptr && plan->col_bits != nullptr) {
+        if ((reinterpret_cast<uintptr_t>(plan->row_bits) | reinterpret_cast<uintptr_t>(plan->col_bits)) & 3u)
+            return fail(BAM_ERR_INVALID_ARGUMENT, "%s: plan: misaligned mask bits", who);
+        p.row_bits = plan->row_bits;
+        p.row_bits_sb = plan->row_bits_stride_b;
+        p.row_bits_sn = plan->row_bits_stride_n;
+        p.col_bits = plan->col_bits;
+        p.col_bits_sb = plan->col_bits_stride_b;
+        p.col_bits_ss = plan->col_bits_stride_s;
+    }
     return BAM_OK;
 }
 
@@ -295,7 +305,7 @@ extern "C" {
 
 const char* bam_last_error(void) { return g_error; }
 
-int bam_abi_version(void) { return 7; }
+int bam_abi_version(void) { return 8; }
 
 int bam_tile_flags(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int64_t flags_stride_b,
                    int64_t flags_stride_m, int B, int S, void* stream) {
@@ -312,6 +322,7 @@ namespace {
 // workspace layout: fine | order, each part 256-byte aligned
 struct PlanLayout {
     int64_t fine_ss, fine_sb, order_sb, entry_sb, fine_off, order_off, entry_off, base_off, count_off, bytes;
+    int64_t row_sn, row_sb, col_ss, col_sb, row_off, col_off, bytes_with_bits;
 };
 PlanLayout plan_layout(int B, int Sq, int Sk) {
     const int64_t num_m = (Sq + 127) / 128, num_n = (Sk + 31) / 32, slots = 4 * num_m;
@@ -327,6 +338,14 @@ PlanLayout plan_layout(int B, int Sq, int Sk) {
     l.base_off = l.entry_off + up(B * l.entry_sb * 4, 256);
     l.count_off = l.base_off + up(B * ((Sk + 127) / 128) * 4, 256);
     l.bytes = l.count_off + 256;
+    // the packed mask of bam_mask_tile_plan: rows padded to 128, keys to 128, 32-key blocks to an even number
+    l.row_sn = num_m * 128;
+    l.row_sb = ((num_n + 1) & ~(int64_t)1) * l.row_sn;
+    l.col_ss = ((Sk + 127) / 128) * 128;
+    l.col_sb = slots * l.col_ss;
+    l.row_off = l.bytes;
+    l.col_off = l.row_off + up(B * l.row_sb * 4, 256);
+    l.bytes_with_bits = l.col_off + up(B * l.col_sb * 4, 256);
     return l;
 }
 }  // namespace
@@ -338,12 +357,17 @@ int64_t bam_plan_workspace_bytes_rect(int B, int Sq, int Sk) {
 
 int64_t bam_plan_workspace_bytes(int B, int S) { return bam_plan_workspace_bytes_rect(B, S, S); }
 
+int64_t bam_mask_plan_workspace_bytes(int B, int Sq, int Sk) {
+    if (bam_plan_workspace_bytes_rect(B, Sq, Sk) == 0) return 0;
+    return plan_layout(B, Sq, Sk).bytes_with_bits;
+}
+
 namespace {
 // Checks the workspace and lays the plan's arrays out in it.
 int place_plan(const char* who, void* workspace, int64_t workspace_bytes, int B, int Sq, int Sk, bam_plan* plan,
-               PlanLayout& l) {
+               PlanLayout& l, bool with_bits = false) {
     if (workspace == nullptr || plan == nullptr) return fail(BAM_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
-    const int64_t need = bam_plan_workspace_bytes_rect(B, Sq, Sk);
+    const int64_t need = with_bits ? bam_mask_plan_workspace_bytes(B, Sq, Sk) : bam_plan_workspace_bytes_rect(B, Sq, Sk);
     if (need == 0) return fail(BAM_ERR_UNSUPPORTED, "%s: no plan is built for Sq = %d, Sk = %d", who, Sq, Sk);
     if (workspace_bytes < need)
         return fail(BAM_ERR_INVALID_ARGUMENT, "%s: workspace of %lld bytes, %lld needed", who, (long long)workspace_bytes,
@@ -363,6 +387,12 @@ int place_plan(const char* who, void* workspace, int64_t workspace_bytes, int B,
     plan->ds_count = (const int32_t*)(w + l.count_off);
     plan->ds_workspace = nullptr;
     plan->ds_capacity = 0;
+    plan->row_bits = with_bits ? (const uint32_t*)(w + l.row_off) : nullptr;
+    plan->row_bits_stride_b = with_bits ? l.row_sb : 0;
+    plan->row_bits_stride_n = with_bits ? l.row_sn : 0;
+    plan->col_bits = with_bits ? (const uint32_t*)(w + l.col_off) : nullptr;
+    plan->col_bits_stride_b = with_bits ? l.col_sb : 0;
+    plan->col_bits_stride_s = with_bits ? l.col_ss : 0;
     plan->B = B;
     plan->Sq = Sq;
     plan->Sk = Sk;
@@ -449,11 +479,13 @@ int bam_mask_tile_plan(const uint8_t* mask, int8_t* flags, int64_t flags_stride_
     if (B > 65535 || (Sq + 127) / 128 > 65535)
         return fail(BAM_ERR_UNSUPPORTED, "bam_mask_tile_plan: grid too large (B = %d, Sq = %d)", B, Sq);
     PlanLayout l;
-    BAM_TRY(place_plan("bam_mask_tile_plan", workspace, workspace_bytes, B, Sq, Sk, plan, l));
+    BAM_TRY(place_plan("bam_mask_tile_plan", workspace, workspace_bytes, B, Sq, Sk, plan, l, true));
     char* w = (char*)workspace;
     BAM_TRY(launched(bam::launch_mask_tile_plan(mask, flags, flags_stride_b, flags_stride_m, (uint8_t*)(w + l.fine_off),
                                                 l.fine_sb, l.fine_ss, (int*)(w + l.order_off), l.order_sb,
-                                                (int*)(w + l.count_off), B, Sq, Sk, (hipStream_t)stream),
+                                                (int*)(w + l.count_off), (unsigned*)(w + l.row_off), l.row_sb, l.row_sn,
+                                                (unsigned*)(w + l.col_off), l.col_sb, l.col_ss, B, Sq, Sk,
+                                                (hipStream_t)stream),
                      "bam_mask_tile_plan"));
     return number_pairs("bam_mask_tile_plan", plan, stream);
 }

@@ -68,6 +68,13 @@ struct AttnParams {
                                // numbered consecutively, by ascending slice
     void* ds_ws;
     int64_t ds_capacity;
+    // MASK_DENSE with a plan: the mask packed to bits, once per orientation (null = read the mask bytes).
+    // row_bits (B, row_bits_sn-strided 32-key blocks, rows): bit c of word (n, r) = mask[r][32 n + c];
+    // col_bits (B, 32-row slices, keys): bit r of word (s, k) = mask[32 s + r][k].  Out-of-range cells are 0.
+    const unsigned* row_bits;
+    int64_t row_bits_sb, row_bits_sn;
+    const unsigned* col_bits;
+    int64_t col_bits_sb, col_bits_ss;
     int B, Sq, Sk, Hq, Hkv, D;
     int Sq_rounded, num_m, num_n, num_kt;  // ceil(Sq/128)*128, ceil(Sq/128), ceil(Sk/32), ceil(Sk/128)
     float scale;
@@ -105,7 +112,8 @@ int launch_indexed_plan(const int64_t* qbits, int64_t qbits_sb, const int64_t* k
 // Flags plus plan of a materialized bool mask.
 int launch_mask_tile_plan(const uint8_t* mask, int8_t* flags, int64_t flags_stride_b, int64_t flags_stride_m,
                           uint8_t* fine, int64_t fine_sb, int64_t fine_ss, int* order, int64_t order_sb, int* pair_count,
-                          int B, int Sq, int Sk, hipStream_t stream);
+                          unsigned* row_bits, int64_t row_bits_sb, int64_t row_bits_sn, unsigned* col_bits,
+                          int64_t col_bits_sb, int64_t col_bits_ss, int B, int Sq, int Sk, hipStream_t stream);
 // Numbers the (slice, 128-key tile) pairs that have work: entry (B, 4 * num_m, ceil(Sk/128)) ints, -1 = none.
 // tile_base (B, ceil(Sk/128)) ints: number of the first pair of each key tile (pairs are numbered tile by tile).
 // *count must be zero when the kernel starts (the plan kernels reset it).

@@ -85,6 +85,8 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
     __shared__ __attribute__((aligned(16))) int64_t sQbf[2][DKDV_QT];    // raw bitfields of the rows
     __shared__ __attribute__((aligned(16))) int sQpos[2][DKDV_QT];       // their global positions (IDX only)
     __shared__ __attribute__((aligned(16))) unsigned sWq[DKDV_THREADS / 64][5][32];  // per-wave rule constants
+    // DENSE with packed mask bits: for the two slices of the tile, one word per key of the workgroup's 128 keys
+    __shared__ unsigned sColBits[MODE == MASK_DENSE ? 2 : 1][2][MODE == MASK_DENSE ? 128 : 1];
     __shared__ int sListStore[MAX_SLICE_LIST + 1];  // entry -1: partner of the first entry of an odd count
     int* const sList = sListStore + 1;
     __shared__ int sCount;
@@ -180,9 +182,15 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
     // small rows of a tile: lse, delta and the two halves of the 64 int64 bitfields, 64 dwords each;
     // wave w copies row w & 3 (waves 4..7 repeat what waves 0..3 write, so that every wave issues the same
     // number of copies)
-    const int small = DENSE ? (wave & 1) : (wave & 3);
-    const unsigned ldsSmall = small == 0 ? lds_addr(sLse) : small == 1 ? lds_addr(sDelta) : lds_addr(sQbf) + (small - 2) * 256u;
-    const unsigned smallBytes = small < 2 ? DKDV_QT * 4u : DKDV_QT * 8u;  // per buffer
+    // (DENSE: rows 2 and 3 are the packed mask words of keys 0..63 / 64..127 of the tile, for the slice of the
+    // copying wave's row stream; without packed bits, waves 2, 3, 6, 7 repeat lse / delta instead)
+    const bool col_bits_on = DENSE && p.col_bits != nullptr;
+    const int small = (DENSE && !col_bits_on) ? (wave & 1) : (wave & 3);
+    const unsigned ldsSmall = small == 0   ? lds_addr(sLse)
+                              : small == 1 ? lds_addr(sDelta)
+                              : DENSE      ? lds_addr(sColBits) + (unsigned)(st * 128 + (small - 2) * 64) * 4u
+                                           : lds_addr(sQbf) + (small - 2) * 256u;
+    const unsigned smallBytes = small < 2 ? DKDV_QT * 4u : DENSE ? 2 * 128 * 4u : DKDV_QT * 8u;  // per buffer
     // Where the copies of a tile read.  The scalar unit is shared by the whole compute unit, so the address
     // arithmetic is kept short: per-head base pointers are carried along and bumped when the head changes, row
     // offsets are 32 x 32 -> 64 bit unsigned products (rows < 2^22, row strides < 2^25 bytes by the host checks).
@@ -199,6 +207,7 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
         hb.g = (const char*)p.dout.ptr + 2 * ((int64_t)b * p.dout.sb + (int64_t)h * p.dout.sh);
         hb.small = small == 0   ? (const char*)(p.lse + ((int64_t)b * p.Hq + h) * p.Sq_rounded)
                    : small == 1 ? (const char*)(p.delta + ((int64_t)b * p.Hq + h) * p.Sq_rounded)
+                   : DENSE      ? (const char*)(p.col_bits + (int64_t)b * p.col_bits_sb + nt * 128 + (small - 2) * 64)
                                 : (const char*)bfrow;
         return hb;
     };
@@ -229,7 +238,10 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
         // lse / delta (small < 2): 32 floats of each slice.  Bitfields: 32 int64 = 64 dwords of slice lo
         // (small == 2) or hi (small == 3).
         const unsigned srow = (unsigned)(small == 3 ? row_hi : row_lo);
-        t.small = hb.small + (small < 2 ? srow * 4u : srow * 8u);
+        if (DENSE && small >= 2)  // the words of the slice this wave's row stream works on
+            t.small = hb.small + (uint64_t)((unsigned)(st ? row_hi : row_lo) >> 5) * (uint64_t)(p.col_bits_ss * 4);
+        else
+            t.small = hb.small + (small < 2 ? srow * 4u : srow * 8u);
         const unsigned shift = (unsigned)((row_hi - row_lo - 32) * 4);
         t.pos_voff = (unsigned)(lane * 4) + (shift & upper_lanes);
         t.small_voff = small < 2 ? t.pos_voff : (unsigned)(lane * 4);
@@ -336,7 +348,11 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
             for (int x = 0; x < 4; ++x) s[4 * grp + x] = __builtin_amdgcn_exp2f(fmaf(s[4 * grp + x], c2, l4[x] * -LOG2E));
         }
         if (DENSE) {
-            if (cls == 1) {
+            if (cls == 1 && col_bits_on) {
+                const unsigned w = sColBits[cur][st][32 * kg + l32];
+#pragma unroll
+                for (int i = 0; i < 16; ++i) s[i] = ((w >> (8 * (i >> 2) + 4 * hi + (i & 3))) & 1u) ? s[i] : 0.f;
+            } else if (cls == 1) {
                 // mask bytes of this lane's key column, one per row of the C fragment
                 const uint8_t* mcol = p.mask + ((int64_t)b * Sq + myrow0) * Sk + key;
 #pragma unroll
@@ -538,6 +554,8 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
                     if (!DENSE) sQbf[0][tid] = ok ? bfrow[row0 + tid] : 0;
                     if (IDX) sQpos[0][tid] = ok ? p.posq[row0 + tid] : 0;
                 }
+                if (col_bits_on && tid < 128)  // the slice sits in row stream 0
+                    sColBits[0][0][tid] = p.col_bits[(int64_t)b * p.col_bits_sb + (int64_t)(row0 >> 5) * p.col_bits_ss + nt * 128 + tid];
                 __syncthreads();
                 load_kv_operands();
                 // the slice sits in LDS rows 0..31: row stream 0 computes it, row stream 1 has nothing to do
@@ -642,6 +660,8 @@ __global__ __launch_bounds__(DQ_THREADS, D == 128 ? 2 : 3) void bwd_dq_kernel(co
     __shared__ __attribute__((aligned(16))) int sKpos[2][DQ_KT];     // their global positions (IDX only)
     __shared__ int sList[MAX_LIST];
     __shared__ int sCount;
+    // DENSE with packed mask bits: per wave, the words of its 32 rows for the tile's two 32-key blocks
+    __shared__ unsigned sRowBits[DENSE ? 2 : 1][4][DENSE ? 64 : 1];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int hi = lane >> 5, l32 = lane & 31, half16 = (lane >> 4) & 1;
@@ -709,12 +729,18 @@ __global__ __launch_bounds__(DQ_THREADS, D == 128 ? 2 : 3) void bwd_dq_kernel(co
     typedef TileStage<D, DQ_KT, DQ_THREADS> Stage;
     constexpr int CPT = Stage::CPT;
     // copy instructions per wave and tile: K, V, the key bitfields and (IDX) the key positions
-    constexpr int NLOADS = 2 * CPT + (DENSE ? 0 : 1) + (IDX ? 1 : 0);
+    constexpr int NLOADS = 2 * CPT + 1 + (IDX ? 1 : 0);
     static_assert(NLOADS <= 2 * KK, "one copy per MFMA of the first S / dP block");
     Stage stK, stV;
     stK.setup(2 * p.k.ss, tid);
     stV.setup(2 * p.v.ss, tid);
     const unsigned ldsK = lds_addr(sK), ldsV = lds_addr(sV), ldsB = lds_addr(sKbf), ldsP = lds_addr(sKpos);
+    const unsigned ldsR = lds_addr(sRowBits);
+    // DENSE: the packed mask rows of this wave's slice (null: no plan, the mask bytes are read instead)
+    const unsigned* row_bits_w = (DENSE && p.row_bits != nullptr)
+                                     ? p.row_bits + (int64_t)b * p.row_bits_sb + (slice < 0 ? 0 : slice) * 32
+                                     : nullptr;
+    const unsigned row_bits_voff = DENSE ? (unsigned)(hi * (int)p.row_bits_sn * 4 + l32 * 4) : 0u;
     constexpr unsigned TILE_BYTES = DQ_KT * NCH * 16, BITS_BYTES = DQ_KT * 8;
     // copy instruction j of full tile kt into buffer buf (key bitfields: 64 dwords per wave, waves 2, 3
     // repeat what waves 0, 1 write, so that every wave issues the same number of copies)
@@ -723,8 +749,14 @@ __global__ __launch_bounds__(DQ_THREADS, D == 128 ? 2 : 3) void bwd_dq_kernel(co
             stK.issue(j, kbase + kt * k_ts, ldsK + buf * TILE_BYTES);
         else if (j < 2 * CPT)
             stV.issue(j - CPT, vbase + kt * v_ts, ldsV + buf * TILE_BYTES);
-        else if (j == 2 * CPT)
-            dma_b32(bfrow + kt * DQ_KT, (unsigned)((wave & 1) * 256 + lane * 4), ldsB + buf * BITS_BYTES + (wave & 1) * 256u);
+        else if (j == 2 * CPT) {
+            if (DENSE) {  // lanes 0..31: block 2 kt, lanes 32..63: block 2 kt + 1, rows of this wave's slice
+                if (row_bits_w != nullptr)
+                    dma_b32(row_bits_w + (int64_t)(2 * kt) * p.row_bits_sn, row_bits_voff, ldsR + (unsigned)(buf * 4 + wave) * 256u);
+            } else {
+                dma_b32(bfrow + kt * DQ_KT, (unsigned)((wave & 1) * 256 + lane * 4), ldsB + buf * BITS_BYTES + (wave & 1) * 256u);
+            }
+        }
         else  // 64 positions; every wave writes the same values
             dma_b32(p.posk + kt * DQ_KT, (unsigned)(lane * 4), ldsP + buf * (DQ_KT * 4u));
     };
@@ -798,7 +830,11 @@ __global__ __launch_bounds__(DQ_THREADS, D == 128 ? 2 : 3) void bwd_dq_kernel(co
                 dp[i] = e * (dp[i] - dlt);  // the factor `scale` of dS is applied to dQ in the epilogue
             }
             if (DENSE) {
-                if (cls == 1) {
+                if (cls == 1 && row_bits_w != nullptr) {
+                    const unsigned w = sRowBits[cur][wave][32 * kb + l32];
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) dp[i] = ((w >> (8 * (i >> 2) + 4 * hi + (i & 3))) & 1u) ? dp[i] : 0.f;
+                } else if (cls == 1) {
                     const int kt0 = kt * DQ_KT;
                     const uint8_t* mrow = p.mask + ((int64_t)b * Sq + (qvalid ? qrow : 0)) * Sk + kt0;
                     const bool dwords = (Sk & 3) == 0;  // rows start 4-byte aligned
@@ -910,6 +946,8 @@ __global__ __launch_bounds__(DQ_THREADS, D == 128 ? 2 : 3) void bwd_dq_kernel(co
                 sKbf[0][tid] = (tid < rows) ? bfrow[kt * DQ_KT + tid] : 0;
                 if (IDX) sKpos[0][tid] = (tid < rows) ? p.posk[kt * DQ_KT + tid] : 0;
             }
+            if (DENSE && row_bits_w != nullptr)
+                sRowBits[0][wave][lane] = row_bits_w[(int64_t)(2 * kt + hi) * p.row_bits_sn + l32];
             __syncthreads();
             tile_step(std::false_type{}, 0, entry, 0);
         }

@@ -45,11 +45,13 @@ __global__ __launch_bounds__(FWD_THREADS, D == 128 ? 2 : 3) void fwd_kernel(cons
     __shared__ __attribute__((aligned(16))) int sKpos[2][FWD_KT];     // their global positions (IDX only)
     __shared__ int sList[MAX_LIST];
     __shared__ int sCount;
+    constexpr bool IDX = MODE == MASK_INDEXED, DENSE = MODE == MASK_DENSE;
+    // DENSE with packed mask bits: per wave, the words of its 32 rows for the tile's two 32-key blocks
+    __shared__ unsigned sRowBits[DENSE ? 2 : 1][4][DENSE ? 64 : 1];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int hi = lane >> 5, l32 = lane & 31, half16 = (lane >> 4) & 1;
     const int wave_lane = tid >> 6;
-    constexpr bool IDX = MODE == MASK_INDEXED, DENSE = MODE == MASK_DENSE;
     const int Sq = p.Sq, Sk = p.Sk;
     const int G = p.Hq / p.Hkv;
 
@@ -112,13 +114,20 @@ __global__ __launch_bounds__(FWD_THREADS, D == 128 ? 2 : 3) void fwd_kernel(cons
 
     typedef TileStage<D, FWD_KT, FWD_THREADS> Stage;
     constexpr int CPT = Stage::CPT;
-    // copy instructions per wave and tile: K, V, the key bitfields and (IDX) the key positions
-    constexpr int NLOADS = 2 * CPT + (DENSE ? 0 : 1) + (IDX ? 1 : 0);
+    // copy instructions per wave and tile: K, V, the key bitfields (DENSE: the mask bits of the wave's rows) and
+    // (IDX) the key positions
+    constexpr int NLOADS = 2 * CPT + 1 + (IDX ? 1 : 0);
     static_assert(NLOADS <= 2 * KK, "one copy per MFMA of the S phase");
     Stage stK, stV;
     stK.setup(2 * p.k.ss, tid);
     stV.setup(2 * p.v.ss, tid);
     const unsigned ldsK = lds_addr(sK), ldsV = lds_addr(sV), ldsB = lds_addr(sKbf), ldsP = lds_addr(sKpos);
+    const unsigned ldsR = lds_addr(sRowBits);
+    // DENSE: the packed mask rows of this wave's slice (null: no plan, the mask bytes are read instead)
+    const unsigned* row_bits_w = (DENSE && p.row_bits != nullptr)
+                                     ? p.row_bits + (int64_t)b * p.row_bits_sb + (slice < 0 ? 0 : slice) * 32
+                                     : nullptr;
+    const unsigned row_bits_voff = DENSE ? (unsigned)(hi * (int)p.row_bits_sn * 4 + l32 * 4) : 0u;
     constexpr unsigned TILE_BYTES = FWD_KT * NCH * 16, BITS_BYTES = FWD_KT * 8;
     // Copy instruction j (0 <= j < NLOADS) of full tile kt into buffer buf.  The 128 dwords of key
     // bitfields are copied 64 dwords per wave (waves 2, 3 repeat what waves 0, 1 write), so that every
@@ -128,8 +137,14 @@ __global__ __launch_bounds__(FWD_THREADS, D == 128 ? 2 : 3) void fwd_kernel(cons
             stK.issue(j, kbase + kt * k_ts, ldsK + buf * TILE_BYTES);
         else if (j < 2 * CPT)
             stV.issue(j - CPT, vbase + kt * v_ts, ldsV + buf * TILE_BYTES);
-        else if (j == 2 * CPT)  // (never reached with a dense mask: NLOADS == 2 * CPT)
-            dma_b32(bfrow + kt * FWD_KT, (unsigned)((wave & 1) * 256 + lane * 4), ldsB + buf * BITS_BYTES + (wave & 1) * 256u);
+        else if (j == 2 * CPT) {
+            if (DENSE) {  // lanes 0..31: block 2 kt, lanes 32..63: block 2 kt + 1, rows of this wave's slice
+                if (row_bits_w != nullptr)
+                    dma_b32(row_bits_w + (int64_t)(2 * kt) * p.row_bits_sn, row_bits_voff, ldsR + (unsigned)(buf * 4 + wave) * 256u);
+            } else {
+                dma_b32(bfrow + kt * FWD_KT, (unsigned)((wave & 1) * 256 + lane * 4), ldsB + buf * BITS_BYTES + (wave & 1) * 256u);
+            }
+        }
         else  // 64 positions; every wave writes the same values
             dma_b32(p.posk + kt * FWD_KT, (unsigned)(lane * 4), ldsP + buf * (FWD_KT * 4u));
     };
@@ -188,7 +203,16 @@ __global__ __launch_bounds__(FWD_THREADS, D == 128 ? 2 : 3) void fwd_kernel(cons
 
         // ---- bitfield rule in registers (partial tiles only) ------------------------------
         if (DENSE) {
-            if (cls == 1) {
+            if (cls == 1 && row_bits_w != nullptr) {
+                const unsigned w01[2] = {sRowBits[cur][wave][l32], sRowBits[cur][wave][32 + l32]};
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) {
+                        const int bit = 8 * (i >> 2) + 4 * hi + (i & 3);
+                        s[kb][i] = ((w01[kb] >> bit) & 1u) ? s[kb][i] : -INFINITY;
+                    }
+            } else if (cls == 1) {
                 // mask bytes of this lane's query row: 4 consecutive keys per C-fragment group
                 const int kt0 = kt * FWD_KT;
                 const uint8_t* mrow = p.mask + ((int64_t)b * Sq + (qvalid ? qrow : 0)) * Sk + kt0;
@@ -371,6 +395,8 @@ __global__ __launch_bounds__(FWD_THREADS, D == 128 ? 2 : 3) void fwd_kernel(cons
                 sKbf[0][tid] = (tid < rows) ? bfrow[kt * FWD_KT + tid] : 0;
                 if (IDX) sKpos[0][tid] = (tid < rows) ? p.posk[kt * FWD_KT + tid] : 0;
             }
+            if (DENSE && row_bits_w != nullptr)
+                sRowBits[0][wave][lane] = row_bits_w[(int64_t)(2 * kt + hi) * p.row_bits_sn + l32];
             __syncthreads();
             tile_step(std::false_type{}, 0, entry, 0);
         }

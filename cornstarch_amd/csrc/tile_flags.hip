@@ -418,12 +418,19 @@ int launch_indexed_plan(const int64_t* qbits, int64_t qbits_sb, const int64_t* k
 // 32-row slice, so that the four slice classes of every flag tile come out of the same pass over the mask.  The
 // slice order is simply "last slice first" (under a causal-like mask the late rows see the most keys); it is
 // written by the workgroups of column 0.
+// The same pass packs the mask to bits, once per orientation, for the attention kernels (which then never touch the
+// mask bytes): thread = key column, so the 32 rows of a slice make one word of col_bits in a register, and a ballot
+// over the 32 columns of a tile makes one word of row_bits per row.  Cells outside the mask are 0; the arrays cover
+// num_m * 128 rows, ceil(Sk / 128) * 128 keys and an even number of 32-key blocks.
 __global__ __launch_bounds__(256) void mask_tile_plan_kernel(const uint8_t* __restrict__ mask, int8_t* __restrict__ flags,
                                                              int64_t flags_stride_b, int64_t flags_stride_m, int Sq,
                                                              int Sk, int num_n, uint8_t* __restrict__ fine,
                                                              int64_t fine_sb, int64_t fine_ss, int* __restrict__ order,
-                                                             int64_t order_sb, int* __restrict__ pair_count) {
-    const int b = blockIdx.z, m = blockIdx.y, tid = threadIdx.x;
+                                                             int64_t order_sb, int* __restrict__ pair_count,
+                                                             unsigned* __restrict__ row_bits, int64_t row_bits_sb,
+                                                             int64_t row_bits_sn, unsigned* __restrict__ col_bits,
+                                                             int64_t col_bits_sb, int64_t col_bits_ss) {
+    const int b = blockIdx.z, m = blockIdx.y, tid = threadIdx.x, lane = tid & 63;
     if (pair_count != nullptr && blockIdx.x == 0 && m == 0 && b == 0 && tid == 0) *pair_count = 0;
     if (blockIdx.x == 0 && tid < 4) {
         const int ns = (Sq + 31) / 32, slot = 4 * m + tid;
@@ -431,21 +438,43 @@ __global__ __launch_bounds__(256) void mask_tile_plan_kernel(const uint8_t* __re
     }
     const int col = blockIdx.x * 256 + tid;
     const int r0 = m * BLOCK_M;
-    int count[4] = {0, 0, 0, 0};
-    if (col < Sk) {
-        const uint8_t* pcol = mask + (int64_t)b * Sq * Sk + col;
+    const int n = blockIdx.x * 8 + (tid >> 5);  // this thread's 32-key block
+    const int num_n_bits = (num_n + 1) & ~1, sk_pad = ((Sk + 127) >> 7) << 7;
+    const bool in = col < Sk;
+    const uint8_t* pcol = mask + (int64_t)b * Sq * Sk + (in ? col : 0);
+    // lanes 0 and 32 of a wave write the row words of its two 32-key blocks
+    unsigned* rb_out = (row_bits != nullptr && (lane & 31) == 0 && n < num_n_bits)
+                           ? row_bits + (int64_t)b * row_bits_sb + (int64_t)n * row_bits_sn + r0
+                           : nullptr;
+    unsigned cw[4];
 #pragma unroll
-        for (int w = 0; w < 4; ++w) {
-            const int ra = r0 + 32 * w, rb = min(ra + 32, Sq);
-            for (int r = ra; r < rb; ++r) count[w] += pcol[(int64_t)r * Sk] != 0;
+    for (int w = 0; w < 4; ++w) {
+        cw[w] = 0;
+        const int ra = r0 + 32 * w;
+        if (row_bits == nullptr) {
+            const int rb = min(ra + 32, Sq);
+            for (int r = ra; r < rb; ++r) cw[w] |= (unsigned)(in && pcol[(int64_t)r * Sk] != 0) << (r - ra);
+        } else {
+            for (int r = ra; r < ra + 32; ++r) {
+                const bool a = in && r < Sq && pcol[(int64_t)r * Sk] != 0;
+                cw[w] |= (unsigned)a << (r - ra);
+                const unsigned long long bal = __ballot(a);
+                if (rb_out != nullptr) rb_out[r - r0] = (unsigned)(lane == 0 ? bal : bal >> 32);
+            }
         }
     }
+    if (col_bits != nullptr && col < sk_pad) {
+#pragma unroll
+        for (int w = 0; w < 4; ++w) col_bits[(int64_t)b * col_bits_sb + (int64_t)(4 * m + w) * col_bits_ss + col] = cw[w];
+    }
+    int count[4];
+#pragma unroll
+    for (int w = 0; w < 4; ++w) count[w] = __popc(cw[w]);
 #pragma unroll
     for (int off = 16; off > 0; off >>= 1) {  // over the 32 columns of a tile
 #pragma unroll
         for (int w = 0; w < 4; ++w) count[w] += __shfl_xor(count[w], off);
     }
-    const int n = blockIdx.x * 8 + (tid >> 5);
     if ((tid & 31) == 0 && n < num_n) {
         const int cols = min(BLOCK_N, Sk - n * BLOCK_N);
         int total = 0, cells = 0;
@@ -463,11 +492,13 @@ __global__ __launch_bounds__(256) void mask_tile_plan_kernel(const uint8_t* __re
 
 int launch_mask_tile_plan(const uint8_t* mask, int8_t* flags, int64_t flags_stride_b, int64_t flags_stride_m,
                           uint8_t* fine, int64_t fine_sb, int64_t fine_ss, int* order, int64_t order_sb, int* pair_count,
-                          int B, int Sq, int Sk, hipStream_t stream) {
+                          unsigned* row_bits, int64_t row_bits_sb, int64_t row_bits_sn, unsigned* col_bits,
+                          int64_t col_bits_sb, int64_t col_bits_ss, int B, int Sq, int Sk, hipStream_t stream) {
     const int num_m = (Sq + BLOCK_M - 1) / BLOCK_M, num_n = (Sk + BLOCK_N - 1) / BLOCK_N;
     dim3 grid((num_n + 7) / 8, num_m, B);
     hipLaunchKernelGGL(mask_tile_plan_kernel, grid, dim3(256), 0, stream, mask, flags, flags_stride_b, flags_stride_m, Sq,
-                       Sk, num_n, fine, fine_sb, fine_ss, order, order_sb, pair_count);
+                       Sk, num_n, fine, fine_sb, fine_ss, order, order_sb, pair_count, row_bits, row_bits_sb, row_bits_sn,
+                       col_bits, col_bits_sb, col_bits_ss);
     return (int)hipGetLastError();
 }
 

@@ -15,7 +15,7 @@ BAM_DTYPE_F16 = 0
 BAM_DTYPE_BF16 = 1
 BAM_MAX_SEQLEN = 4194304
 BAM_STATIC_PLAN_BYTES = 8 << 20
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 _i64 = ctypes.c_int64
 _int = ctypes.c_int
@@ -64,6 +64,12 @@ class Plan(ctypes.Structure):
         ("ds_count", ctypes.c_void_p),
         ("ds_workspace", ctypes.c_void_p),
         ("ds_capacity", ctypes.c_int64),
+        ("row_bits", ctypes.c_void_p),
+        ("row_bits_stride_b", ctypes.c_int64),
+        ("row_bits_stride_n", ctypes.c_int64),
+        ("col_bits", ctypes.c_void_p),
+        ("col_bits_stride_b", ctypes.c_int64),
+        ("col_bits_stride_s", ctypes.c_int64),
         ("B", ctypes.c_int32),
         ("Sq", ctypes.c_int32),
         ("Sk", ctypes.c_int32),
@@ -126,6 +132,8 @@ def load() -> ctypes.CDLL:
     lib.bam_plan_workspace_bytes.argtypes = [_int, _int]
     lib.bam_plan_workspace_bytes_rect.restype = _i64
     lib.bam_plan_workspace_bytes_rect.argtypes = [_int, _int, _int]
+    lib.bam_mask_plan_workspace_bytes.restype = _i64
+    lib.bam_mask_plan_workspace_bytes.argtypes = [_int, _int, _int]
     lib.bam_ds_workspace_bytes.restype = _i64
     lib.bam_ds_workspace_bytes.argtypes = [_int, _i64]
     for name, argtypes in SIGNATURES.items():

@@ -53,7 +53,8 @@ def mask_tile_flags(mask: Optional[torch.Tensor], batch: int, seqlen_q: int, seq
 
 
 class _MaskPlan:
-    """Flags and plan (classes of the 32 x 32 tiles, slice order) of a bool mask, from one pass over it.  The forward
+    """Flags and plan (classes of the 32 x 32 tiles, slice order, the mask packed to bits for the kernels: a quarter
+    of the mask's size in all) of a bool mask, from one pass over it.  The forward
     and, later, the backward of one call bring the same mask tensor: the last result is kept, together with the mask
     it was computed from (so its address cannot be handed to another tensor meanwhile), and reused while that is
     unchanged."""
@@ -72,7 +73,7 @@ class _MaskPlan:
 
         num_m, num_n = -(-seqlen_q // BLOCK_M), -(-seqlen_k // BLOCK_N)
         with torch.cuda.device(device):
-            ws_bytes = _bam_hip.load().bam_plan_workspace_bytes_rect(batch, seqlen_q, seqlen_k)
+            ws_bytes = _bam_hip.load().bam_mask_plan_workspace_bytes(batch, seqlen_q, seqlen_k)
             if ws_bytes > 0:
                 flags = torch.empty((batch, num_m, num_n), dtype=torch.int8, device=device)
                 workspace = torch.empty((ws_bytes,), dtype=torch.uint8, device=device)

@@ -118,6 +118,16 @@ typedef struct bam_plan {
     const int32_t* ds_count;   /* device, one int: how many such pairs there are */
     void* ds_workspace;        /* device, at least bam_ds_workspace_bytes(Hq, pairs) bytes, 16-byte aligned */
     int64_t ds_capacity;       /* pairs the workspace has room for: at least *ds_count */
+    /* Materialized masks only (bam_mask_tile_plan; null otherwise): the mask packed to bits, once per orientation, so
+     * that the attention kernels never read the mask bytes.  row_bits: bit c of word
+     * [b * row_bits_stride_b + n * row_bits_stride_n + r] = mask[b][r][32 n + c]; col_bits: bit r of word
+     * [b * col_bits_stride_b + s * col_bits_stride_s + k] = mask[b][32 s + r][k]; cells outside the mask are 0. */
+    const uint32_t* row_bits;
+    int64_t row_bits_stride_b;
+    int64_t row_bits_stride_n;
+    const uint32_t* col_bits;
+    int64_t col_bits_stride_b;
+    int64_t col_bits_stride_s;
     int32_t B;
     int32_t Sq;         /* query rows and keys the plan was built for (equal for plain bitfield attention) */
     int32_t Sk;
@@ -364,11 +374,15 @@ int bam_bwd_dq_masked(const void* q, const void* k, const void* v, const void* d
         void* stream);
 
 /*
- * bam_mask_tile_flags plus a plan, in one pass over the mask: the four 32-row classes of every flag tile and a slice
- * order (last slice first).  workspace: at least bam_plan_workspace_bytes_rect(B, Sq, Sk) bytes, 256-byte aligned.
+ * bam_mask_tile_flags plus a plan, in one pass over the mask: the four 32-row classes of every flag tile, a slice
+ * order (last slice first) and the mask packed to bits in both orientations (plan->row_bits, plan->col_bits: an
+ * eighth of the mask's size each), which is what the attention kernels consult in partial tiles when they are given
+ * the plan -- without one they read the mask bytes.  workspace: at least bam_mask_plan_workspace_bytes(B, Sq, Sk)
+ * bytes (0 = no plan is built for that size), 256-byte aligned.
  * Serves `_flash_attn_forward` / `_flash_attn_backward` of the reference's cornstarch/kernel/attention.py:855-1146,
- * whose kernels decide per 128 x 32 tile inside the attention loop (:188-200).
+ * whose kernels decide per 128 x 32 tile inside the attention loop (:188-200) and load the mask bytes there (:217-232).
  */
+int64_t bam_mask_plan_workspace_bytes(int B, int Sq, int Sk);
 int bam_mask_tile_plan(const uint8_t* mask, int8_t* flags, int64_t flags_stride_b, int64_t flags_stride_m, void* workspace,
                        int64_t workspace_bytes, int B, int Sq, int Sk, bam_plan* plan, void* stream);
 

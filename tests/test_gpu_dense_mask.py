@@ -162,6 +162,26 @@ def test_mask_plan_classes_and_results_do_not_depend_on_the_plan(Sq, Sk, D, monk
         order = plan.slice_order()[b].cpu().tolist()
         assert order[:n_q] == list(range(n_q - 1, -1, -1)) and all(x == -1 for x in order[n_q:])
 
+    # the mask packed to bits, both orientations, zero outside the mask
+    st, ws = plan.struct, plan.workspace
+
+    def words(ptr, count):
+        off = ptr - ws.data_ptr()
+        return ws[off : off + 4 * count].view(torch.int32).cpu().to(torch.int64) & 0xFFFFFFFF
+
+    rows_pad, keys_pad, n_blocks = 128 * -(-Sq // 128), 128 * -(-Sk // 128), 2 * -(-n_k // 2)
+    assert (st.row_bits_stride_n, st.row_bits_stride_b) == (rows_pad, n_blocks * rows_pad)
+    assert (st.col_bits_stride_s, st.col_bits_stride_b) == (keys_pad, (rows_pad // 32) * keys_pad)
+    big = torch.zeros(2, rows_pad, max(keys_pad, 32 * n_blocks), dtype=torch.int64)
+    big[:, :Sq, :Sk] = mask
+    weights = 1 << torch.arange(32, dtype=torch.int64)
+    want_rows = (big[:, :, : 32 * n_blocks].view(2, rows_pad, n_blocks, 32) * weights).sum(-1).permute(0, 2, 1)
+    got_rows = words(st.row_bits, 2 * n_blocks * rows_pad).view(2, n_blocks, rows_pad)
+    assert torch.equal(got_rows, want_rows)
+    want_cols = (big[:, :, :keys_pad].view(2, rows_pad // 32, 32, keys_pad) * weights[None, None, :, None]).sum(2)
+    got_cols = words(st.col_bits, 2 * (rows_pad // 32) * keys_pad).view(2, rows_pad // 32, keys_pad)
+    assert torch.equal(got_cols, want_cols)
+
     q, k, v, do = (t.to(d) for t in inputs(2, Sq, Sk, 4, 2, D, torch.bfloat16, seed=Sq))
 
     def run():

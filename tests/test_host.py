@@ -41,7 +41,7 @@ def test_library_exports_every_declared_symbol():
     # the binding's prototypes cover every compute entry point of the header
     assert set(_bam_hip.SIGNATURES) == set(names) - {
         "bam_last_error", "bam_abi_version", "bam_plan_workspace_bytes", "bam_plan_workspace_bytes_rect",
-        "bam_ds_workspace_bytes"}
+        "bam_ds_workspace_bytes", "bam_mask_plan_workspace_bytes"}
     # plan workspace: sized without a GPU; no plan beyond 4096 row slices
     lib2 = _bam_hip.load()
     assert lib2.bam_plan_workspace_bytes(1, 8192) >= 256 * 256 + 256 * 4 and lib2.bam_plan_workspace_bytes(1, 8192) % 256 == 0
@@ -50,6 +50,9 @@ def test_library_exports_every_declared_symbol():
     assert lib2.bam_plan_workspace_bytes_rect(1, 8192, 8192) == lib2.bam_plan_workspace_bytes(1, 8192)
     assert lib2.bam_plan_workspace_bytes_rect(1, 4096, 8192) >= 128 * 256 + 128 * 4
     assert lib2.bam_plan_workspace_bytes_rect(1, 131073, 64) == 0 and lib2.bam_plan_workspace_bytes_rect(1, 64, 262144) > 0
+    # a mask plan also holds the mask packed to bits, once per orientation: a quarter of the mask's bytes
+    extra = lib2.bam_mask_plan_workspace_bytes(1, 8192, 8192) - lib2.bam_plan_workspace_bytes_rect(1, 8192, 8192)
+    assert extra == 2 * 8192 * 8192 // 8 and lib2.bam_mask_plan_workspace_bytes(1, 131073, 64) == 0
 
 
 def test_abi_rejects_bad_arguments_without_touching_the_gpu():
