@@ -274,6 +274,16 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
     // i.e. in the order of the slice list: pair number = ds_base + position in the list
     int ds_base = 0;
     if (SAVE) ds_base = __builtin_amdgcn_readfirstlane(p.ds_tile_base[(int64_t)b * p.num_kt + nt]);
+    // BIAS, per-key form (row stride 0): this lane's bias value for the head in work
+    float bias_key = 0.f;
+    int bias_head = -1;
+    auto fetch_bias_key = [&](int h) {
+        if (BIAS && p.bias_sm == 0 && h != bias_head) {
+            bias_head = h;
+            bias_key = kvalid ? load_bias1<T>(p.bias, (int64_t)b * p.bias_sb + (int64_t)h * p.bias_sh + key, p.bias_f32 != 0) : 0.f;
+            asm volatile("" : "+v"(bias_key));  // arrives here, not at its first use between the tile copies
+        }
+    };
     // ds_pos: position of the wave's slice in the slice list.
     // returns true when the wave has issued its two dS stores (they may stay in flight over the end of the iteration)
     auto tile_step = [&](auto prefetch, int cur, int cls, int h_cur, int myrow0, int ds_pos, const TileSource& next) -> bool {
@@ -330,7 +340,11 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
         // ---- P = exp(scale s - lse) on allowed pairs, -dS/scale = P (delta - dP)   (the factor `-scale` of dS
         // is applied once to dK in the epilogue).  C fragment: register i <-> query row
         // 8*(i/4) + 4*hi + i%4 of this wave's 32 rows.
-        if (BIAS) {
+        if (BIAS && p.bias_sm == 0) {
+            // the per-key ("vector") form: one value per key and head, fetched when the head changes
+#pragma unroll
+            for (int i = 0; i < 16; ++i) s[i] = fmaf(s[i], p.scale, bias_key);
+        } else if (BIAS) {
             // column `key` of the bias, one element per row of the C fragment
             const int64_t col = (int64_t)b * p.bias_sb + (int64_t)h_cur * p.bias_sh + key;
 #pragma unroll
@@ -514,6 +528,7 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
                 const int a_lo = entry_lo(r_aft), a_hi = entry_hi(r_aft);
                 const TileSource next = tile_source(hb_nxt, (n_lo >> 8) * 32, (n_hi >> 8) * 32);
                 const int mine = st ? e_hi : e_lo;
+                fetch_bias_key(hk * G + g_cur);
                 const bool stored = tile_step(std::true_type{}, cur, (mine >> (2 * kg_lane)) & 3, hk * G + g_cur,
                                               (mine >> 8) * 32, n - 2 - 2 * r_cur + st, next);
                 g_cur = g_nxt;
@@ -558,6 +573,7 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
                     sColBits[0][0][tid] = p.col_bits[(int64_t)b * p.col_bits_sb + (int64_t)(row0 >> 5) * p.col_bits_ss + nt * 128 + tid];
                 __syncthreads();
                 load_kv_operands();
+                fetch_bias_key(h);
                 // the slice sits in LDS rows 0..31: row stream 0 computes it, row stream 1 has nothing to do
                 tile_step(std::false_type{}, 0, st ? 0 : (entry >> (2 * kg_lane)) & 3, h, row0, n_all - 1, TileSource{});
             }

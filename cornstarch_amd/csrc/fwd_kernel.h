@@ -48,6 +48,8 @@ __global__ __launch_bounds__(FWD_THREADS, D == 128 ? 2 : 3) void fwd_kernel(cons
     constexpr bool IDX = MODE == MASK_INDEXED, DENSE = MODE == MASK_DENSE;
     // DENSE with packed mask bits: per wave, the words of its 32 rows for the tile's two 32-key blocks
     __shared__ unsigned sRowBits[DENSE ? 2 : 1][4][DENSE ? 64 : 1];
+    // BIAS in its per-key ("vector") form: the 64 values of the tile (raw words; 16-bit elements fill half)
+    __shared__ __attribute__((aligned(16))) unsigned sBias[BIAS ? 2 : 1][BIAS ? 64 : 1];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int hi = lane >> 5, l32 = lane & 31, half16 = (lane >> 4) & 1;
@@ -116,13 +118,19 @@ __global__ __launch_bounds__(FWD_THREADS, D == 128 ? 2 : 3) void fwd_kernel(cons
     constexpr int CPT = Stage::CPT;
     // copy instructions per wave and tile: K, V, the key bitfields (DENSE: the mask bits of the wave's rows) and
     // (IDX) the key positions
-    constexpr int NLOADS = 2 * CPT + 1 + (IDX ? 1 : 0);
-    static_assert(NLOADS <= 2 * KK, "one copy per MFMA of the S phase");
+    constexpr int NLOADS = 2 * CPT + 1 + (IDX ? 1 : 0) + (BIAS ? 1 : 0);
+    static_assert(NLOADS <= 2 * KK + 1, "one copy per MFMA of the S phase (and at most one behind it)");
     Stage stK, stV;
     stK.setup(2 * p.k.ss, tid);
     stV.setup(2 * p.v.ss, tid);
     const unsigned ldsK = lds_addr(sK), ldsV = lds_addr(sV), ldsB = lds_addr(sKbf), ldsP = lds_addr(sKpos);
     const unsigned ldsR = lds_addr(sRowBits);
+    // A per-key bias whose groups of four keys are aligned, in-range accesses travels with the tile copies: 64 values
+    // per tile, one word per lane (16-bit elements: lanes 32..63 repeat lanes 0..31).
+    const bool bias_lds = BIAS && p.bias_sm == 0 && p.bias_vec != 0;
+    const char* bias_head = BIAS ? (const char*)p.bias + (p.bias_f32 ? 4 : 2) * ((int64_t)b * p.bias_sb + (int64_t)h * p.bias_sh) : nullptr;
+    const unsigned bias_voff = (unsigned)((p.bias_f32 ? lane : (lane & 31)) * 4);
+    const int bias_tile_bytes = FWD_KT * (p.bias_f32 ? 4 : 2);
     // DENSE: the packed mask rows of this wave's slice (null: no plan, the mask bytes are read instead)
     const unsigned* row_bits_w = (DENSE && p.row_bits != nullptr)
                                      ? p.row_bits + (int64_t)b * p.row_bits_sb + (slice < 0 ? 0 : slice) * 32
@@ -145,8 +153,10 @@ __global__ __launch_bounds__(FWD_THREADS, D == 128 ? 2 : 3) void fwd_kernel(cons
                 dma_b32(bfrow + kt * FWD_KT, (unsigned)((wave & 1) * 256 + lane * 4), ldsB + buf * BITS_BYTES + (wave & 1) * 256u);
             }
         }
-        else  // 64 positions; every wave writes the same values
+        else if (IDX && j == 2 * CPT + 1)  // 64 positions; every wave writes the same values
             dma_b32(p.posk + kt * FWD_KT, (unsigned)(lane * 4), ldsP + buf * (FWD_KT * 4u));
+        else if (bias_lds)  // BIAS: the tile's 64 bias values; every wave writes the same values
+            dma_b32(bias_head + (int64_t)kt * bias_tile_bytes, bias_voff, lds_addr(sBias) + buf * 256u);
     };
 
     // One 64-key tile held in buffer `cur`.  With PREFETCH the copies of tile `kt_next` into the other
@@ -186,11 +196,34 @@ __global__ __launch_bounds__(FWD_THREADS, D == 128 ? 2 : 3) void fwd_kernel(cons
                 s[j & 1] = T::mfma(ka[j], qreg[j >> 1], j < 2 ? zero16 : s[j & 1]);
                 if (PREFETCH && j < NLOADS) issue_copy(j, kt_next, cur ^ 1);
             }
+            if (PREFETCH) {
+#pragma unroll
+                for (int j = NOP; j < NLOADS; ++j) issue_copy(j, kt_next, cur ^ 1);
+            }
             __builtin_amdgcn_sched_barrier(0);
         }
         __builtin_amdgcn_s_setprio(0);
 
-        if (BIAS) {
+        if (BIAS && PREFETCH && bias_lds) {  // (the ragged last tile is staged without the bias)
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int grp = 0; grp < 4; ++grp) {
+                    const int koff = 32 * kb + 8 * grp + 4 * hi;
+                    f32x4 b4;
+                    if (p.bias_f32) {
+                        b4 = *(const f32x4*)&sBias[cur][koff];
+                    } else {
+                        const u32x2 w = *(const u32x2*)((const char*)sBias[cur] + 2 * koff);
+                        b4[0] = T::to_float((unsigned short)(w[0] & 0xFFFFu));
+                        b4[1] = T::to_float((unsigned short)(w[0] >> 16));
+                        b4[2] = T::to_float((unsigned short)(w[1] & 0xFFFFu));
+                        b4[3] = T::to_float((unsigned short)(w[1] >> 16));
+                    }
+#pragma unroll
+                    for (int x = 0; x < 4; ++x) s[kb][4 * grp + x] = fmaf(s[kb][4 * grp + x], p.scale, b4[x]);
+                }
+        } else if (BIAS) {
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
