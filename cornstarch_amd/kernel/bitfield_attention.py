@@ -153,10 +153,17 @@ class _TilePlan:
         nbytes = _bam_hip.load().bam_ds_workspace_bytes(nheads, pairs)
         if nbytes <= 0 or nbytes > _ds_workspace_limit(self.workspace.device) or nheads * pairs >= 1 << 31:
             return None
-        ws = torch.empty((nbytes,), dtype=torch.uint8, device=self.workspace.device)
+        try:
+            ws = self._allocate(nbytes, self.workspace.device)
+        except torch.cuda.OutOfMemoryError:
+            return None  # no room for it right now: the dQ kernel recomputes what it needs, as without a workspace
         self.struct.ds_workspace = ws.data_ptr()
         self.struct.ds_capacity = pairs
         return ws
+
+    @staticmethod
+    def _allocate(nbytes: int, device) -> torch.Tensor:
+        return torch.empty((nbytes,), dtype=torch.uint8, device=device)
 
     def detach_ds_workspace(self) -> None:
         self.struct.ds_workspace = None

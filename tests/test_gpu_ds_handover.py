@@ -187,3 +187,35 @@ def test_head_dim_64_and_a_zero_limit_keep_the_recomputing_backward():
     plan.detach_ds_workspace()
     assert plan.struct.ds_workspace is None and plan.struct.ds_capacity == 0
     BA.BitfieldUtils.clear_cache()
+
+
+def test_a_workspace_that_cannot_be_allocated_means_recomputation(monkeypatch):
+    # no room for the dS workspace: the backward runs without it (the dQ kernel recomputes) instead of failing
+    d = dev()
+    q, k, v, do = (t.to(d) for t in inputs(1, 517, 4, 2, 128, torch.bfloat16, seed=3))
+    bf = random_bitfield(1, 517, seed=4, pad=5).to(d)
+
+    def grads():
+        BA.BitfieldUtils.clear_cache()
+        qg, kg, vg = (t.clone().requires_grad_(True) for t in (q, k, v))
+        out = BA.bitfield_attn_func(qg, kg, vg, bf)
+        res = torch.autograd.grad(out, (qg, kg, vg), do)
+        torch.cuda.synchronize()
+        return res
+
+    with_ws = grads()
+    calls = []
+
+    def no_memory(nbytes, device):
+        calls.append(nbytes)
+        raise torch.cuda.OutOfMemoryError("no room (test)")
+
+    monkeypatch.setattr(BA._TilePlan, "_allocate", staticmethod(no_memory))
+    without = grads()
+    assert calls and calls[0] == 4 * 8192 * BA.BitfieldUtils.plan_for(
+        BA.BitfieldUtils.materialize_compressed_mask_from_bitfield_mask(bf), bf).ds_pairs()
+    want = O.attention_backward(q.cpu(), k.cpu(), v.cpu(), bf.cpu(), do.cpu())
+    for a, b, w in zip(with_ws, without, want):
+        assert rel_l2(a.float(), b.float()) <= 2e-3
+        assert rel_l2(b.float().cpu(), w) <= GRAD_REL_L2
+    BA.BitfieldUtils.clear_cache()
