@@ -150,6 +150,7 @@ int fill_plan(bam::AttnParams& p, const char* who, const bam_plan* plan, int B, 
     p.fine_ss = plan->fine_stride_s;
     p.order = plan->order;
     p.order_sb = plan->order_stride_b;
+    p.tile_order = plan->ds_tile_order;  // may be null
     // hand-over of dS from dK/dV to dQ: only with a workspace, for the head dim and lengths its kernels cover
     if (plan->ds_workspace != nullptr && plan->ds_entry != nullptr && plan->ds_tile_base != nullptr && p.D == 128 &&
         Sk <= bam::MAX_LIST * 64) {
@@ -322,7 +323,7 @@ namespace {
 // workspace layout: fine | order, each part 256-byte aligned
 struct PlanLayout {
     int64_t fine_ss, fine_sb, order_sb, entry_sb, fine_off, order_off, entry_off, base_off, count_off, bytes;
-    int64_t row_sn, row_sb, col_ss, col_sb, row_off, col_off, bytes_with_bits;
+    int64_t row_sn, row_sb, col_ss, col_sb, row_off, col_off, bytes_with_bits, tile_count_off, tile_order_off;
 };
 PlanLayout plan_layout(int B, int Sq, int Sk) {
     const int64_t num_m = (Sq + 127) / 128, num_n = (Sk + 31) / 32, slots = 4 * num_m;
@@ -337,7 +338,9 @@ PlanLayout plan_layout(int B, int Sq, int Sk) {
     l.entry_off = l.order_off + up(B * slots * 4, 256);
     l.base_off = l.entry_off + up(B * l.entry_sb * 4, 256);
     l.count_off = l.base_off + up(B * ((Sk + 127) / 128) * 4, 256);
-    l.bytes = l.count_off + 256;
+    l.tile_count_off = l.count_off + 256;
+    l.tile_order_off = l.tile_count_off + up(B * ((Sk + 127) / 128) * 4, 256);
+    l.bytes = l.tile_order_off + up(B * ((Sk + 127) / 128) * 4, 256);
     // the packed mask of bam_mask_tile_plan: rows padded to 128, keys to 128, 32-key blocks to an even number
     l.row_sn = num_m * 128;
     l.row_sb = ((num_n + 1) & ~(int64_t)1) * l.row_sn;
@@ -385,6 +388,7 @@ int place_plan(const char* who, void* workspace, int64_t workspace_bytes, int B,
     plan->ds_entry_stride_b = l.entry_sb;
     plan->ds_tile_base = (const int32_t*)(w + l.base_off);
     plan->ds_count = (const int32_t*)(w + l.count_off);
+    plan->ds_tile_order = (int64_t)B * ((Sk + 127) / 128) <= 1024 ? (const int32_t*)(w + l.tile_order_off) : nullptr;
     plan->ds_workspace = nullptr;
     plan->ds_capacity = 0;
     plan->row_bits = with_bits ? (const uint32_t*)(w + l.row_off) : nullptr;
@@ -401,11 +405,13 @@ int place_plan(const char* who, void* workspace, int64_t workspace_bytes, int B,
 }
 
 // second launch of every plan builder: numbers the (slice, 128-key tile) pairs that have work
-int number_pairs(const char* who, const bam_plan* plan, void* stream) {
+int number_pairs(const char* who, const bam_plan* plan, const PlanLayout& l, void* workspace, void* stream) {
     return launched(bam::launch_ds_entries(plan->fine, plan->fine_stride_b, plan->fine_stride_s, plan->B, plan->Sq, plan->Sk,
                                            const_cast<int*>(plan->ds_entry), plan->ds_entry_stride_b,
                                            const_cast<int*>(plan->ds_tile_base),
                                            const_cast<int*>(plan->ds_count),
+                                           (int*)((char*)workspace + l.tile_count_off),
+                                           const_cast<int*>(plan->ds_tile_order),
                                            (hipStream_t)stream),
                     who);
 }
@@ -426,7 +432,7 @@ int bam_tile_plan(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int64_t
                                            l.fine_sb, l.fine_ss, (int*)(w + l.order_off), l.order_sb,
                                            (int*)(w + l.count_off), B, S, (hipStream_t)stream),
                      "bam_tile_plan"));
-    return number_pairs("bam_tile_plan", plan, stream);
+    return number_pairs("bam_tile_plan", plan, l, workspace, stream);
 }
 
 int bam_tile_plan_static(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int64_t flags_stride_b,
@@ -469,7 +475,7 @@ int bam_plan_indexed(const bam_index_view* iv, void* workspace, int64_t workspac
                                               (uint8_t*)(w + l.fine_off), l.fine_sb, l.fine_ss, (int*)(w + l.order_off),
                                               l.order_sb, (int*)(w + l.count_off), B, (hipStream_t)stream),
                      "bam_plan_indexed"));
-    return number_pairs("bam_plan_indexed", plan, stream);
+    return number_pairs("bam_plan_indexed", plan, l, workspace, stream);
 }
 
 int bam_mask_tile_plan(const uint8_t* mask, int8_t* flags, int64_t flags_stride_b, int64_t flags_stride_m, void* workspace,
@@ -487,7 +493,7 @@ int bam_mask_tile_plan(const uint8_t* mask, int8_t* flags, int64_t flags_stride_
                                                 (unsigned*)(w + l.col_off), l.col_sb, l.col_ss, B, Sq, Sk,
                                                 (hipStream_t)stream),
                      "bam_mask_tile_plan"));
-    return number_pairs("bam_mask_tile_plan", plan, stream);
+    return number_pairs("bam_mask_tile_plan", plan, l, workspace, stream);
 }
 
 int64_t bam_ds_workspace_bytes(int Hq, int64_t pairs) {

@@ -100,8 +100,13 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
     const int unit = blockIdx.x;
     const int hk = unit % p.Hkv;
     const int ub = unit / p.Hkv;
-    const int b = ub % p.B;
-    const int nt = ub / p.B;  // early key tiles (most queries under causality) first
+    int b = ub % p.B;
+    int nt = ub / p.B;  // early key tiles (most queries under causality) first
+    if (p.tile_order != nullptr) {  // with a plan: the tiles by falling amount of work, whatever the mask looks like
+        const int code = p.tile_order[ub];
+        b = code / p.num_kt;
+        nt = code - b * p.num_kt;
+    }
 
     const int ns_total = (Sq + 31) >> 5;
     // first pass (usually the only one): the last MAX_SLICE_LIST slices

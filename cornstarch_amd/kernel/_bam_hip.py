@@ -62,6 +62,7 @@ class Plan(ctypes.Structure):
         ("ds_entry_stride_b", ctypes.c_int64),
         ("ds_tile_base", ctypes.c_void_p),
         ("ds_count", ctypes.c_void_p),
+        ("ds_tile_order", ctypes.c_void_p),
         ("ds_workspace", ctypes.c_void_p),
         ("ds_capacity", ctypes.c_int64),
         ("row_bits", ctypes.c_void_p),

@@ -116,6 +116,9 @@ typedef struct bam_plan {
     int64_t ds_entry_stride_b;
     const int32_t* ds_tile_base; /* device, (B, ceil(Sk/128)): number of the first pair of each key tile */
     const int32_t* ds_count;   /* device, one int: how many such pairs there are */
+    const int32_t* ds_tile_order; /* device, B * ceil(Sk/128) ints, or null (more than 1024 key tiles): the key tiles
+                                     (code b * ceil(Sk/128) + t) by falling number of pairs, the order in which the
+                                     dK/dV kernel takes its workgroups so that the longest start first */
     void* ds_workspace;        /* device, at least bam_ds_workspace_bytes(Hq, pairs) bytes, 16-byte aligned */
     int64_t ds_capacity;       /* pairs the workspace has room for: at least *ds_count */
     /* Materialized masks only (bam_mask_tile_plan; null otherwise): the mask packed to bits, once per orientation, so

@@ -66,6 +66,10 @@ def test_pair_numbering_against_the_fine_classes(S):
     assert all(blocks[i][0] + blocks[i][1] == blocks[i + 1][0] for i in range(len(blocks) - 1))
     assert not blocks or (blocks[0][0] == 0 and blocks[-1][0] + blocks[-1][1] == int(has.sum()))
     assert plan.ds_pairs() == int(has.sum())
+    # the order in which the dK/dV kernel takes the key tiles: every (batch, tile) once, most pairs first, ties by code
+    order = torch.as_strided(i32, (3 * nkt,), (1,), (st.ds_tile_order - ws.data_ptr()) // 4).cpu().tolist()
+    counts = has.sum(dim=1).reshape(-1).tolist()                                 # by code b * nkt + t
+    assert order == sorted(range(3 * nkt), key=lambda c: (-counts[c], c))
     BA.BitfieldUtils.clear_cache()
 
 
