@@ -51,7 +51,7 @@ struct AttnParams {
     int bias_vec;              // every group of four keys starting at a multiple of four is one aligned, in-range access
     const int8_t* flags;       // (B, num_m, num_n)
     int64_t flags_sb, flags_sm;
-    // Optional plan (plain bitfield attention only; null = none).  fine: class 0 / 1 / 2 of every 32-row x 32-key
+    // Optional plan (null = none; every mask mode has a builder of its own).  fine: class 0 / 1 / 2 of every 32-row x 32-key
     // tile, (B, 4 * num_m, fine_ss) bytes; order: the 32-row slices of each sequence sorted so that four
     // neighbours need about the same keys, heaviest first, (B, 4 * num_m) ints, -1 = no slice.
     const uint8_t* fine;

@@ -74,9 +74,14 @@ class _MaskPlan:
         num_m, num_n = -(-seqlen_q // BLOCK_M), -(-seqlen_k // BLOCK_N)
         with torch.cuda.device(device):
             ws_bytes = _bam_hip.load().bam_mask_plan_workspace_bytes(batch, seqlen_q, seqlen_k)
+            workspace = None
             if ws_bytes > 0:
+                try:
+                    workspace = torch.empty((ws_bytes,), dtype=torch.uint8, device=device)
+                except torch.cuda.OutOfMemoryError:
+                    workspace = None  # no room for a quarter of the mask: flags only, the kernels read the mask bytes
+            if workspace is not None:
                 flags = torch.empty((batch, num_m, num_n), dtype=torch.int8, device=device)
-                workspace = torch.empty((ws_bytes,), dtype=torch.uint8, device=device)
                 struct = _bam_hip.Plan()
                 _bam_hip.call(
                     "bam_mask_tile_plan", mask.data_ptr(), flags.data_ptr(), flags.stride(0), flags.stride(1),
