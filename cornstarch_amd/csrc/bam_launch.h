@@ -119,9 +119,9 @@ int launch_mask_tile_plan(const uint8_t* mask, int8_t* flags, int64_t flags_stri
                           int64_t col_bits_sb, int64_t col_bits_ss, int B, int Sq, int Sk, hipStream_t stream);
 // Numbers the (slice, 128-key tile) pairs that have work: entry (B, 4 * num_m, ceil(Sk/128)) ints, -1 = none.
 // tile_base (B, ceil(Sk/128)) ints: number of the first pair of each key tile (pairs are numbered tile by tile).
-// count[0] (pairs) and count[1] (finished workgroups) must be zero when the kernel starts (the plan kernels reset
-// them).  tile_count (B, ceil(Sk/128)) scratch and tile_order (B * ceil(Sk/128)): the key tiles by falling number of
-// pairs; both may be null, and no order is written beyond 1024 tiles.
+// *count must be zero when the kernel starts (the plan kernels reset it).  tile_count (B, ceil(Sk/128)) scratch and
+// tile_order (B * ceil(Sk/128)): the key tiles by falling number of pairs, written by a second small launch; both may
+// be null, and no order is written beyond 1024 tiles.
 int launch_ds_entries(const uint8_t* fine, int64_t fine_sb, int64_t fine_ss, int B, int Sq, int Sk, int* entry,
                       int64_t entry_sb, int* tile_base, int* count, int* tile_count, int* tile_order, hipStream_t stream);
 int launch_fwd(const AttnParams& p, int dtype, hipStream_t stream);

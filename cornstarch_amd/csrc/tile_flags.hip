@@ -126,7 +126,7 @@ __global__ __launch_bounds__(FLAG_WAVES * 64) void tile_flags_kernel(const int64
                                                                     int* __restrict__ pair_count) {
     // (the pair counter of the numbering kernel that follows in the stream starts from zero)
     if (FINE && pair_count != nullptr && blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0 && threadIdx.x == 0)
-        pair_count[0] = pair_count[1] = 0;  // pairs, finished numbering workgroups
+        *pair_count = 0;
     if (FINE && (int)blockIdx.x >= flag_blocks_x) {  // the workgroups that sort the slices (see slice_order_part)
         const int part = blockIdx.y;
         if (part * 256 < 4 * (int)gridDim.y)
@@ -341,7 +341,7 @@ __global__ __launch_bounds__(FLAG_WAVES * 64) void indexed_plan_kernel(
     int* __restrict__ pair_count) {
     const int b = blockIdx.z;
     const int64_t* qrow = qbits + (int64_t)b * qbits_sb;
-    if (pair_count != nullptr && blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0 && threadIdx.x == 0) pair_count[0] = pair_count[1] = 0;
+    if (pair_count != nullptr && blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0 && threadIdx.x == 0) *pair_count = 0;
     if ((int)blockIdx.x >= flag_blocks_x) {
         const int part = blockIdx.y;
         const int ns = (Sq + 31) / 32, slots = 4 * (int)gridDim.y;
@@ -431,7 +431,7 @@ __global__ __launch_bounds__(256) void mask_tile_plan_kernel(const uint8_t* __re
                                                              int64_t row_bits_sn, unsigned* __restrict__ col_bits,
                                                              int64_t col_bits_sb, int64_t col_bits_ss) {
     const int b = blockIdx.z, m = blockIdx.y, tid = threadIdx.x, lane = tid & 63;
-    if (pair_count != nullptr && blockIdx.x == 0 && m == 0 && b == 0 && tid == 0) pair_count[0] = pair_count[1] = 0;
+    if (pair_count != nullptr && blockIdx.x == 0 && m == 0 && b == 0 && tid == 0) *pair_count = 0;
     if (blockIdx.x == 0 && tid < 4) {
         const int ns = (Sq + 31) / 32, slot = 4 * m + tid;
         order[(int64_t)b * order_sb + slot] = slot < ns ? ns - 1 - slot : -1;
@@ -505,14 +505,12 @@ int launch_mask_tile_plan(const uint8_t* mask, int8_t* flags, int64_t flags_stri
 // Numbering of the (32-row slice, 128-key tile) pairs that have work, for the backward that hands dS from the dK/dV
 // kernel to the dQ kernel through memory.  The pairs of one key tile -- exactly the slices a dK/dV workgroup lists --
 // get consecutive numbers, by ascending slice; the tiles themselves take their blocks of numbers in the order their
-// workgroups arrive (one atomic add per tile on count[0], which the plan kernels reset):
+// workgroups arrive (one atomic add per tile on *count, which the plan kernels reset):
 //   entry[b][s][t]  = number of pair (b, s, t), or -1 where its four classes are all "empty"  (what the dQ kernel looks up)
 //   tile_base[b][t] = number of the first pair of key tile (b, t)                             (what dK/dV starts from)
-//   count[0]        = how many pairs there are.
+//   *count          = how many pairs there are.
 // Which tile gets which block of numbers only decides where a record sits in the workspace, never a result.
-// tile_order (optional): the key tiles (code b * nkt + t) sorted by their number of pairs, most first -- the order in
-// which the dK/dV kernel takes them, so that the long workgroups start first whatever the mask looks like.  It is
-// written by whichever workgroup finishes last (count[1] counts the finished ones; reset by the plan kernels too).
+// tile_count[b][t] (optional) = number of pairs of key tile (b, t): what tile_order_kernel ranks the tiles by.
 // One workgroup per (key tile, batch); thread = slice, 256 slices per sweep.
 constexpr int DS_NUM_THREADS = 256;
 constexpr int DS_MAX_ORDERED_TILES = 1024;
@@ -520,10 +518,9 @@ __global__ __launch_bounds__(DS_NUM_THREADS) void ds_entries_kernel(const uint8_
                                                                    int64_t fine_ss, int slots, int nkt, int num_n,
                                                                    int* __restrict__ entry, int64_t entry_sb,
                                                                    int* __restrict__ tile_base, int* __restrict__ count,
-                                                                   int* tile_count, int* __restrict__ tile_order) {
+                                                                   int* __restrict__ tile_count) {
     __shared__ int wave_sum[DS_NUM_THREADS / 64];
-    __shared__ int s_base, s_last;
-    __shared__ int s_cnt[DS_MAX_ORDERED_TILES];
+    __shared__ int s_base;
     const int t = blockIdx.x, b = blockIdx.y;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const uint8_t* col = fine + (int64_t)b * fine_sb + 4 * t;
@@ -544,7 +541,7 @@ __global__ __launch_bounds__(DS_NUM_THREADS) void ds_entries_kernel(const uint8_
         const int base = atomicAdd(count, total);
         s_base = base;
         tile_base[(int64_t)b * nkt + t] = base;
-        if (tile_order != nullptr) tile_count[b * nkt + t] = total;
+        if (tile_count != nullptr) tile_count[b * nkt + t] = total;
     }
     __syncthreads();
     int next = s_base;
@@ -564,32 +561,44 @@ __global__ __launch_bounds__(DS_NUM_THREADS) void ds_entries_kernel(const uint8_
         if (sl < slots) out[(int64_t)sl * nkt] = h ? next + before + __popcll(bal & ((1ull << lane) - 1ull)) : -1;
         next += all;
     }
-    if (tile_order == nullptr) return;
-    // the workgroup that finishes last ranks the tiles by their counts (ties: lower code first)
-    const int n_tiles = nkt * gridDim.y;
-    if (tid == 0) {
-        __threadfence();  // this workgroup's tile_count is visible before it is counted as finished
-        s_last = atomicAdd(count + 1, 1) == n_tiles - 1;
-    }
+}
+
+// The key tiles (code b * nkt + t) sorted by their number of pairs, most first (ties: lower code first): the order in
+// which the dK/dV kernel takes them, so that the long workgroups start first whatever the mask looks like.
+// 64 tiles per workgroup, four threads per tile, each comparing against a quarter of all counts (staged in LDS).
+__global__ __launch_bounds__(256) void tile_order_kernel(const int* __restrict__ tile_count, int n_tiles,
+                                                         int* __restrict__ tile_order) {
+    __shared__ __attribute__((aligned(16))) int s_cnt[DS_MAX_ORDERED_TILES];
+    const int tid = threadIdx.x;
+    const int padded = (n_tiles + 15) & ~15;
+    for (int i = tid; i < padded; i += 256) s_cnt[i] = i < n_tiles ? tile_count[i] : -1;  // padding ranks behind everything
     __syncthreads();
-    if (!s_last) return;
-    __threadfence();
-    for (int i = tid; i < n_tiles; i += DS_NUM_THREADS) s_cnt[i] = __atomic_load_n(tile_count + i, __ATOMIC_RELAXED);
-    __syncthreads();
-    for (int i = tid; i < n_tiles; i += DS_NUM_THREADS) {
-        const int c = s_cnt[i];
-        int rank = 0;
-        for (int j = 0; j < n_tiles; ++j) rank += (s_cnt[j] > c) | ((s_cnt[j] == c) & (j < i));
-        tile_order[rank] = i;
+    const int i = blockIdx.x * 64 + (tid >> 2), sub = tid & 3;
+    const int c = i < n_tiles ? s_cnt[i] : 0;
+    int rank = 0;
+    // thread `sub` of a tile takes the groups of four counts number sub, sub + 4, ...
+    for (int j4 = sub; 4 * j4 < padded; j4 += 4) {
+        const int4 v = *(const int4*)&s_cnt[4 * j4];
+        const int j = 4 * j4;
+        rank += (v.x > c) | ((v.x == c) & (j < i));
+        rank += (v.y > c) | ((v.y == c) & (j + 1 < i));
+        rank += (v.z > c) | ((v.z == c) & (j + 2 < i));
+        rank += (v.w > c) | ((v.w == c) & (j + 3 < i));
     }
+    rank += __shfl_xor(rank, 1);
+    rank += __shfl_xor(rank, 2);
+    if (sub == 0 && i < n_tiles) tile_order[rank] = i;
 }
 
 int launch_ds_entries(const uint8_t* fine, int64_t fine_sb, int64_t fine_ss, int B, int Sq, int Sk, int* entry,
                       int64_t entry_sb, int* tile_base, int* count, int* tile_count, int* tile_order, hipStream_t stream) {
     const int slots = 4 * ((Sq + BLOCK_M - 1) / BLOCK_M), nkt = (Sk + 127) / 128, num_n = (Sk + BLOCK_N - 1) / BLOCK_N;
-    if ((int64_t)nkt * B > DS_MAX_ORDERED_TILES) tile_order = nullptr;
+    const int n_tiles = nkt * B;
+    if (n_tiles > DS_MAX_ORDERED_TILES || tile_count == nullptr) tile_order = nullptr;
     hipLaunchKernelGGL(ds_entries_kernel, dim3(nkt, B), dim3(DS_NUM_THREADS), 0, stream, fine, fine_sb, fine_ss, slots, nkt,
-                       num_n, entry, entry_sb, tile_base, count, tile_count, tile_order);
+                       num_n, entry, entry_sb, tile_base, count, tile_order != nullptr ? tile_count : nullptr);
+    if (tile_order != nullptr)
+        hipLaunchKernelGGL(tile_order_kernel, dim3((n_tiles + 63) / 64), dim3(256), 0, stream, tile_count, n_tiles, tile_order);
     return (int)hipGetLastError();
 }
 
