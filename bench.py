@@ -263,7 +263,8 @@ def run_neighbouring_entry_points(dev, steps):
     """C2-shaped records for the entry points either side of plain bitfield attention, forward + backward each:
     a context-parallel shard (index tensors: rank 0 of a two-rank zigzag split, 4096 rows against all 8192 keys,
     through `_bitfield_attn_forward` / `_bitfield_attn_backward`), the materialized C2 mask through `flash_attn_func`,
-    and an ALiBi-like bias vector through `bitfield_attn_func`.  Effective TFLOP/s over each case's unmasked pairs."""
+    and an ALiBi-like bias vector through `bitfield_attn_func`.  Effective TFLOP/s over each case's unmasked pairs.
+    Last, the single-token decode step (HBM-bound: rate at which the key / value cache is read)."""
     import torch
 
     from cornstarch_amd import workloads as W
@@ -353,6 +354,20 @@ def run_neighbouring_entry_points(dev, steps):
         "steps": steps,
     }
     BA.BitfieldUtils.clear_cache()
+    del qg, kg, vg, bias
+    # --- single-token decode step of the HF adapter (eval mode): 8 sequences, a cache of C2's length and head layout
+    from cornstarch_amd.kernel import interface as I
+
+    Bd = 8
+    qd = torch.randn(Bd, w.Hq, 1, w.D, device=dev, dtype=torch.bfloat16)
+    kd = torch.randn(Bd, w.Hkv, w.S, w.D, device=dev, dtype=torch.bfloat16)
+    vd = torch.randn(Bd, w.Hkv, w.S, w.D, device=dev, dtype=torch.bfloat16)
+    ms = timed(lambda: I._decode_attention(qd, kd, vd, None, 0.0, None, None))
+    cache_bytes = 2 * Bd * w.S * w.Hkv * w.D * 2
+    out["decode_step"] = {
+        "ms_per_step": round(ms, 4), "batch": Bd, "cache_len": w.S, "cache_gbytes_per_s": round(cache_bytes / (ms * 1e-3) / 1e9, 1),
+        "hbm_frac": round(cache_bytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, 4), "steps": steps,
+    }
     return out
 
 

@@ -674,10 +674,17 @@ int bam_bwd_dq_indexed(const void* q, const void* k, const void* v, const void* 
     return launched(launch_dq(p, dtype, stream), "bam_bwd_dq_indexed");
 }
 
+int64_t bam_decode_workspace_bytes(int B, int Sk, int Hq, int Hkv, int D, int window) {
+    if (B <= 0 || Sk <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0 || D <= 0 || window < 0) return 0;
+    int nsplit = 1, tps = 1, rgs = 1;
+    bam::decode_split_plan(B, Hq, Hkv, Sk, window, &nsplit, &tps, &rgs);
+    return nsplit > 1 ? (int64_t)B * Hq * nsplit * (D + 2) * 4 : 0;
+}
+
 int bam_decode(const void* q, const void* k, const void* v, void* o, int64_t q_stride_b, int64_t q_stride_h,
                int64_t k_stride_b, int64_t k_stride_s, int64_t k_stride_h, int64_t v_stride_b, int64_t v_stride_s,
                int64_t v_stride_h, int64_t o_stride_b, int64_t o_stride_h, int B, int Sk, int Hq, int Hkv, int D, float scale,
-               int dtype, int window, float softcap, void* stream) {
+               int dtype, int window, float softcap, void* workspace, int64_t workspace_bytes, void* stream) {
     BAM_TRY(check_problem(B, 1, Sk, Hq, Hkv, D, dtype));
     BAM_TRY(check_half_tensor("k", k, k_stride_b, k_stride_s, k_stride_h));
     BAM_TRY(check_half_tensor("v", v, v_stride_b, v_stride_s, v_stride_h));
@@ -689,6 +696,19 @@ int bam_decode(const void* q, const void* k, const void* v, void* o, int64_t q_s
     if (!(softcap >= 0.f)) return fail(BAM_ERR_INVALID_ARGUMENT, "bam_decode: softcap must be >= 0 (0 = none), got %g", softcap);
     if ((int64_t)B * Hq > 0x7FFFFFFFll) return fail(BAM_ERR_UNSUPPORTED, "bam_decode: grid too large");
     bam::DecodeParams p = {};
+    bam::decode_split_plan(B, Hq, Hkv, Sk, window, &p.nsplit, &p.tiles_per_split, &p.row_groups);
+    if ((int64_t)B * p.row_groups > 65535 || Hkv > 65535)
+        return fail(BAM_ERR_UNSUPPORTED, "bam_decode: grid too large (B = %d, Hkv = %d)", B, Hkv);
+    if (p.nsplit > 1) {
+        const int64_t need = bam_decode_workspace_bytes(B, Sk, Hq, Hkv, D, window);
+        if (workspace == nullptr || workspace_bytes < need)
+            return fail(BAM_ERR_INVALID_ARGUMENT, "bam_decode: workspace of %lld bytes, %lld needed",
+                        (long long)(workspace == nullptr ? 0 : workspace_bytes), (long long)need);
+        if (reinterpret_cast<uintptr_t>(workspace) & 15u)
+            return fail(BAM_ERR_INVALID_ARGUMENT, "bam_decode: workspace is not 16-byte aligned");
+        p.ws_o = (float*)workspace;
+        p.ws_ml = p.ws_o + (int64_t)B * Hq * p.nsplit * D;
+    }
     p.q = q;
     p.k = k;
     p.v = v;

@@ -91,7 +91,14 @@ struct DecodeParams {
     int B, Sk, Hq, Hkv, D;
     int window;                    // > 0: only the last `window` keys are attended to
     float scale, softcap;          // softcap > 0: scores become softcap * tanh(score / softcap)
+    // How the keys are split over workgroups (decode_split_plan) and where the splits leave their partial results:
+    // ws_o (B, Hq, nsplit, D) unnormalized outputs, ws_ml (B, Hq, nsplit, 2) maximum (log2 domain) and sum; unused
+    // when nsplit == 1.  row_groups = ceil((Hq / Hkv) / 32): q heads of one kv head per workgroup, 32 at a time.
+    float* ws_o;
+    float* ws_ml;
+    int nsplit, tiles_per_split, row_groups;
 };
+void decode_split_plan(int B, int Hq, int Hkv, int Sk, int window, int* nsplit, int* tiles_per_split, int* row_groups);
 
 int launch_tile_flags(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int64_t flags_stride_b,
                       int64_t flags_stride_m, int B, int S, hipStream_t stream);

@@ -5,141 +5,235 @@
 //   s_j = scale * q.k_j ;  s_j = softcap * tanh(s_j / softcap)  (if softcap > 0)
 //   keys j < Sk - window are dropped                            (if 0 < window < Sk)
 //   o = softmax(s) V
-// No bitfield is consulted.  The kernel is bound by reading K and V once per q head (HBM / L2), not by arithmetic.
+// No bitfield is consulted.
+//
+// The step is bound by reading K and V once; there is one query row per head, so the parallelism has to come from the
+// keys.  decode_split_kernel: one wave per (range of 32-key tiles, kv head, batch element); the q heads of the kv
+// head (up to 32 per workgroup) are the 32 "query rows" of the attention kernels' S^T = K Q^T layout, so the tile is
+// read once for all of them:
+//   S^T (32 keys x 32 heads) = K Q^T with the K rows as the A operand straight from global memory,
+//   a lane owns one head (softmax state = per-lane scalars), P^T feeds O^T = V^T P^T from registers,
+//   V^T comes from the V tile (copied global -> LDS) through the transposing LDS read.
+// Every split writes its unnormalized output, maximum and sum for the heads that exist; decode_combine_kernel merges
+// them.  A single split writes the result itself.
 #include "bam_common.h"
 #include "bam_launch.h"
+#include "bam_tiles.h"
 
 namespace bam {
 
-constexpr int DEC_THREADS = 256;
-constexpr int DEC_CHUNK = 1024;  // keys whose scores sit in LDS at a time
-
-__device__ __forceinline__ float wave_max(float x) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) x = fmaxf(x, __shfl_xor(x, off));
-    return x;
-}
-__device__ __forceinline__ float wave_sum(float x) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) x += __shfl_xor(x, off);
-    return x;
-}
+constexpr int DEC_KT = 32;  // keys per tile
 
 template <typename T, int D>
-__global__ __launch_bounds__(DEC_THREADS) void decode_kernel(const DecodeParams p) {
-    constexpr int LPR = D / 8;               // lanes that share one key row, 16 bytes each
-    constexpr int NK = DEC_THREADS / LPR;    // keys in flight per sweep
-    __shared__ float sQ[D];
-    __shared__ float sS[DEC_CHUNK];
-    __shared__ float sRed[DEC_THREADS / 64];
-    __shared__ float sAcc[NK][D + 1];
+__global__ __launch_bounds__(64) void decode_split_kernel(const DecodeParams p) {
+    constexpr int NCH = D / 8, KK = D / 16, DB = D / 32;
+    __shared__ u32x4 sV[DEC_KT * NCH];
+    __shared__ __attribute__((aligned(16))) unsigned short sQ[32 * D];
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int b = blockIdx.x / p.Hq, h = blockIdx.x % p.Hq, hk = h / (p.Hq / p.Hkv);
-    const int dg = tid % LPR, kl = tid / LPR;
-
-    if (tid < D)
-        sQ[tid] = T::to_float(((const unsigned short*)p.q)[(int64_t)b * p.q_sb + (int64_t)h * p.q_sh + tid]);
-    __syncthreads();
-    float qv[8];
-#pragma unroll
-    for (int x = 0; x < 8; ++x) qv[x] = sQ[8 * dg + x];
-
-    const char* kbase = (const char*)p.k + 2 * ((int64_t)b * p.k_sb + (int64_t)hk * p.k_sh) + 16 * dg;
-    const char* vbase = (const char*)p.v + 2 * ((int64_t)b * p.v_sb + (int64_t)hk * p.v_sh) + 16 * dg;
+    const int lane = threadIdx.x, hi = lane >> 5, l32 = lane & 31, half16 = (lane >> 4) & 1;
+    const int split = blockIdx.x, hk = blockIdx.y;
+    const int b = blockIdx.z / p.row_groups, rg = blockIdx.z % p.row_groups;
+    const int G = p.Hq / p.Hkv;
+    const int h0 = hk * G + 32 * rg;         // first q head of this workgroup
+    const int rows = min(32, G - 32 * rg);   // q heads it holds
     const int first = (p.window > 0 && p.window < p.Sk) ? p.Sk - p.window : 0;
+    const int n_tiles = (p.Sk - first + DEC_KT - 1) / DEC_KT;
+    const int t0 = split * p.tiles_per_split, t1 = min(n_tiles, t0 + p.tiles_per_split);
 
-    auto block_reduce = [&](float x, bool is_max) {
-        x = is_max ? wave_max(x) : wave_sum(x);
-        __syncthreads();  // sRed is free again
-        if (lane == 0) sRed[wave] = x;
-        __syncthreads();
-        float r = sRed[0];
-#pragma unroll
-        for (int w = 1; w < DEC_THREADS / 64; ++w) r = is_max ? fmaxf(r, sRed[w]) : r + sRed[w];
-        return r;
-    };
-
-    float m = -INFINITY, l = 0.f, acc[8];
-#pragma unroll
-    for (int x = 0; x < 8; ++x) acc[x] = 0.f;
-
-    for (int c0 = first; c0 < p.Sk; c0 += DEC_CHUNK) {
-        const int n = min(DEC_CHUNK, p.Sk - c0);
-        // scores of the chunk: LPR neighbouring lanes share a key
-        for (int j0 = 0; j0 < n; j0 += NK) {
-            const int j = j0 + kl;
-            float part = 0.f;
-            if (j < n) {
-                const u32x4 kv = *(const u32x4*)(kbase + 2 * (int64_t)(c0 + j) * p.k_ss);
-#pragma unroll
-                for (int x = 0; x < 4; ++x) {
-                    part = fmaf(T::to_float((unsigned short)(kv[x] & 0xFFFFu)), qv[2 * x], part);
-                    part = fmaf(T::to_float((unsigned short)(kv[x] >> 16)), qv[2 * x + 1], part);
-                }
-            }
-#pragma unroll
-            for (int off = LPR / 2; off > 0; off >>= 1) part += __shfl_xor(part, off);
-            if (j < n && dg == 0) {
-                float s = part * p.scale;
-                if (p.softcap > 0.f) s = p.softcap * tanhf(s / p.softcap);
-                sS[j] = s;
-            }
-        }
-        __syncthreads();
-        float cm = -INFINITY;
-        for (int j = tid; j < n; j += DEC_THREADS) cm = fmaxf(cm, sS[j]);
-        cm = block_reduce(cm, true);
-        const float mnew = fmaxf(m, cm);            // finite: every chunk holds at least one key
-        const float alpha = __expf(m - mnew);       // 0 for the first chunk
-        float ls = 0.f;
-        for (int j = tid; j < n; j += DEC_THREADS) {
-            const float e = __expf(sS[j] - mnew);
-            sS[j] = e;
-            ls += e;
-        }
-        ls = block_reduce(ls, false);               // (its barriers also publish the probabilities)
-        l = l * alpha + ls;
-        m = mnew;
-#pragma unroll
-        for (int x = 0; x < 8; ++x) acc[x] *= alpha;
-        for (int j = kl; j < n; j += NK) {
-            const float pj = sS[j];
-            const u32x4 vv = *(const u32x4*)(vbase + 2 * (int64_t)(c0 + j) * p.v_ss);
-#pragma unroll
-            for (int x = 0; x < 4; ++x) {
-                acc[2 * x] = fmaf(pj, T::to_float((unsigned short)(vv[x] & 0xFFFFu)), acc[2 * x]);
-                acc[2 * x + 1] = fmaf(pj, T::to_float((unsigned short)(vv[x] >> 16)), acc[2 * x + 1]);
-            }
-        }
-        __syncthreads();  // everybody is done with this chunk's probabilities
+    // ---- Q: rows = heads, zero rows past the last head; element-wise loads (q is only 2-byte aligned) ----
+    for (int i = lane; i < 32 * D; i += 64) {
+        const int r = i / D, d = i % D;
+        sQ[i] = r < rows ? ((const unsigned short*)p.q)[(int64_t)b * p.q_sb + (int64_t)(h0 + r) * p.q_sh + d] : (unsigned short)0;
     }
-#pragma unroll
-    for (int x = 0; x < 8; ++x) sAcc[kl][8 * dg + x] = acc[x];
     __syncthreads();
-    if (tid < D) {
-        float r = 0.f;
-        for (int k2 = 0; k2 < NK; ++k2) r += sAcc[k2][tid];
-        r /= l;
-        unsigned short* op = (unsigned short*)p.o + (int64_t)b * p.o_sb + (int64_t)h * p.o_sh + tid;
-        *op = (unsigned short)(T::pack2(r, 0.f) & 0xFFFFu);
+    u32x4 qreg[KK];
+#pragma unroll
+    for (int kk = 0; kk < KK; ++kk) qreg[kk] = *(const u32x4*)&sQ[l32 * D + 16 * kk + 8 * hi];
+
+    const char* kbase = (const char*)p.k + 2 * ((int64_t)b * p.k_sb + (int64_t)hk * p.k_sh);
+    const char* vbase = (const char*)p.v + 2 * ((int64_t)b * p.v_sb + (int64_t)hk * p.v_sh);
+    TileStage<D, DEC_KT, 64> stV;
+    stV.setup(2 * p.v_ss, lane);
+
+    f32x16 o[DB];
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o[db][i] = 0.f;
+    f32x16 zero16;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) zero16[i] = 0.f;
+    float m_i = -INFINITY, l_i = 0.f;  // maximum in the log2 domain; this lane's share of the sum (16 of 32 keys)
+
+    for (int t = t0; t < t1; ++t) {
+        const int key0 = first + t * DEC_KT;
+        const int nvalid = min(DEC_KT, p.Sk - key0);
+        // K rows of the tile as the A operand (rows past the end repeat the last one; their scores are masked below)
+        const char* krow = kbase + 2 * (int64_t)(key0 + min(l32, nvalid - 1)) * p.k_ss;
+        u32x4 ka[KK];
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) ka[kk] = *(const u32x4*)(krow + (2 * kk + hi) * 16);
+        // V tile -> LDS (zero rows past the end); the previous tile's reads of it have all been consumed by MFMAs
+        wait_lds();
+        stV.load(vbase + 2 * (int64_t)key0 * p.v_ss, sV, nvalid, lane);
+
+        f32x16 s = zero16;
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) s = T::mfma(ka[kk], qreg[kk], s);
+
+        // scores in the log2 domain: scale, cap, keys past the end
+        float mx = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int koff = 8 * (i >> 2) + 4 * hi + (i & 3);
+            float x = s[i] * p.scale;
+            if (p.softcap > 0.f) x = p.softcap * tanhf(x / p.softcap);
+            x = koff < nvalid ? x * LOG2E : -INFINITY;
+            s[i] = x;
+            mx = fmaxf(mx, x);
+        }
+        const float mloc = half_swap_max(mx);        // finite: every tile holds at least one key
+        const float mnew = fmaxf(m_i, mloc);
+        const float alpha = __builtin_amdgcn_exp2f(m_i - mnew);  // 0 for the first tile
+        m_i = mnew;
+        float ls = 0.f;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            s[i] = __builtin_amdgcn_exp2f(s[i] - mnew);
+            ls += s[i];
+        }
+        l_i = l_i * alpha + ls;
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) o[db][i] *= alpha;
+        u32x4 pb[2];
+#pragma unroll
+        for (int h2 = 0; h2 < 2; ++h2) pb[h2] = pack8<T>(s, 8 * h2);
+
+        wait_async();   // the V tile has landed (one wave: no barrier needed, LDS reads follow in program order)
+        wait_lds();     // ... and so have the synchronous stores of a ragged tile
+#pragma unroll
+        for (int h2 = 0; h2 < 2; ++h2)
+#pragma unroll
+            for (int db = 0; db < DB; ++db) {
+                const u32x4 va = lds_read_transposed<D>(sV, lane, 16 * h2 + 4 * hi, 32 * db + 16 * half16);
+                o[db] = T::mfma(va, pb[h2], o[db]);
+            }
     }
+
+    // ---- this split's result for head h0 + l32: O^T fragment register i of block db <-> column 32 db + 8 (i/4) + 4 hi + i%4
+    const float ltot = half_swap_sum(l_i);
+    if (l32 >= rows) return;
+    const int h = h0 + l32;
+    if (p.nsplit == 1) {
+        const float inv = 1.f / ltot;
+        unsigned short* op = (unsigned short*)p.o + (int64_t)b * p.o_sb + (int64_t)h * p.o_sh;
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int i = 0; i < 16; ++i)
+                op[32 * db + 8 * (i >> 2) + 4 * hi + (i & 3)] = (unsigned short)(T::pack2(o[db][i] * inv, 0.f) & 0xFFFFu);
+        return;
+    }
+    const int64_t rec = ((int64_t)b * p.Hq + h) * p.nsplit + split;
+    float* wo = p.ws_o + rec * D;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int grp = 0; grp < 4; ++grp) {
+            f32x4 w = {o[db][4 * grp], o[db][4 * grp + 1], o[db][4 * grp + 2], o[db][4 * grp + 3]};
+            *(f32x4*)(wo + 32 * db + 8 * grp + 4 * hi) = w;
+        }
+    if (hi == 0) {
+        p.ws_ml[2 * rec] = m_i;
+        p.ws_ml[2 * rec + 1] = ltot;
+    }
+}
+
+// Merges the splits of one (batch, head).  Thread = four output columns x one of COMBINE_LANES interleaved subsets of
+// the splits, merged with the usual running maximum / rescale; the subsets then meet in LDS.
+constexpr int COMBINE_THREADS = 256;
+template <typename T>
+__global__ __launch_bounds__(COMBINE_THREADS) void decode_combine_kernel(const DecodeParams p) {
+    __shared__ float s_m[COMBINE_THREADS], s_l[COMBINE_THREADS];
+    __shared__ __attribute__((aligned(16))) float s_acc[COMBINE_THREADS][4];
+    const int bh = blockIdx.x, tid = threadIdx.x;
+    const int cols = p.D / 4;                 // threads across the columns: 8, 16 or 32
+    const int lanes = COMBINE_THREADS / cols; // subsets of the splits
+    const int c4 = tid % cols, sl = tid / cols;
+    const float* ml = p.ws_ml + 2 * (int64_t)bh * p.nsplit;
+    const float* wo = p.ws_o + (int64_t)bh * p.nsplit * p.D + 4 * c4;
+    float m = -INFINITY, l = 0.f;
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
+    for (int s = sl; s < p.nsplit; s += lanes) {
+        const float ms = ml[2 * s], ls = ml[2 * s + 1];
+        const f32x4 o4 = *(const f32x4*)(wo + (int64_t)s * p.D);
+        const float mnew = fmaxf(m, ms);
+        const float a = __builtin_amdgcn_exp2f(m - mnew), w = __builtin_amdgcn_exp2f(ms - mnew);  // a = 0 at first
+        m = mnew;
+        l = l * a + ls * w;
+#pragma unroll
+        for (int x = 0; x < 4; ++x) acc[x] = acc[x] * a + o4[x] * w;
+    }
+    s_m[tid] = m;
+    s_l[tid] = l;
+    *(f32x4*)s_acc[tid] = acc;
+    __syncthreads();
+    if (sl != 0) return;
+    for (int j = 1; j < lanes; ++j) {
+        const int t = j * cols + c4;
+        const float ms = s_m[t];
+        if (ms == -INFINITY) continue;  // a subset without splits
+        const float mnew = fmaxf(m, ms);
+        const float a = __builtin_amdgcn_exp2f(m - mnew), w = __builtin_amdgcn_exp2f(ms - mnew);
+        m = mnew;
+        l = l * a + s_l[t] * w;
+#pragma unroll
+        for (int x = 0; x < 4; ++x) acc[x] = acc[x] * a + s_acc[t][x] * w;
+    }
+    const int b = bh / p.Hq, h = bh % p.Hq;
+    unsigned short* op = (unsigned short*)p.o + (int64_t)b * p.o_sb + (int64_t)h * p.o_sh + 4 * c4;
+    const float inv = 1.f / l;
+#pragma unroll
+    for (int x = 0; x < 4; ++x) op[x] = (unsigned short)(T::pack2(acc[x] * inv, 0.f) & 0xFFFFu);
 }
 
 template <typename T>
 static int launch_decode_t(const DecodeParams& p, hipStream_t stream) {
-    const dim3 grid(p.B * p.Hq), block(DEC_THREADS);
+    const dim3 grid(p.nsplit, p.Hkv, p.B * p.row_groups), block(64);
     if (p.D == 128)
-        hipLaunchKernelGGL((decode_kernel<T, 128>), grid, block, 0, stream, p);
+        hipLaunchKernelGGL((decode_split_kernel<T, 128>), grid, block, 0, stream, p);
     else if (p.D == 64)
-        hipLaunchKernelGGL((decode_kernel<T, 64>), grid, block, 0, stream, p);
+        hipLaunchKernelGGL((decode_split_kernel<T, 64>), grid, block, 0, stream, p);
     else
-        hipLaunchKernelGGL((decode_kernel<T, 32>), grid, block, 0, stream, p);
+        hipLaunchKernelGGL((decode_split_kernel<T, 32>), grid, block, 0, stream, p);
+    if (p.nsplit > 1)
+        hipLaunchKernelGGL((decode_combine_kernel<T>), dim3(p.B * p.Hq), dim3(COMBINE_THREADS), 0, stream, p);
     return (int)hipGetLastError();
 }
 
 int launch_decode(const DecodeParams& p, int dtype, hipStream_t stream) {
     return dtype == 1 ? launch_decode_t<BF16>(p, stream) : launch_decode_t<F16>(p, stream);
+}
+
+// How the keys of one decode step are split over workgroups: about ten waves per compute unit, at least two tiles per
+// split where the cache is long enough.  Shared by the workspace size and the launch.
+void decode_split_plan(int B, int Hq, int Hkv, int Sk, int window, int* nsplit, int* tiles_per_split, int* row_groups) {
+    const int G = Hq / Hkv;
+    const int rgs = (G + 31) / 32;
+    const int keys = (window > 0 && window < Sk) ? window : Sk;
+    const int n_tiles = (keys + DEC_KT - 1) / DEC_KT;
+    const int64_t units = (int64_t)B * Hkv * rgs;
+    int64_t want = (2560 + units - 1) / units;
+    const int most = n_tiles >= 2 ? n_tiles / 2 : 1;
+    if (want > most) want = most;
+    if (want < 1) want = 1;
+    const int tps = (int)((n_tiles + want - 1) / want);
+    *tiles_per_split = tps;
+    *nsplit = (n_tiles + tps - 1) / tps;
+    *row_groups = rgs;
 }
 
 }  // namespace bam

@@ -104,7 +104,7 @@ SIGNATURES = {
     "bam_fwd_indexed": [_ptr] * 5 + [_view, _ptr] + [_i64] * 14 + [_int] * 4 + [_f32, _int, _bias, _plan, _ptr],
     "bam_bwd_dkdv_indexed": [_ptr] * 8 + [_view, _ptr] + [_i64] * 20 + [_int] * 4 + [_f32, _int, _int, _bias, _plan, _ptr],
     "bam_bwd_dq_indexed": [_ptr] * 7 + [_view, _ptr] + [_i64] * 17 + [_int] * 4 + [_f32, _int, _int, _bias, _plan, _ptr],
-    "bam_decode": [_ptr] * 4 + [_i64] * 10 + [_int] * 5 + [_f32, _int, _int, _f32, _ptr],
+    "bam_decode": [_ptr] * 4 + [_i64] * 10 + [_int] * 5 + [_f32, _int, _int, _f32, _ptr, _i64, _ptr],
 }
 
 _lib = None
@@ -135,6 +135,8 @@ def load() -> ctypes.CDLL:
     lib.bam_plan_workspace_bytes_rect.argtypes = [_int, _int, _int]
     lib.bam_mask_plan_workspace_bytes.restype = _i64
     lib.bam_mask_plan_workspace_bytes.argtypes = [_int, _int, _int]
+    lib.bam_decode_workspace_bytes.restype = _i64
+    lib.bam_decode_workspace_bytes.argtypes = [_int] * 6
     lib.bam_ds_workspace_bytes.restype = _i64
     lib.bam_ds_workspace_bytes.argtypes = [_int, _i64]
     for name, argtypes in SIGNATURES.items():

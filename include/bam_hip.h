@@ -398,11 +398,16 @@ int bam_mask_tile_plan(const uint8_t* mask, int8_t* flags, int64_t flags_stride_
  *   keys j < Sk - window are dropped when 0 < window < Sk ;  o = softmax(s) v.
  * q, o: (B, Hq, D) with element strides for batch and head, unit stride along D, 2-byte aligned; k, v: (B, Sk, Hkv, D)
  * under the common layout rules.  window = 0 / softcap = 0 mean "none".
+ * The keys are split over many workgroups (there is only one query row per head) whose partial results meet in
+ * `workspace`: device memory of at least bam_decode_workspace_bytes(...) bytes for the same sizes, 16-byte aligned,
+ * free again once the stream has passed the call; 0 bytes (short caches: one split) means no workspace is needed
+ * and null may be passed.
  */
+int64_t bam_decode_workspace_bytes(int B, int Sk, int Hq, int Hkv, int D, int window);
 int bam_decode(const void* q, const void* k, const void* v, void* o, int64_t q_stride_b, int64_t q_stride_h,
                int64_t k_stride_b, int64_t k_stride_s, int64_t k_stride_h, int64_t v_stride_b, int64_t v_stride_s,
                int64_t v_stride_h, int64_t o_stride_b, int64_t o_stride_h, int B, int Sk, int Hq, int Hkv, int D, float scale,
-               int dtype, int window, float softcap, void* stream);
+               int dtype, int window, float softcap, void* workspace, int64_t workspace_bytes, void* stream);
 
 #ifdef __cplusplus
 }

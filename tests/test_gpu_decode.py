@@ -65,6 +65,19 @@ def test_decode_step_head_dims_between_the_native_ones_and_head_groupings(dtype,
         assert (got.float() - O.decode_step(q, k, v, **kw)).abs().max().item() <= (1e-2 if dtype == torch.float16 else O_MAX_ABS)
 
 
+@pytest.mark.parametrize("B,Hq,Hkv,Sk,D", [(1, 32, 8, 8192, 128), (2, 16, 16, 5000, 64), (1, 8, 1, 20001, 128),
+                                           (3, 40, 1, 700, 32), (1, 66, 2, 1300, 64)])
+def test_decode_step_long_caches_split_over_many_workgroups(B, Hq, Hkv, Sk, D):
+    # long caches: many splits and the combine pass; 40 and 33 q heads per kv head: more than one group of 32 heads
+    lib = _bam_hip.load()
+    assert lib.bam_decode_workspace_bytes(B, Sk, Hq, Hkv, D, 0) > 0
+    q, k, v = inputs(B, Hq, Hkv, Sk, D, torch.bfloat16, seed=Sk)
+    for kw in ({}, {"sliding_window": Sk // 3, "softcap": 20.0}, {"sliding_window": 33}):
+        got = decode(q, k, v, **kw)
+        want = O.decode_step(q, k, v, **kw)
+        assert (got.float() - want).abs().max().item() <= O_MAX_ABS
+
+
 def test_decode_step_closed_forms_on_the_device():
     q, k, v = inputs(2, 4, 2, 500, 64, torch.bfloat16, seed=1)
     plain = decode(q, k, v)
@@ -115,4 +128,4 @@ def test_training_mode_takes_the_bitfield_path_and_bad_arguments_are_refused():
     with pytest.raises(_bam_hip.BamError, match="window"):
         _bam_hip.call("bam_decode", q.data_ptr(), kt.data_ptr(), vt.data_ptr(), o.data_ptr(), q.stride(0), q.stride(1),
                       kt.stride(0), kt.stride(1), kt.stride(2), vt.stride(0), vt.stride(1), vt.stride(2), o.stride(0),
-                      o.stride(1), 1, 8, 4, 2, 64, 0.125, BA._dtype_code(q.dtype), -1, 0.0, BA._stream_ptr(dev()))
+                      o.stride(1), 1, 8, 4, 2, 64, 0.125, BA._dtype_code(q.dtype), -1, 0.0, None, 0, BA._stream_ptr(dev()))

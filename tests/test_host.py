@@ -41,7 +41,7 @@ def test_library_exports_every_declared_symbol():
     # the binding's prototypes cover every compute entry point of the header
     assert set(_bam_hip.SIGNATURES) == set(names) - {
         "bam_last_error", "bam_abi_version", "bam_plan_workspace_bytes", "bam_plan_workspace_bytes_rect",
-        "bam_ds_workspace_bytes", "bam_mask_plan_workspace_bytes"}
+        "bam_ds_workspace_bytes", "bam_mask_plan_workspace_bytes", "bam_decode_workspace_bytes"}
     # plan workspace: sized without a GPU; no plan beyond 4096 row slices
     lib2 = _bam_hip.load()
     assert lib2.bam_plan_workspace_bytes(1, 8192) >= 256 * 256 + 256 * 4 and lib2.bam_plan_workspace_bytes(1, 8192) % 256 == 0
@@ -151,7 +151,7 @@ def test_adapter_requires_int64_mask():
 def test_decode_entry_rejects_bad_arguments_without_touching_the_gpu():
     lib = _bam_hip.load()
     P = ctypes.c_void_p
-    good = [P(16)] * 4 + [8] * 10 + [1, 64, 4, 2, 64] + [0.125, 1, 0, 0.0, None]
+    good = [P(16)] * 4 + [8] * 10 + [1, 64, 4, 2, 64] + [0.125, 1, 0, 0.0, None, 0, None]
     bad_window = list(good)
     bad_window[21] = -3
     assert lib.bam_decode(*bad_window) == -1 and b"window" in lib.bam_last_error()
@@ -162,6 +162,14 @@ def test_decode_entry_rejects_bad_arguments_without_touching_the_gpu():
     bad_heads[16:18] = [4, 3]
     assert lib.bam_decode(*bad_heads) == -1 and b"multiple of Hkv" in lib.bam_last_error()
     assert lib.bam_decode(*([None] + good[1:])) == -1 and b"null" in lib.bam_last_error()
+    # long caches are split over many workgroups and need a workspace for the partial results; short ones do not
+    assert lib.bam_decode_workspace_bytes(1, 32, 4, 2, 64, 0) == 0
+    need = lib.bam_decode_workspace_bytes(1, 8192, 32, 8, 128, 0)
+    assert need > 0 and need % (32 * (128 + 2) * 4) == 0
+    assert lib.bam_decode_workspace_bytes(1, 8192, 32, 8, 128, 32) == 0  # a window of one tile: one split
+    long_cache = list(good)
+    long_cache[15] = 8192
+    assert lib.bam_decode(*long_cache) == -1 and b"workspace" in lib.bam_last_error()
 
 
 # The import statements of the reference's callers, verbatim (file:line of /root/reference/cornstarch/...).
