@@ -99,7 +99,17 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
 
     const int unit = blockIdx.x;
     const int hk = unit % p.Hkv;
-    const int ub = unit / p.Hkv;
+    int ub = unit / p.Hkv;  // position of the (batch, key tile) in the order of falling work
+    {
+        // The hardware deals the workgroups of an XCD to its four shader engines in turn and launches them strictly
+        // in order: a workgroup waits for a free compute unit on ITS engine while free units of the other engines sit
+        // idle behind it.  In a plainly sorted list one engine would get the heaviest workgroup of every four and
+        // hold everybody back (measured: units idle 19 us at the median, up to 90 us, before their second workgroup),
+        // so every other run of 32 workgroups -- four per XCD, one per engine -- takes its tiles in reverse.
+        const int P = (p.Hkv <= 32 && 32 % p.Hkv == 0) ? 32 / p.Hkv : 1;
+        const int g = ub / P, r = ub - g * P;
+        if ((g & 1) && (g + 1) * P <= p.num_kt * p.B) ub = g * P + (P - 1 - r);
+    }
     int b = ub % p.B;
     int nt = ub / p.B;  // early key tiles (most queries under causality) first
     if (p.tile_order != nullptr) {  // with a plan: the tiles by falling amount of work, whatever the mask looks like
