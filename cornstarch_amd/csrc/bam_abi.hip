@@ -2,6 +2,7 @@
 // The declarations (with the reference call sites they replace) are in include/bam_hip.h.
 #include "../../include/bam_hip.h"
 
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 
@@ -15,10 +16,11 @@ static __device__ __align__(256) unsigned char g_static_plan_scratch[BAM_STATIC_
 namespace {
 
 constexpr int kMaxDevices = 64;
-void* g_static_plan_ptr[kMaxDevices] = {};  // per device, resolved on first use
+// per device, resolved on first use (two host threads that get there together both store the same address)
+std::atomic<void*> g_static_plan_ptr[kMaxDevices] = {};
 // Every bam_tile_plan_static call on a device starts a new generation of that device's array; the plan it returns
 // carries the number, and a plan of an older generation (its arrays have been overwritten since) is refused.
-int32_t g_static_plan_generation[kMaxDevices] = {};
+std::atomic<int32_t> g_static_plan_generation[kMaxDevices] = {};
 
 thread_local char g_error[512] = "";
 
@@ -139,7 +141,8 @@ int fill_plan(bam::AttnParams& p, const char* who, const bam_plan* plan, int B, 
     if (plan->generation != 0) {  // laid out in the built-in array of bam_tile_plan_static
         int dev = -1;
         if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices ||
-            plan->fine != (const uint8_t*)g_static_plan_ptr[dev] || plan->generation != g_static_plan_generation[dev])
+            plan->fine != (const uint8_t*)g_static_plan_ptr[dev].load() ||
+            plan->generation != g_static_plan_generation[dev].load())
             return fail(BAM_ERR_INVALID_ARGUMENT,
                         "%s: plan of bam_tile_plan_static is stale (a later call on this GPU has reused the built-in array)",
                         who);
@@ -447,18 +450,19 @@ int bam_tile_plan_static(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, 
     int dev = -1;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices)
         return fail(BAM_ERR_LAUNCH, "bam_tile_plan_static: no current device (or more than %d devices)", kMaxDevices);
-    if (g_static_plan_ptr[dev] == nullptr) {
+    void* ptr = g_static_plan_ptr[dev].load(std::memory_order_acquire);
+    if (ptr == nullptr) {
         // once per device, with that device current: the array's own address on this GPU
-        void* ptr = nullptr;
         const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(g_static_plan_scratch));
         if (e != hipSuccess || ptr == nullptr)
             return fail(BAM_ERR_LAUNCH, "bam_tile_plan_static: hipGetSymbolAddress failed: %s", hipGetErrorString(e));
-        g_static_plan_ptr[dev] = ptr;
+        g_static_plan_ptr[dev].store(ptr, std::memory_order_release);
     }
-    BAM_TRY(bam_tile_plan(bf, bf_stride_b, flags, flags_stride_b, flags_stride_m, g_static_plan_ptr[dev],
-                          BAM_STATIC_PLAN_BYTES, B, S, plan, stream));
-    if (++g_static_plan_generation[dev] <= 0) g_static_plan_generation[dev] = 1;
-    plan->generation = g_static_plan_generation[dev];
+    BAM_TRY(bam_tile_plan(bf, bf_stride_b, flags, flags_stride_b, flags_stride_m, ptr, BAM_STATIC_PLAN_BYTES, B, S, plan,
+                          stream));
+    int32_t gen = g_static_plan_generation[dev].fetch_add(1) + 1;
+    if (gen <= 0) g_static_plan_generation[dev].store(gen = 1);
+    plan->generation = gen;
     return BAM_OK;
 }
 

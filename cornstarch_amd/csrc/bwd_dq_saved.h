@@ -8,7 +8,7 @@
 // Work decomposition: as the forward -- a workgroup is four 32-row slices of one (batch, q head), one per wave (taken
 // from the plan's slice order), and walks the 64-key tiles any of them needs; K tiles are shared through LDS (double
 // buffered), every wave copies its own dS blocks (two 2 KiB blocks per tile, one per 32-key half) into a wave-private
-// LDS area.  Both MFMA operands come from transposing LDS reads: K^T (d x keys) from the row-major K tile, dS^T
+// LDS area, two tiles ahead: a buffer is refilled as soon as its operands are in registers.  Both MFMA operands come from transposing LDS reads: K^T (d x keys) from the row-major K tile, dS^T
 // (keys x rows) from the block, which the dK/dV lanes wrote key by key.
 #pragma once
 #include "bam_common.h"
@@ -115,52 +115,75 @@ __global__ __launch_bounds__(DQS_THREADS, 2) void bwd_dq_saved_kernel(const Attn
     const char* ds_head = (const char*)p.ds_ws + (((int64_t)h * p.ds_capacity) << 13);
     const int* entry_row = p.ds_entry + (int64_t)b * p.ds_entry_sb + (int64_t)(slice < 0 ? 0 : slice) * p.num_kt;
 
-    // record numbers of the coming list entries, 64 at a time: lane j holds the one of list entry base + j
+    // record numbers of the coming list entries, 64 at a time: lane j holds the one of list entry base + j.
+    // The loaded value is handed on through an instruction of its own, so that the compiler's wait for the load sits
+    // right here (once per 64 tiles) and not in front of every later use: a wait for this load is a wait for every
+    // tile copy in flight.
     int ent_vec = 0;
     auto load_entries = [&](int base, int n) {
         const int j = base + lane;
         int e = 0;
         if (j < n && slice >= 0) e = entry_row[sList[j] >> 17];  // 64-key tile kt -> 128-key tile kt / 2
-        ent_vec = e;
+        asm volatile("v_mov_b32 %0, %1" : "=v"(ent_vec) : "v"(e));
     };
 
-    // copies of tile `entry` into buffer buf: the K tile (shared) and this wave's dS blocks of the halves that have work
-    auto issue_copies = [&](int entry, int e, int buf) {
-        const int kt = entry >> 16;
+    // copy of the K tile of list entry `entry` into buffer buf (shared by the four waves)
+    auto issue_k = [&](int entry, int buf) {
 #pragma unroll
-        for (int j = 0; j < CPT; ++j) stK.issue(j, kbase + kt * k_ts, ldsK + buf * TILE_BYTES);
+        for (int j = 0; j < CPT; ++j) stK.issue(j, kbase + (entry >> 16) * k_ts, ldsK + buf * TILE_BYTES);
+    };
+    // copies of this wave's dS blocks of tile `entry` (record e), the halves that have work, into its buffer buf;
+    // returns the number of copy instructions issued (wave-uniform)
+    auto issue_ds = [&](int entry, int e, int buf) -> int {
+        const int kt = entry >> 16;
         const int c = (entry >> (4 * wave)) & 15;  // wave-uniform
         const char* rec = ds_head + ((int64_t)e << 13) + (kt & 1) * 4096;
+        int issued = 0;
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb)
             if ((c >> (2 * kb)) & 3) {
                 dma_b128<1>(rec + kb * 2048, (unsigned)(lane * 16), ldsDS + buf * 4096u + kb * 2048u);
                 dma_b128<2>(rec + kb * 2048, (unsigned)(lane * 16 + 1024), ldsDS + buf * 4096u + kb * 2048u + 1024u);
+                issued += 2;
             }
+        return issued;
     };
 
-    auto tile_step = [&](int cur, int entry) {
+    // One 64-key tile.  The dS operands are read first; the wave's buffer is then free again and takes the blocks of
+    // the tile after next (`entry2`, record `e2`; negative entry2 = nothing left), so that two tiles' worth of
+    // workspace reads are in flight per wave: the kernel waits for HBM, not for the MFMAs.  Returns the number of
+    // copies issued.
+    auto tile_step = [&](int cur, int entry, int entry2, int e2) -> int {
         // (per-lane copy of the wave number: a skip branch the compiler can prove wave-uniform makes it restructure the loop)
         const int c = (entry >> (4 * wave_lane)) & 15;
-        if (c == 0) return;
         const u32x4* tK = sK[cur];
         const char* tDS = (const char*)sDS[wave][cur];
+        u32x4 bop[2][2];
+        if (c != 0) {
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+                    if ((c >> (2 * kb)) & 3) bop[kb][t] = ds_block_read_transposed(tDS + kb * 2048, lane, 16 * t + 4 * hi, 16 * half16);
+            wait_lds();  // the copies below overwrite what was just read
+        }
+        const int issued = entry2 >= 0 ? issue_ds(entry2, e2, cur) : 0;
+        if (c == 0) return issued;
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) {
             if (((c >> (2 * kb)) & 3) == 0) continue;
-            u32x4 bop[2], ta[2][DB];
-#pragma unroll
-            for (int t = 0; t < 2; ++t) {
-                bop[t] = ds_block_read_transposed(tDS + kb * 2048, lane, 16 * t + 4 * hi, 16 * half16);
-#pragma unroll
-                for (int db = 0; db < DB; ++db)
-                    ta[t][db] = lds_read_transposed<D>(tK, lane, 32 * kb + 16 * t + 4 * hi, 32 * db + 16 * half16);
-            }
+            u32x4 ta[2][DB];
 #pragma unroll
             for (int t = 0; t < 2; ++t)
 #pragma unroll
-                for (int db = 0; db < DB; ++db) dq[db] = T::mfma(ta[t][db], bop[t], dq[db]);
+                for (int db = 0; db < DB; ++db)
+                    ta[t][db] = lds_read_transposed<D>(tK, lane, 32 * kb + 16 * t + 4 * hi, 32 * db + 16 * half16);
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int db = 0; db < DB; ++db) dq[db] = T::mfma(ta[t][db], bop[kb][t], dq[db]);
         }
+        return issued;
     };
 
     __syncthreads();
@@ -173,19 +196,34 @@ __global__ __launch_bounds__(DQS_THREADS, 2) void bwd_dq_saved_kernel(const Attn
     if (n > 0) {
         load_entries(0, n_all);
         int entry = __builtin_amdgcn_readfirstlane(sList[0]);
-        issue_copies(entry, __builtin_amdgcn_readlane(ent_vec, 0), 0);
+        int next = __builtin_amdgcn_readfirstlane(sList[n > 1 ? 1 : 0]);
+        issue_k(entry, 0);
+        issue_ds(entry, __builtin_amdgcn_readlane(ent_vec, 0), 0);
+        if (n > 1) issue_ds(next, __builtin_amdgcn_readlane(ent_vec, 1), 1);
         wait_async();
         __syncthreads();
         for (int it = 0; it < n; ++it) {
             const int cur = it & 1;
-            const int nx = it + 1 < n ? it + 1 : it;  // past the end the last tile is copied again (nobody reads it)
-            if ((nx & 63) == 0 && nx != it) load_entries(nx, n_all);
-            const int next = __builtin_amdgcn_readfirstlane(sList[nx]);
-            const int e_next = __builtin_amdgcn_readlane(ent_vec, nx & 63);
-            issue_copies(next, e_next, cur ^ 1);
-            tile_step(cur, entry);
+            // the K tile of the next entry (past the end the last tile is copied again: nobody reads it)
+            issue_k(next, cur ^ 1);
+            // the dS blocks of the entry after next
+            const int i2 = it + 2;
+            int entry2 = -1, e2 = 0;
+            if (i2 < n) {
+                if ((i2 & 63) == 0) load_entries(i2, n_all);
+                entry2 = __builtin_amdgcn_readfirstlane(sList[i2]);
+                e2 = __builtin_amdgcn_readlane(ent_vec, i2 & 63);
+            }
+            const int issued = tile_step(cur, entry, entry2, e2);
             entry = next;
-            wait_async();
+            next = entry2 >= 0 ? entry2 : next;
+            // everything but the copies of the entry after next has to have landed: copies complete in order
+            if (issued == 4)
+                asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+            else if (issued == 2)
+                asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+            else
+                wait_async();
             __syncthreads();
         }
     }
@@ -207,7 +245,7 @@ __global__ __launch_bounds__(DQS_THREADS, 2) void bwd_dq_saved_kernel(const Attn
                 }
         }
         __syncthreads();
-        tile_step(0, entry);
+        tile_step(0, entry, -1, 0);
     }
 
     // ---- epilogue: dq holds -dQ / scale (C fragment: lane = query column, registers = head dims 8 g + 4 hi + x)

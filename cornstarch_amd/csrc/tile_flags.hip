@@ -15,6 +15,7 @@ namespace bam {
 constexpr int FLAG_WAVES = 4;
 constexpr int FLAG_TILES_PER_WAVE = 2;  // few tiles per wave: the grid, not the wave, covers the row of tiles
 constexpr int FLAG_COLS_PER_BLOCK = FLAG_WAVES * FLAG_TILES_PER_WAVE;
+constexpr int FLAG_MAX_BLOCKS_X = 64;  // workgroups per 128-row block; longer rows of tiles are walked in a loop
 
 // ---------------------------------------------------------------------------------------------------------
 // Slice order.  The forward and dQ kernels give each of the four waves of a workgroup one 32-row slice and walk
@@ -26,48 +27,35 @@ constexpr int FLAG_COLS_PER_BLOCK = FLAG_WAVES * FLAG_TILES_PER_WAVE;
 // MAX_PLAN_SLICES of them); slots past the last slice are set to -1.  The work rides in the launch of the flag
 // kernel, as extra workgroups of its grid (it needs the bitfields only): workgroup `part` of sequence b ranks
 // slices [256 part, +256).
-__device__ __forceinline__ void slice_sort_key(const int64_t* __restrict__ row, int S, int ns, int s,
-                                               unsigned long long& k1, unsigned long long& k2) {
-    k1 = ~0ull;
-    k2 = ~0ull;
-    if (s >= ns) return;
-    const int64_t M = (((int64_t)1) << 62) - 1;
-    int64_t sig = 0;
-    bool text = false;
-#pragma unroll
-    for (int r = 0; r < 32; ++r) {  // 32 independent loads, all in flight together
-        const int i = s * 32 + r;
-        const int64_t f = i < S ? row[i] : 0;
-        sig |= f & M;
-        text |= (f & 1) != 0;
-    }
-    k1 = text ? 0ull : (1ull << 62) | (unsigned long long)sig;
-    k2 = text ? (unsigned long long)(ns - 1 - s) : (unsigned long long)s;
-}
-
-// Ranks the slices [256 part, +256) of one sequence among all `ns` slices by the two-word keys `key(s, k1, k2)`
-// delivers (distinct for distinct slices; slices >= ns get the largest key) and writes order_row[rank] = slice;
-// the slots past the last slice are set to -1.
-template <typename KeyFn>
-__device__ __forceinline__ void slice_order_ranked(KeyFn key, int ns, int slots, int part, int* __restrict__ order_row) {
-    __shared__ unsigned long long sk[2 * 256];
+// Ranks the slices [256 part, +256) of one sequence among all `ns` slices by two-word keys (distinct for distinct
+// slices; slices >= ns get the largest key) and writes order_row[rank] = slice; the slots past the last slice are set
+// to -1.  `fill(base, sk)` puts the keys of slices [base, base + 256) into sk[2 i], sk[2 i + 1] (all 256 threads take
+// part).  The compares read the keys eight at a time, so that the loop runs at the rate of the LDS and not at its
+// latency.
+typedef unsigned long long u64x2 __attribute__((ext_vector_type(2)));
+template <typename FillFn>
+__device__ __forceinline__ void slice_order_ranked(FillFn fill, int ns, int slots, int part, int* __restrict__ order_row) {
+    __shared__ __attribute__((aligned(16))) unsigned long long sk[2 * 256];
     const int tid = threadIdx.x, s = part * 256 + tid;
-    unsigned long long my1, my2;
-    key(s, my1, my2);
+    unsigned long long my1 = 0, my2 = 0;
     int rank = 0;
-    for (int base = 0; base < ns; base += 256) {
+    // this workgroup's own slices first (their keys are what the others are compared with), then the other chunks
+    const int nchunks = (ns + 255) / 256;
+    for (int c = 0; c < nchunks; ++c) {
+        const int base = 256 * (c == 0 ? part : c <= part ? c - 1 : c);
         __syncthreads();
-        if (base == part * 256) {  // this workgroup's own slices: the keys are already there
-            sk[2 * tid] = my1;
-            sk[2 * tid + 1] = my2;
-        } else {
-            key(base + tid, sk[2 * tid], sk[2 * tid + 1]);
+        fill(base, sk);
+        __syncthreads();
+        if (c == 0) {
+            my1 = sk[2 * tid];
+            my2 = sk[2 * tid + 1];
         }
-        __syncthreads();
-        const int cnt = min(256, ns - base);
-        for (int j = 0; j < cnt; ++j) {
-            const unsigned long long o1 = sk[2 * j], o2 = sk[2 * j + 1];
-            rank += (o1 < my1 || (o1 == my1 && o2 < my2)) ? 1 : 0;  // (k1, k2) pairs are distinct
+        for (int j0 = 0; j0 < 256; j0 += 8) {  // entries past the last slice hold the largest key: never smaller
+            u64x2 o[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) o[u] = *(const u64x2*)&sk[2 * (j0 + u)];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) rank += (o[u][0] < my1 || (o[u][0] == my1 && o[u][1] < my2)) ? 1 : 0;
         }
     }
     if (s < ns)
@@ -76,11 +64,47 @@ __device__ __forceinline__ void slice_order_ranked(KeyFn key, int ns, int slots,
         order_row[s] = -1;
 }
 
+// OR over the 16 lanes of a DPP row, result in every lane (quad swaps, then the two mirror patterns).
+__device__ __forceinline__ unsigned row_or(unsigned x) {
+    x |= (unsigned)__builtin_amdgcn_mov_dpp((int)x, 0xB1, 0xF, 0xF, false);   // quad_perm [1,0,3,2]
+    x |= (unsigned)__builtin_amdgcn_mov_dpp((int)x, 0x4E, 0xF, 0xF, false);   // quad_perm [2,3,0,1]
+    x |= (unsigned)__builtin_amdgcn_mov_dpp((int)x, 0x141, 0xF, 0xF, false);  // row_half_mirror
+    x |= (unsigned)__builtin_amdgcn_mov_dpp((int)x, 0x140, 0xF, 0xF, false);  // row_mirror
+    return x;
+}
+
+// Keys of slices [base, base + 256) from the bitfields (k1 = 0 for a slice with a text row, else bit 62 + the OR of
+// its bitfields; k2 = the position rank inside the class), read in order: 16 lanes take the 32 rows of one slice (two
+// each) and OR them together; bit 0 of the OR says whether the slice holds a text row.
+__device__ __forceinline__ void slice_keys_chunk(const int64_t* __restrict__ row, int S, int ns, int base,
+                                                 unsigned long long* sk) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int64_t M = (((int64_t)1) << 62) - 1;
+#pragma unroll 4
+    for (int pass = 0; pass < 16; ++pass) {
+        const int local = 64 * wave + 4 * pass + (lane >> 4);  // slice within the chunk
+        const int s = base + local;
+        const int i = s * 32 + 2 * (lane & 15);
+        const int64_t f0 = i < S ? row[i] : 0, f1 = i + 1 < S ? row[i + 1] : 0;
+        const uint64_t f = (uint64_t)(f0 | f1);
+        const unsigned lo = row_or((unsigned)f), hi = row_or((unsigned)(f >> 32));
+        if ((lane & 15) == 0) {
+            const bool text = (lo & 1u) != 0;
+            const unsigned long long sig = (((unsigned long long)hi << 32) | lo) & (unsigned long long)M;
+            unsigned long long k1 = text ? 0ull : (1ull << 62) | sig;
+            unsigned long long k2 = text ? (unsigned long long)(ns - 1 - s) : (unsigned long long)s;
+            if (s >= ns) k1 = k2 = ~0ull;
+            sk[2 * local] = k1;
+            sk[2 * local + 1] = k2;
+        }
+    }
+}
+
 __device__ __forceinline__ void slice_order_part(const int64_t* __restrict__ row, int S, int part,
                                                  int* __restrict__ order_row) {
     const int ns = (S + 31) / 32, slots = 4 * ((S + BLOCK_M - 1) / BLOCK_M);
-    slice_order_ranked([&](int s, unsigned long long& k1, unsigned long long& k2) { slice_sort_key(row, S, ns, s, k1, k2); },
-                       ns, slots, part, order_row);
+    slice_order_ranked([&](int base, unsigned long long* sk) { slice_keys_chunk(row, S, ns, base, sk); }, ns, slots, part,
+                       order_row);
 }
 
 // The same ordering idea for index-tensor attention, where a local row's position is pos[row]: slices holding a
@@ -123,7 +147,7 @@ __global__ __launch_bounds__(FLAG_WAVES * 64) void tile_flags_kernel(const int64
                                                                     uint8_t* __restrict__ fine, int64_t fine_sb,
                                                                     int64_t fine_ss, int* __restrict__ order,
                                                                     int64_t order_sb, int flag_blocks_x,
-                                                                    int* __restrict__ pair_count) {
+                                                                    int flag_groups, int* __restrict__ pair_count) {
     // (the pair counter of the numbering kernel that follows in the stream starts from zero)
     if (FINE && pair_count != nullptr && blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0 && threadIdx.x == 0)
         *pair_count = 0;
@@ -136,101 +160,137 @@ __global__ __launch_bounds__(FLAG_WAVES * 64) void tile_flags_kernel(const int64
     __shared__ int64_t q_bits[BLOCK_M];
     // classes of this workgroup's eight column tiles: row 0 the flag, rows 1..4 the four row slices; written out
     // together at the end (eight bytes per row in one store where the layout guarantees alignment)
-    __shared__ __attribute__((aligned(8))) uint8_t s_out[5][FLAG_COLS_PER_BLOCK];
+    // (two copies: a workgroup that takes several groups of column tiles fills one while the other is stored)
+    __shared__ __attribute__((aligned(8))) uint8_t s_out_buf[2][5][FLAG_COLS_PER_BLOCK];
     const int b = blockIdx.z, m = blockIdx.y;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int64_t* row = bf + (int64_t)b * bf_stride_b;
-    if (tid < 5 * FLAG_COLS_PER_BLOCK) s_out[0][tid] = 0;
     if (tid < BLOCK_M) {
         const int i = m * BLOCK_M + tid;
         q_bits[tid] = (i < S) ? row[i] : 0;  // out-of-range positions read 0 (reference :86-87)
     }
     __syncthreads();
     const int rows_in_range = min(BLOCK_M, S - m * BLOCK_M);
-    const int half = lane >> 5;
-    const int64_t q0 = q_bits[0];
-    const bool rows_uniform = rows_in_range == BLOCK_M && __all(q_bits[lane] == q0 && q_bits[lane + 64] == q0);
-    // the key bitfields of all tiles of this wave, requested together (one memory latency instead of one per tile)
-    int64_t kfs[FLAG_TILES_PER_WAVE];
+    const int half = lane >> 5, l32 = lane & 31;
+    // Runs of equal bitfields inside each of the four 32-row slices: bit r of slice_starts[w] = row r starts a run
+    // (rows past the end of the sequence read 0 and make a run of their own).  The count of a column over a run
+    // follows from one evaluation of the bit test, so a tile costs one evaluation per run, not one per row.
+    int64_t slice_q[4];
+    unsigned slice_starts[4];
 #pragma unroll
-    for (int t = 0; t < FLAG_TILES_PER_WAVE; ++t) {
-        const int j = (blockIdx.x * FLAG_COLS_PER_BLOCK + wave * FLAG_TILES_PER_WAVE + t) * BLOCK_N + (lane & 31);
-        kfs[t] = (j < S) ? row[j] : 0;
+    for (int w = 0; w < 4; ++w) {
+        slice_q[w] = q_bits[32 * w];
+        slice_starts[w] = (unsigned)__ballot(l32 == 0 || q_bits[32 * w + l32] != q_bits[32 * w + max(l32, 1) - 1]);
     }
+    const int64_t q0 = slice_q[0];
+    const bool rows_uniform = rows_in_range == BLOCK_M && slice_starts[0] == 1u && slice_starts[1] == 1u &&
+                              slice_starts[2] == 1u && slice_starts[3] == 1u && slice_q[1] == q0 && slice_q[2] == q0 &&
+                              slice_q[3] == q0;
+    // A workgroup takes the groups of eight column tiles bx = blockIdx.x, blockIdx.x + flag_blocks_x, ...: one group
+    // for sequences of up to 16384 keys, several for longer ones (the setup above is then paid once).
+    int it = 0;
+    for (int bx = blockIdx.x; bx < flag_groups; bx += flag_blocks_x, ++it) {
+        uint8_t (*s_out)[FLAG_COLS_PER_BLOCK] = s_out_buf[it & 1];
+        if (tid < 5 * FLAG_COLS_PER_BLOCK) s_out[0][tid] = 0;
+        __syncthreads();
+        static_assert(FLAG_TILES_PER_WAVE == 2, "the counting path gives each half of a wave one tile");
+        // the key bitfields of both tiles of this wave, requested together (one memory latency instead of one per tile)
+        int64_t kfs[FLAG_TILES_PER_WAVE];
 #pragma unroll
-    for (int t = 0; t < FLAG_TILES_PER_WAVE; ++t) {
-        const int n = blockIdx.x * FLAG_COLS_PER_BLOCK + wave * FLAG_TILES_PER_WAVE + t;
-        if (n >= num_n) break;  // wave-uniform
-        const int j = n * BLOCK_N + (lane & 31);
-        const int64_t kf = kfs[t];
-        if (rows_uniform && (n + 1) * BLOCK_N <= S) {
-            const unsigned klo = __builtin_amdgcn_readfirstlane((unsigned)kf);
-            const unsigned khi = __builtin_amdgcn_readfirstlane((unsigned)((uint64_t)kf >> 32));
-            const int64_t k0 = (int64_t)(((uint64_t)khi << 32) | klo);
-            if (__all(kf == k0)) {
-                const int64_t M = (((int64_t)1) << 62) - 1;
-                const int64_t qb = q0 & M, kb = k0 & M;
-                int8_t f;
-                const int r0 = m * BLOCK_M, c0 = n * BLOCK_N;
-                if (q0 & 1) {  // text rows: causal over keys that share a bit
-                    f = (qb & kb) == 0 ? 0 : r0 >= c0 + BLOCK_N - 1 ? 2 : r0 + BLOCK_M - 1 < c0 ? 0 : 1;
-                } else {
-                    f = (qb == kb && qb != 0) ? 2 : 0;
+        for (int t = 0; t < FLAG_TILES_PER_WAVE; ++t) {
+            const int j = (bx * FLAG_COLS_PER_BLOCK + wave * FLAG_TILES_PER_WAVE + t) * BLOCK_N + l32;
+            kfs[t] = (j < S) ? row[j] : 0;
+        }
+        bool counted[FLAG_TILES_PER_WAVE];  // wave-uniform: the tile still needs the counting path
+#pragma unroll
+        for (int t = 0; t < FLAG_TILES_PER_WAVE; ++t) {
+            const int n = bx * FLAG_COLS_PER_BLOCK + wave * FLAG_TILES_PER_WAVE + t;
+            counted[t] = n < num_n;
+            if (n >= num_n) continue;  // wave-uniform
+            const int64_t kf = kfs[t];
+            if (rows_uniform && (n + 1) * BLOCK_N <= S) {
+                const unsigned klo = __builtin_amdgcn_readfirstlane((unsigned)kf);
+                const unsigned khi = __builtin_amdgcn_readfirstlane((unsigned)((uint64_t)kf >> 32));
+                const int64_t k0 = (int64_t)(((uint64_t)khi << 32) | klo);
+                if (__all(kf == k0)) {
+                    const int64_t M = (((int64_t)1) << 62) - 1;
+                    const int64_t qb = q0 & M, kb = k0 & M;
+                    int8_t f;
+                    const int r0 = m * BLOCK_M, c0 = n * BLOCK_N;
+                    if (q0 & 1) {  // text rows: causal over keys that share a bit
+                        f = (qb & kb) == 0 ? 0 : r0 >= c0 + BLOCK_N - 1 ? 2 : r0 + BLOCK_M - 1 < c0 ? 0 : 1;
+                    } else {
+                        f = (qb == kb && qb != 0) ? 2 : 0;
+                    }
+                    const int col = wave * FLAG_TILES_PER_WAVE + t;
+                    if (lane == 0) s_out[0][col] = (uint8_t)f;
+                    if (FINE && lane < 4) {  // the same closed form for the 32 rows of slice `lane`
+                        const int rs = r0 + 32 * lane;
+                        int8_t fw = f;
+                        if (q0 & 1) fw = (qb & kb) == 0 ? 0 : rs >= c0 + BLOCK_N - 1 ? 2 : rs + 31 < c0 ? 0 : 1;
+                        s_out[1 + lane][col] = (uint8_t)fw;
+                    }
+                    counted[t] = false;
                 }
+            }
+        }
+        if (counted[0] || counted[1]) {
+            // Counting path, both tiles at once: lanes [0, 32) own the columns of tile 0, lanes [32, 64) those of tile 1.
+            const int t = half;
+            const int n = bx * FLAG_COLS_PER_BLOCK + wave * FLAG_TILES_PER_WAVE + t;
+            const int j = n * BLOCK_N + l32;
+            const int64_t kf = half ? kfs[1] : kfs[0];
+            const int64_t M = (((int64_t)1) << 62) - 1;
+            const int64_t kb = kf & M;
+            int cnt[4];
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                const int r0 = m * BLOCK_M + 32 * w;
+                unsigned starts = slice_starts[w];  // wave-uniform, bit 0 set
+                int c = 0;
+                while (starts != 0u) {
+                    const int a = __builtin_ctz(starts);
+                    starts &= starts - 1u;
+                    const int e = starts != 0u ? __builtin_ctz(starts) : 32;  // the run is rows [a, e) of the slice
+                    const int64_t qf = q_bits[32 * w + a];
+                    const int64_t qb = qf & M;
+                    if (qf & 1)  // text rows: those at or after column j (reference :93-97)
+                        c += (qb & kb) != 0 ? min(e - a, max(0, r0 + e - max(r0 + a, j))) : 0;
+                    else
+                        c += (qb == kb && qb != 0) ? e - a : 0;
+                }
+                cnt[w] = c;
+            }
+#pragma unroll
+            for (int off = 16; off > 0; off >>= 1)  // over the 32 columns, inside each half of the wave
+#pragma unroll
+                for (int w = 0; w < 4; ++w) cnt[w] += __shfl_xor(cnt[w], off);
+            const bool mine = half ? counted[1] : counted[0];
+            if (l32 == 0 && mine) {
+                const int cols_in_range = min(BLOCK_N, S - n * BLOCK_N);
                 const int col = wave * FLAG_TILES_PER_WAVE + t;
-                if (lane == 0) s_out[0][col] = (uint8_t)f;
-                if (FINE && lane < 4) {  // the same closed form for the 32 rows of slice `lane`
-                    const int rs = r0 + 32 * lane;
-                    int8_t fw = f;
-                    if (q0 & 1) fw = (qb & kb) == 0 ? 0 : rs >= c0 + BLOCK_N - 1 ? 2 : rs + 31 < c0 ? 0 : 1;
-                    s_out[1 + lane][col] = (uint8_t)fw;
+                if (FINE) {
+#pragma unroll
+                    for (int w = 0; w < 4; ++w) {
+                        const int rows = max(0, min(32, S - (m * BLOCK_M + 32 * w)));
+                        s_out[1 + w][col] = (uint8_t)(cnt[w] == 0 ? 0 : cnt[w] == rows * cols_in_range ? 2 : 1);
+                    }
                 }
-                continue;
+                const int total = cnt[0] + cnt[1] + cnt[2] + cnt[3];
+                // full over in-range cells (:149-153)
+                s_out[0][col] = (uint8_t)(total == 0 ? 0 : total == rows_in_range * cols_in_range ? 2 : 1);
             }
         }
-        int cnt_a = 0, cnt_b = 0;  // rows [64 half, +32) and [64 half + 32, +32)
-#pragma unroll 8
-        for (int r = 0; r < 32; ++r) {
-            const int ri = half * 64 + r;
-            cnt_a += allow_rule(q_bits[ri], kf, (int64_t)m * BLOCK_M + ri, j) ? 1 : 0;
-            cnt_b += allow_rule(q_bits[ri + 32], kf, (int64_t)m * BLOCK_M + ri + 32, j) ? 1 : 0;
+        __syncthreads();
+        const int n0 = bx * FLAG_COLS_PER_BLOCK;
+        if (tid < FLAG_COLS_PER_BLOCK && n0 + tid < num_n)  // the flag row may start anywhere: single bytes
+            flags[(int64_t)b * flags_stride_b + (int64_t)m * flags_stride_m + n0 + tid] = (int8_t)s_out[0][tid];
+        if (FINE && tid >= 64 && tid < 68) {  // rows of the class matrix are padded to 16 bytes: one 8-byte store
+            static_assert(FLAG_COLS_PER_BLOCK == 8, "one 64-bit word per row");
+            const int w = tid - 64;
+            *(unsigned long long*)(fine + (int64_t)b * fine_sb + (int64_t)(4 * m + w) * fine_ss + n0) =
+                *(const unsigned long long*)s_out[1 + w];
         }
-        const int cols_in_range = min(BLOCK_N, S - n * BLOCK_N);
-        const int col = wave * FLAG_TILES_PER_WAVE + t;
-        if (FINE) {
-#pragma unroll
-            for (int off = 16; off > 0; off >>= 1) {  // over the 32 columns, inside each half of the wave
-                cnt_a += __shfl_xor(cnt_a, off);
-                cnt_b += __shfl_xor(cnt_b, off);
-            }
-            if ((lane & 31) == 0) {
-#pragma unroll
-                for (int x = 0; x < 2; ++x) {
-                    const int w = 2 * half + x, c = x ? cnt_b : cnt_a;
-                    const int rows = max(0, min(32, S - (m * BLOCK_M + 32 * w)));
-                    s_out[1 + w][col] = (uint8_t)(c == 0 ? 0 : c == rows * cols_in_range ? 2 : 1);
-                }
-            }
-            int cnt = cnt_a + cnt_b;
-            cnt += __shfl_xor(cnt, 32);
-            // full over in-range cells (:149-153)
-            if (lane == 0) s_out[0][col] = (uint8_t)(cnt == 0 ? 0 : cnt == rows_in_range * cols_in_range ? 2 : 1);
-        } else {
-            int cnt = cnt_a + cnt_b;
-#pragma unroll
-            for (int off = 32; off > 0; off >>= 1) cnt += __shfl_xor(cnt, off);
-            if (lane == 0) s_out[0][col] = (uint8_t)(cnt == 0 ? 0 : cnt == rows_in_range * cols_in_range ? 2 : 1);
-        }
-    }
-    __syncthreads();
-    const int n0 = blockIdx.x * FLAG_COLS_PER_BLOCK;
-    if (tid < FLAG_COLS_PER_BLOCK && n0 + tid < num_n)  // the flag row may start anywhere: single bytes
-        flags[(int64_t)b * flags_stride_b + (int64_t)m * flags_stride_m + n0 + tid] = (int8_t)s_out[0][tid];
-    if (FINE && tid >= 64 && tid < 68) {  // rows of the class matrix are padded to 16 bytes: one 8-byte store
-        static_assert(FLAG_COLS_PER_BLOCK == 8, "one 64-bit word per row");
-        const int w = tid - 64;
-        *(unsigned long long*)(fine + (int64_t)b * fine_sb + (int64_t)(4 * m + w) * fine_ss + n0) =
-            *(const unsigned long long*)s_out[1 + w];
     }
 }
 
@@ -346,9 +406,11 @@ __global__ __launch_bounds__(FLAG_WAVES * 64) void indexed_plan_kernel(
         const int part = blockIdx.y;
         const int ns = (Sq + 31) / 32, slots = 4 * (int)gridDim.y;
         if (part * 256 < slots)
-            slice_order_ranked([&](int s, unsigned long long& k1,
-                                   unsigned long long& k2) { slice_sort_key_indexed(qrow, qpos, Sq, ns, s, k1, k2); },
-                               ns, slots, part, order + (int64_t)b * order_sb);
+            slice_order_ranked(
+                [&](int base, unsigned long long* sk) {
+                    slice_sort_key_indexed(qrow, qpos, Sq, ns, base + (int)threadIdx.x, sk[2 * threadIdx.x], sk[2 * threadIdx.x + 1]);
+                },
+                ns, slots, part, order + (int64_t)b * order_sb);
         return;
     }
     __shared__ int64_t q_bits[BLOCK_M];
@@ -605,10 +667,12 @@ int launch_ds_entries(const uint8_t* fine, int64_t fine_sb, int64_t fine_ss, int
 int launch_tile_flags(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int64_t flags_stride_b,
                       int64_t flags_stride_m, int B, int S, hipStream_t stream) {
     const int num_m = (S + BLOCK_M - 1) / BLOCK_M, num_n = (S + BLOCK_N - 1) / BLOCK_N;
-    dim3 grid((num_n + FLAG_COLS_PER_BLOCK - 1) / FLAG_COLS_PER_BLOCK, num_m, B);
+    const int flag_groups = (num_n + FLAG_COLS_PER_BLOCK - 1) / FLAG_COLS_PER_BLOCK;
+    const int flag_blocks_x = min(flag_groups, FLAG_MAX_BLOCKS_X);
+    dim3 grid(flag_blocks_x, num_m, B);
     hipLaunchKernelGGL(tile_flags_kernel<false>, grid, dim3(FLAG_WAVES * 64), 0, stream, bf, bf_stride_b, flags,
                        flags_stride_b, flags_stride_m, S, num_n, (uint8_t*)nullptr, (int64_t)0, (int64_t)0, (int*)nullptr,
-                       (int64_t)0, 0, (int*)nullptr);
+                       (int64_t)0, flag_blocks_x, flag_groups, (int*)nullptr);
     return (int)hipGetLastError();
 }
 
@@ -616,13 +680,14 @@ int launch_tile_plan(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int6
                      int64_t flags_stride_m, uint8_t* fine, int64_t fine_sb, int64_t fine_ss, int* order,
                      int64_t order_sb, int* pair_count, int B, int S, hipStream_t stream) {
     const int num_m = (S + BLOCK_M - 1) / BLOCK_M, num_n = (S + BLOCK_N - 1) / BLOCK_N;
-    const int flag_blocks_x = (num_n + FLAG_COLS_PER_BLOCK - 1) / FLAG_COLS_PER_BLOCK;
+    const int flag_groups = (num_n + FLAG_COLS_PER_BLOCK - 1) / FLAG_COLS_PER_BLOCK;
+    const int flag_blocks_x = min(flag_groups, FLAG_MAX_BLOCKS_X);
     // one more column of workgroups: (flag_blocks_x, part, b) ranks 256 slices; 4 num_m slots need
     // ceil(4 num_m / 256) <= num_m parts
     dim3 grid(flag_blocks_x + 1, num_m, B);
     hipLaunchKernelGGL(tile_flags_kernel<true>, grid, dim3(FLAG_WAVES * 64), 0, stream, bf, bf_stride_b, flags,
                        flags_stride_b, flags_stride_m, S, num_n, fine, fine_sb, fine_ss, order, order_sb, flag_blocks_x,
-                       pair_count);
+                       flag_groups, pair_count);
     return (int)hipGetLastError();
 }
 
