@@ -32,6 +32,16 @@ def build_plan(bf):
     return flags, fine.clone(), order.clone(), plan
 
 
+def flags_only(bf):
+    """The flags through bam_tile_flags, the entry point that builds no plan (same kernel, other instantiation)."""
+    B, S = bf.shape
+    out = torch.empty((B, -(-S // 128), -(-S // 32)), dtype=torch.int8, device=bf.device)
+    _bam_hip.call("bam_tile_flags", bf.data_ptr(), bf.stride(0), out.data_ptr(), out.stride(0), out.stride(1), B, S,
+                  torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    return out
+
+
 def brute_force_fine(mask, S):
     """Class of every 32 x 32 tile from the (B, S, S) bool mask: 0 nothing allowed, 2 every in-range cell."""
     B = mask.shape[0]
@@ -70,6 +80,30 @@ def test_fine_classes_and_order_on_irregular_bitfields(S, wide):
         for gval in set(groups):
             members = [s for s in rest if int(sig[s]) == gval]
             assert members == sorted(members)
+
+
+@pytest.mark.parametrize("S", [33, 96, 129, 500, 1111])
+@pytest.mark.parametrize("max_run", [1, 3])
+def test_classes_when_the_bitfield_changes_every_few_rows(S, max_run):
+    # up to 32 runs of equal bitfields inside one 32-row slice: text, five modalities (one above bit 31) and 0, at random
+    g = torch.Generator().manual_seed(1000 * S + max_run)
+    text = (1 << 62) | 1 | (1 << 3) | (1 << 40)
+    values = torch.tensor([text, 1 << 1, 1 << 2, 1 << 3, 1 << 4, 1 << 40, 0], dtype=torch.int64)
+    bf = torch.empty((2, S), dtype=torch.int64)
+    for b in range(2):
+        pos = 0
+        while pos < S:
+            run = int(torch.randint(1, max_run + 1, (1,), generator=g))
+            bf[b, pos : pos + run] = values[int(torch.randint(0, len(values), (1,), generator=g))]
+            pos += run
+    flags, fine, order, _ = build_plan(bf.to(dev()))
+    assert torch.equal(flags.cpu(), O.tile_flags(bf))
+    assert torch.equal(flags_only(bf.to(dev())).cpu(), O.tile_flags(bf))  # the kernel form that writes no classes
+    n = -(-S // 32)
+    assert torch.equal(fine[:, :n].cpu(), brute_force_fine(O.materialize_mask(bf), S))
+    for b in range(2):
+        o = order[b].cpu().tolist()
+        assert sorted(o[:n]) == list(range(n)) and all(x == -1 for x in o[n:])
 
 
 @pytest.mark.parametrize("name", ["C1", "C2", "C4"])
