@@ -11,7 +11,7 @@
 // keys.  decode_split_kernel: one wave per (range of 32-key tiles, kv head, batch element); the q heads of the kv
 // head (up to 32 per workgroup) are the 32 "query rows" of the attention kernels' S^T = K Q^T layout, so the tile is
 // read once for all of them:
-//   S^T (32 keys x 32 heads) = K Q^T with the K rows as the A operand straight from global memory,
+//   S^T (32 keys x 32 heads) = K Q^T with the K rows of the tile (copied global -> LDS) as the A operand,
 //   a lane owns one head (softmax state = per-lane scalars), P^T feeds O^T = V^T P^T from registers,
 //   V^T comes from the V tile (copied global -> LDS) through the transposing LDS read.
 // Every split writes its unnormalized output, maximum and sum for the heads that exist; decode_combine_kernel merges
@@ -25,10 +25,13 @@ namespace bam {
 constexpr int DEC_KT = 32;  // keys per tile
 
 template <typename T, int D>
-__global__ __launch_bounds__(64) void decode_split_kernel(const DecodeParams p) {
+__global__ __launch_bounds__(64, 2) void decode_split_kernel(const DecodeParams p) {
     constexpr int NCH = D / 8, KK = D / 16, DB = D / 32;
-    __shared__ u32x4 sV[DEC_KT * NCH];
-    __shared__ __attribute__((aligned(16))) unsigned short sQ[32 * D];
+    // one K tile (refilled as soon as its rows are in registers) and two V tiles (the copy of tile t + 1 runs under the
+    // arithmetic of tile t); before the loop the V tiles' memory stages a q that is not 16-byte aligned
+    __shared__ u32x4 sK[DEC_KT * NCH];
+    __shared__ u32x4 sV[2][DEC_KT * (NCH < 8 ? 8 : NCH)];
+    static_assert(sizeof(sV) >= 32 * D * 2, "the q staging area fits");
 
     const int lane = threadIdx.x, hi = lane >> 5, l32 = lane & 31, half16 = (lane >> 4) & 1;
     const int split = blockIdx.x, hk = blockIdx.y;
@@ -40,19 +43,36 @@ __global__ __launch_bounds__(64) void decode_split_kernel(const DecodeParams p) 
     const int n_tiles = (p.Sk - first + DEC_KT - 1) / DEC_KT;
     const int t0 = split * p.tiles_per_split, t1 = min(n_tiles, t0 + p.tiles_per_split);
 
-    // ---- Q: rows = heads, zero rows past the last head; element-wise loads (q is only 2-byte aligned) ----
-    for (int i = lane; i < 32 * D; i += 64) {
-        const int r = i / D, d = i % D;
-        sQ[i] = r < rows ? ((const unsigned short*)p.q)[(int64_t)b * p.q_sb + (int64_t)(h0 + r) * p.q_sh + d] : (unsigned short)0;
-    }
-    __syncthreads();
+    // ---- Q: rows = heads, zero rows past the last head ----
     u32x4 qreg[KK];
+    const bool q_aligned = ((reinterpret_cast<uintptr_t>(p.q) | (uintptr_t)(2 * p.q_sb) | (uintptr_t)(2 * p.q_sh)) & 15u) == 0;
+    if (q_aligned) {  // wave-uniform: the lane's 16-byte pieces straight from global memory
+        const char* qrow = (const char*)p.q + 2 * ((int64_t)b * p.q_sb + (int64_t)(h0 + min(l32, rows - 1)) * p.q_sh);
 #pragma unroll
-    for (int kk = 0; kk < KK; ++kk) qreg[kk] = *(const u32x4*)&sQ[l32 * D + 16 * kk + 8 * hi];
+        for (int kk = 0; kk < KK; ++kk) {
+            const u32x4 x = *(const u32x4*)(qrow + (2 * kk + hi) * 16);
+            const u32x4 z = {0u, 0u, 0u, 0u};
+            qreg[kk] = l32 < rows ? x : z;
+        }
+    } else {  // element-wise loads through LDS (a view of q may be only 2-byte aligned)
+        unsigned short* sQ = (unsigned short*)sV;
+        for (int i = lane; i < rows * D; i += 64) {
+            const int r = i / D, d = i % D;
+            sQ[i] = ((const unsigned short*)p.q)[(int64_t)b * p.q_sb + (int64_t)(h0 + r) * p.q_sh + d];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < KK; ++kk) {
+            const u32x4 z = {0u, 0u, 0u, 0u};
+            qreg[kk] = l32 < rows ? *(const u32x4*)&sQ[l32 * D + 16 * kk + 8 * hi] : z;
+        }
+        wait_lds();  // the staging area becomes the V tiles
+    }
 
     const char* kbase = (const char*)p.k + 2 * ((int64_t)b * p.k_sb + (int64_t)hk * p.k_sh);
     const char* vbase = (const char*)p.v + 2 * ((int64_t)b * p.v_sb + (int64_t)hk * p.v_sh);
-    TileStage<D, DEC_KT, 64> stV;
+    TileStage<D, DEC_KT, 64> stK, stV;
+    stK.setup(2 * p.k_ss, lane);
     stV.setup(2 * p.v_ss, lane);
 
     f32x16 o[DB];
@@ -65,18 +85,31 @@ __global__ __launch_bounds__(64) void decode_split_kernel(const DecodeParams p) 
     for (int i = 0; i < 16; ++i) zero16[i] = 0.f;
     float m_i = -INFINITY, l_i = 0.f;  // maximum in the log2 domain; this lane's share of the sum (16 of 32 keys)
 
-    for (int t = t0; t < t1; ++t) {
+    // Tile t: its K rows into the K buffer, its V rows into V buffer buf (zero rows past the end of the cache).  Both
+    // travel as 1 KiB pieces, global -> LDS; the K rows are the A operand of S^T = K Q^T (one 16-byte LDS read per MFMA).
+    auto fetch = [&](int t, int buf) {
         const int key0 = first + t * DEC_KT;
         const int nvalid = min(DEC_KT, p.Sk - key0);
-        // K rows of the tile as the A operand (rows past the end repeat the last one; their scores are masked below)
-        const char* krow = kbase + 2 * (int64_t)(key0 + min(l32, nvalid - 1)) * p.k_ss;
+        stK.load(kbase + 2 * (int64_t)key0 * p.k_ss, sK, nvalid, lane);
+        stV.load(vbase + 2 * (int64_t)key0 * p.v_ss, sV[buf], nvalid, lane);
+    };
+
+    if (t0 < t1) {
+        fetch(t0, 0);
+        wait_async();
+        wait_lds();
+    }
+    for (int t = t0; t < t1; ++t) {
+        const int cur = (t - t0) & 1;
+        const int nvalid = min(DEC_KT, p.Sk - (first + t * DEC_KT));
         u32x4 ka[KK];
 #pragma unroll
-        for (int kk = 0; kk < KK; ++kk) ka[kk] = *(const u32x4*)(krow + (2 * kk + hi) * 16);
-        // V tile -> LDS (zero rows past the end); the previous tile's reads of it have all been consumed by MFMAs
+        for (int kk = 0; kk < KK; ++kk) ka[kk] = lds_read_chunk<D>(sK, l32, 2 * kk + hi);
         wait_lds();
-        stV.load(vbase + 2 * (int64_t)key0 * p.v_ss, sV, nvalid, lane);
-
+        // The next tile is requested as soon as this one's K rows are in registers: its latency runs under this
+        // tile's arithmetic and under the other waves of the compute unit.  (The reads of that V buffer ended before
+        // the previous iteration did.)
+        if (t + 1 < t1) fetch(t + 1, cur ^ 1);
         f32x16 s = zero16;
 #pragma unroll
         for (int kk = 0; kk < KK; ++kk) s = T::mfma(ka[kk], qreg[kk], s);
@@ -111,15 +144,17 @@ __global__ __launch_bounds__(64) void decode_split_kernel(const DecodeParams p) 
 #pragma unroll
         for (int h2 = 0; h2 < 2; ++h2) pb[h2] = pack8<T>(s, 8 * h2);
 
-        wait_async();   // the V tile has landed (one wave: no barrier needed, LDS reads follow in program order)
-        wait_lds();     // ... and so have the synchronous stores of a ragged tile
 #pragma unroll
         for (int h2 = 0; h2 < 2; ++h2)
 #pragma unroll
             for (int db = 0; db < DB; ++db) {
-                const u32x4 va = lds_read_transposed<D>(sV, lane, 16 * h2 + 4 * hi, 32 * db + 16 * half16);
+                const u32x4 va = lds_read_transposed<D>(sV[cur], lane, 16 * h2 + 4 * hi, 32 * db + 16 * half16);
                 o[db] = T::mfma(va, pb[h2], o[db]);
             }
+        // the next tile has landed (one wave: no barrier needed, LDS reads follow in program order), this tile's
+        // reads of its V buffer are done, and so are the synchronous stores of a ragged next tile
+        wait_async();
+        wait_lds();
     }
 
     // ---- this split's result for head h0 + l32: O^T fragment register i of block db <-> column 32 db + 8 (i/4) + 4 hi + i%4
@@ -218,15 +253,17 @@ int launch_decode(const DecodeParams& p, int dtype, hipStream_t stream) {
     return dtype == 1 ? launch_decode_t<BF16>(p, stream) : launch_decode_t<F16>(p, stream);
 }
 
-// How the keys of one decode step are split over workgroups: about ten waves per compute unit, at least two tiles per
-// split where the cache is long enough.  Shared by the workspace size and the launch.
+// How the keys of one decode step are split over workgroups: about four waves per compute unit, all resident at once
+// (1024 workgroups; more of them only add per-workgroup set-up and partial results to merge: 2560 measured 10 % slower,
+// 512 leave too little in flight), at least two tiles per split where the cache is long enough.  Shared by the
+// workspace size and the launch.
 void decode_split_plan(int B, int Hq, int Hkv, int Sk, int window, int* nsplit, int* tiles_per_split, int* row_groups) {
     const int G = Hq / Hkv;
     const int rgs = (G + 31) / 32;
     const int keys = (window > 0 && window < Sk) ? window : Sk;
     const int n_tiles = (keys + DEC_KT - 1) / DEC_KT;
     const int64_t units = (int64_t)B * Hkv * rgs;
-    int64_t want = (2560 + units - 1) / units;
+    int64_t want = (1024 + units - 1) / units;
     const int most = n_tiles >= 2 ? n_tiles / 2 : 1;
     if (want > most) want = most;
     if (want < 1) want = 1;

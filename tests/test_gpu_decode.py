@@ -113,6 +113,21 @@ def test_decode_step_large_scores_and_a_cache_view_with_strides():
         assert (out.float().cpu() - want).abs().max().item() <= 4e-2 * max(1.0, want.abs().max().item())
 
 
+@pytest.mark.parametrize("D", [64, 128])
+def test_decode_step_with_a_query_view_that_is_only_two_byte_aligned(D):
+    # the kernel reads an aligned q with 16-byte loads and any other q element by element: both must agree
+    q, k, v = inputs(2, 8, 2, 777, D, torch.bfloat16, seed=D)
+    want = O.decode_step(q, k, v)
+    wide = torch.zeros(2, 8, 1, D + 1, dtype=q.dtype)
+    wide[..., 1:] = q
+    view = wide.to(dev())[..., 1:]  # first element at byte offset 2, head stride D + 1
+    assert view.data_ptr() % 16 != 0 and view.stride(-1) == 1
+    out, _ = interface.bitfield_attention_forward(_Module().eval(), view, k.to(dev()), v.to(dev()), None)
+    aligned = decode(q, k, v)
+    assert torch.equal(out.cpu(), aligned)
+    assert (aligned.float() - want).abs().max().item() <= O_MAX_ABS
+
+
 def test_training_mode_takes_the_bitfield_path_and_bad_arguments_are_refused():
     q, k, v = (t.to(dev()) for t in inputs(1, 4, 2, 8, 64, torch.bfloat16))
     with pytest.raises(AssertionError, match="int64"):
