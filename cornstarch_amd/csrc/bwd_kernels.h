@@ -708,8 +708,6 @@ __global__ __launch_bounds__(DQ_THREADS, D == 128 ? 2 : 3) void bwd_dq_kernel(co
     const int h = hk * G + g;
     const WaveSlices ws = pick_wave_slices(p, b, ub / p.B);  // group 0 is the heaviest
 
-    if (wave == 0) build_key_tile_list(ws, p.num_n, Sk, lane, 0, sList, &sCount);  // first pass (usually the only one)
-
     const int slice = __builtin_amdgcn_readfirstlane(wave == 0 ? ws.slice[0] : wave == 1 ? ws.slice[1] : wave == 2 ? ws.slice[2] : ws.slice[3]);
     const int qrow = (slice < 0 ? 0 : slice) * 32 + l32;
     const bool qvalid = slice >= 0 && qrow < Sq;
@@ -729,14 +727,16 @@ __global__ __launch_bounds__(DQ_THREADS, D == 128 ? 2 : 3) void bwd_dq_kernel(co
         }
     }
     const int64_t qf = (!DENSE && qvalid) ? p.bfq[(int64_t)b * p.bfq_sb + qrow] : 0;
-    const QueryBits qb = make_query_bits(qf, (IDX && qvalid) ? p.posq[qrow] : qrow);
-    float lse2 = INFINITY, dlt = 0.f;
+    float lse_row = 0.f, dlt = 0.f;
     if (qvalid) {
         const int64_t off = ((int64_t)b * p.Hq + h) * p.Sq_rounded + qrow;
-        const float l = p.lse[off];
-        lse2 = (l == -INFINITY) ? INFINITY : l * LOG2E;
+        lse_row = p.lse[off];
         dlt = p.delta[off];
     }
+    // (the row loads above are in flight while wave 0 reads the class rows)
+    if (wave == 0) build_key_tile_list(ws, p.num_n, Sk, lane, 0, sList, &sCount);  // first pass (usually the only one)
+    const QueryBits qb = make_query_bits(qf, (IDX && qvalid) ? p.posq[qrow] : qrow);
+    const float lse2 = (!qvalid || lse_row == -INFINITY) ? INFINITY : lse_row * LOG2E;
 
     f32x16 dq[DB];
 #pragma unroll
