@@ -82,10 +82,8 @@ __global__ __launch_bounds__(DQS_THREADS, 2) void bwd_dq_saved_kernel(const Attn
     const int Sq = p.Sq, Sk = p.Sk;
     const int G = p.Hq / p.Hkv;
 
-    int unit, g;
-    xcd_group_map(blockIdx.x, p.num_m * p.B * p.Hkv, G, unit, g);
-    const int hk = unit % p.Hkv;
-    const int ub = unit / p.Hkv;
+    int ub, hk, g;
+    head_unit_map(blockIdx.x, p.num_m * p.B, p.Hkv, G, ub, hk, g);
     const int b = ub % p.B;
     const int h = hk * G + g;
     const WaveSlices ws = pick_wave_slices(p, b, ub / p.B);  // the plan's order (the launcher requires a plan)

@@ -57,10 +57,8 @@ __global__ __launch_bounds__(FWD_THREADS, D == 128 ? 2 : 3) void fwd_kernel(cons
     const int Sq = p.Sq, Sk = p.Sk;
     const int G = p.Hq / p.Hkv;
 
-    int unit, g;
-    xcd_group_map(blockIdx.x, p.num_m * p.B * p.Hkv, G, unit, g);
-    const int hk = unit % p.Hkv;
-    const int ub = unit / p.Hkv;
+    int ub, hk, g;
+    head_unit_map(blockIdx.x, p.num_m * p.B, p.Hkv, G, ub, hk, g);
     const int b = ub % p.B;
     const int h = hk * G + g;
     const int grp = ub / p.B;
