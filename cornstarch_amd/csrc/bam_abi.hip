@@ -154,6 +154,9 @@ int fill_plan(bam::AttnParams& p, const char* who, const bam_plan* plan, int B, 
     p.order = plan->order;
     p.order_sb = plan->order_stride_b;
     p.tile_order = plan->ds_tile_order;  // may be null
+    if (reinterpret_cast<uintptr_t>(plan->group_order) & 3u)
+        return fail(BAM_ERR_INVALID_ARGUMENT, "%s: plan: misaligned group order", who);
+    p.group_order = plan->group_order;   // may be null
     // hand-over of dS from dK/dV to dQ: only with a workspace, for the head dim and lengths its kernels cover
     if (plan->ds_workspace != nullptr && plan->ds_entry != nullptr && plan->ds_tile_base != nullptr && p.D == 128 &&
         Sk <= bam::MAX_LIST * 64) {
@@ -309,7 +312,7 @@ extern "C" {
 
 const char* bam_last_error(void) { return g_error; }
 
-int bam_abi_version(void) { return 8; }
+int bam_abi_version(void) { return 9; }
 
 int bam_tile_flags(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int64_t flags_stride_b,
                    int64_t flags_stride_m, int B, int S, void* stream) {
@@ -327,6 +330,7 @@ namespace {
 struct PlanLayout {
     int64_t fine_ss, fine_sb, order_sb, entry_sb, fine_off, order_off, entry_off, base_off, count_off, bytes;
     int64_t row_sn, row_sb, col_ss, col_sb, row_off, col_off, bytes_with_bits, tile_count_off, tile_order_off;
+    int64_t group_count_off, group_order_off;
 };
 PlanLayout plan_layout(int B, int Sq, int Sk) {
     const int64_t num_m = (Sq + 127) / 128, num_n = (Sk + 31) / 32, slots = 4 * num_m;
@@ -343,7 +347,9 @@ PlanLayout plan_layout(int B, int Sq, int Sk) {
     l.count_off = l.base_off + up(B * ((Sk + 127) / 128) * 4, 256);
     l.tile_count_off = l.count_off + 256;
     l.tile_order_off = l.tile_count_off + up(B * ((Sk + 127) / 128) * 4, 256);
-    l.bytes = l.tile_order_off + up(B * ((Sk + 127) / 128) * 4, 256);
+    l.group_count_off = l.tile_order_off + up(B * ((Sk + 127) / 128) * 4, 256);
+    l.group_order_off = l.group_count_off + up(B * num_m * 4, 256);
+    l.bytes = l.group_order_off + up(B * num_m * 4, 256);
     // the packed mask of bam_mask_tile_plan: rows padded to 128, keys to 128, 32-key blocks to an even number
     l.row_sn = num_m * 128;
     l.row_sb = ((num_n + 1) & ~(int64_t)1) * l.row_sn;
@@ -392,6 +398,7 @@ int place_plan(const char* who, void* workspace, int64_t workspace_bytes, int B,
     plan->ds_tile_base = (const int32_t*)(w + l.base_off);
     plan->ds_count = (const int32_t*)(w + l.count_off);
     plan->ds_tile_order = (int64_t)B * ((Sk + 127) / 128) <= 1024 ? (const int32_t*)(w + l.tile_order_off) : nullptr;
+    plan->group_order = (int64_t)B * ((Sq + 127) / 128) <= 1024 ? (const int32_t*)(w + l.group_order_off) : nullptr;
     plan->ds_workspace = nullptr;
     plan->ds_capacity = 0;
     plan->row_bits = with_bits ? (const uint32_t*)(w + l.row_off) : nullptr;
@@ -414,8 +421,9 @@ int number_pairs(const char* who, const bam_plan* plan, const PlanLayout& l, voi
                                            const_cast<int*>(plan->ds_tile_base),
                                            const_cast<int*>(plan->ds_count),
                                            (int*)((char*)workspace + l.tile_count_off),
-                                           const_cast<int*>(plan->ds_tile_order),
-                                           (hipStream_t)stream),
+                                           const_cast<int*>(plan->ds_tile_order), plan->order, plan->order_stride_b,
+                                           (int*)((char*)workspace + l.group_count_off),
+                                           const_cast<int*>(plan->group_order), (hipStream_t)stream),
                     who);
 }
 }  // namespace

@@ -71,6 +71,10 @@ struct AttnParams {
     // Optional (plan): the key tiles of all sequences (code b * num_kt + t) by falling number of (slice, tile) pairs
     // with work; the dK/dV kernel takes its workgroups in this order (null: early tiles first).
     const int* tile_order;
+    // Optional (plan): the groups of four slices of all sequences (code b * num_m + group) by falling number of
+    // 64-key tiles their workgroup visits; the forward and dQ kernels take their workgroups in this order (null:
+    // group by group, the sequences of the batch side by side).
+    const int* group_order;
     // MASK_DENSE with a plan: the mask packed to bits, once per orientation (null = read the mask bytes).
     // row_bits (B, row_bits_sn-strided 32-key blocks, rows): bit c of word (n, r) = mask[r][32 n + c];
     // col_bits (B, 32-row slices, keys): bit r of word (s, k) = mask[32 s + r][k].  Out-of-range cells are 0.
@@ -128,9 +132,12 @@ int launch_mask_tile_plan(const uint8_t* mask, int8_t* flags, int64_t flags_stri
 // tile_base (B, ceil(Sk/128)) ints: number of the first pair of each key tile (pairs are numbered tile by tile).
 // *count must be zero when the kernel starts (the plan kernels reset it).  tile_count (B, ceil(Sk/128)) scratch and
 // tile_order (B * ceil(Sk/128)): the key tiles by falling number of pairs, written by a second small launch; both may
-// be null, and no order is written beyond 1024 tiles.
+// be null, and no order is written beyond 1024 tiles.  The same for the groups of four slices in the plan's slice
+// order (order, order_sb): group_count (B * num_m) scratch, group_order (B * num_m) = the groups by falling number of
+// 64-key tiles they visit.
 int launch_ds_entries(const uint8_t* fine, int64_t fine_sb, int64_t fine_ss, int B, int Sq, int Sk, int* entry,
-                      int64_t entry_sb, int* tile_base, int* count, int* tile_count, int* tile_order, hipStream_t stream);
+                      int64_t entry_sb, int* tile_base, int* count, int* tile_count, int* tile_order, const int* order,
+                      int64_t order_sb, int* group_count, int* group_order, hipStream_t stream);
 int launch_fwd(const AttnParams& p, int dtype, hipStream_t stream);
 int launch_bwd_preprocess(const AttnParams& p, int dtype, hipStream_t stream);
 int launch_bwd_dkdv(const AttnParams& p, int dtype, hipStream_t stream);

@@ -84,9 +84,14 @@ __global__ __launch_bounds__(DQS_THREADS, 2) void bwd_dq_saved_kernel(const Attn
 
     int ub, hk, g;
     head_unit_map(blockIdx.x, p.num_m * p.B, p.Hkv, G, ub, hk, g);
-    const int b = ub % p.B;
+    int b = ub % p.B, grp = ub / p.B;
+    if (p.group_order != nullptr) {  // with a plan: the groups of all sequences by falling length of their tile lists
+        const int code = p.group_order[ub];
+        b = code / p.num_m;
+        grp = code - b * p.num_m;
+    }
     const int h = hk * G + g;
-    const WaveSlices ws = pick_wave_slices(p, b, ub / p.B);  // the plan's order (the launcher requires a plan)
+    const WaveSlices ws = pick_wave_slices(p, b, grp);  // the plan's order (the launcher requires a plan)
 
     if (wave == 0) build_key_half_list(ws, p.num_n, Sk, lane, sList, &sCount);
 

@@ -702,9 +702,14 @@ __global__ __launch_bounds__(DQ_THREADS, D == 128 ? 2 : 3) void bwd_dq_kernel(co
 
     int ub, hk, g;
     head_unit_map(blockIdx.x, p.num_m * p.B, p.Hkv, G, ub, hk, g);
-    const int b = ub % p.B;
+    int b = ub % p.B, grp = ub / p.B;
+    if (p.group_order != nullptr) {  // with a plan: the groups of all sequences by falling length of their tile lists
+        const int code = p.group_order[ub];
+        b = code / p.num_m;
+        grp = code - b * p.num_m;
+    }
     const int h = hk * G + g;
-    const WaveSlices ws = pick_wave_slices(p, b, ub / p.B);  // group 0 is the heaviest
+    const WaveSlices ws = pick_wave_slices(p, b, grp);  // group 0 is the heaviest
 
     const int slice = __builtin_amdgcn_readfirstlane(wave == 0 ? ws.slice[0] : wave == 1 ? ws.slice[1] : wave == 2 ? ws.slice[2] : ws.slice[3]);
     const int qrow = (slice < 0 ? 0 : slice) * 32 + l32;

@@ -59,9 +59,13 @@ __global__ __launch_bounds__(FWD_THREADS, D == 128 ? 2 : 3) void fwd_kernel(cons
 
     int ub, hk, g;
     head_unit_map(blockIdx.x, p.num_m * p.B, p.Hkv, G, ub, hk, g);
-    const int b = ub % p.B;
+    int b = ub % p.B, grp = ub / p.B;
+    if (p.group_order != nullptr) {  // with a plan: the groups of all sequences by falling length of their tile lists
+        const int code = p.group_order[ub];
+        b = code / p.num_m;
+        grp = code - b * p.num_m;
+    }
     const int h = hk * G + g;
-    const int grp = ub / p.B;
     const WaveSlices ws = pick_wave_slices(p, b, grp);  // group 0 is the heaviest
 
     if (wave == 0) build_key_tile_list(ws, p.num_n, Sk, lane, 0, sList, &sCount);  // first pass (usually the only one)

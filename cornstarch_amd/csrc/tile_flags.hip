@@ -580,11 +580,41 @@ __global__ __launch_bounds__(DS_NUM_THREADS) void ds_entries_kernel(const uint8_
                                                                    int64_t fine_ss, int slots, int nkt, int num_n,
                                                                    int* __restrict__ entry, int64_t entry_sb,
                                                                    int* __restrict__ tile_base, int* __restrict__ count,
-                                                                   int* __restrict__ tile_count) {
+                                                                   int* __restrict__ tile_count,
+                                                                   const int* __restrict__ order, int64_t order_sb,
+                                                                   int* __restrict__ group_count) {
     __shared__ int wave_sum[DS_NUM_THREADS / 64];
     __shared__ int s_base;
-    const int t = blockIdx.x, b = blockIdx.y;
+    const int b = blockIdx.y;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    if ((int)blockIdx.x >= nkt) {
+        // Extra workgroups, one per group of four slices of the slice order: how many 64-key tiles the forward / dQ
+        // workgroup of that group visits (the union over its slices), which is what group_order ranks the groups by.
+        const int grp = blockIdx.x - nkt, num_m = slots / 4;
+        const int* ord = order + (int64_t)b * order_sb + 4 * grp;
+        const uint8_t* rows[4];
+#pragma unroll
+        for (int x = 0; x < 4; ++x) rows[x] = ord[x] >= 0 ? fine + (int64_t)b * fine_sb + (int64_t)ord[x] * fine_ss : nullptr;
+        int visits = 0;
+        for (int kt = tid; 2 * kt < num_n; kt += DS_NUM_THREADS) {
+            unsigned any = 0;
+#pragma unroll
+            for (int x = 0; x < 4; ++x)
+                if (rows[x] != nullptr) any |= rows[x][2 * kt] | (2 * kt + 1 < num_n ? rows[x][2 * kt + 1] : 0);
+            visits += any != 0 ? 1 : 0;
+        }
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) visits += __shfl_xor(visits, off);
+        if (lane == 0) wave_sum[wave] = visits;
+        __syncthreads();
+        if (tid == 0) {
+            int total = 0;
+            for (int w = 0; w < DS_NUM_THREADS / 64; ++w) total += wave_sum[w];
+            group_count[b * num_m + grp] = total;
+        }
+        return;
+    }
+    const int t = blockIdx.x;
     const uint8_t* col = fine + (int64_t)b * fine_sb + 4 * t;
     unsigned valid = 0;  // which of the tile's four 32-key columns exist
 #pragma unroll
@@ -628,10 +658,20 @@ __global__ __launch_bounds__(DS_NUM_THREADS) void ds_entries_kernel(const uint8_
 // The key tiles (code b * nkt + t) sorted by their number of pairs, most first (ties: lower code first): the order in
 // which the dK/dV kernel takes them, so that the long workgroups start first whatever the mask looks like.
 // 64 tiles per workgroup, four threads per tile, each comparing against a quarter of all counts (staged in LDS).
+// blockIdx.y = 1 ranks a second, independent array the same way (the groups of four slices, for the forward and dQ
+// kernels); either array may be absent (n = 0).
 __global__ __launch_bounds__(256) void tile_order_kernel(const int* __restrict__ tile_count, int n_tiles,
-                                                         int* __restrict__ tile_order) {
+                                                         int* __restrict__ tile_order,
+                                                         const int* __restrict__ group_count, int n_groups,
+                                                         int* __restrict__ group_order) {
     __shared__ __attribute__((aligned(16))) int s_cnt[DS_MAX_ORDERED_TILES];
     const int tid = threadIdx.x;
+    if (blockIdx.y == 1) {
+        tile_count = group_count;
+        n_tiles = n_groups;
+        tile_order = group_order;
+    }
+    if ((int)blockIdx.x * 64 >= n_tiles) return;  // (workgroup-uniform)
     const int padded = (n_tiles + 15) & ~15;
     for (int i = tid; i < padded; i += 256) s_cnt[i] = i < n_tiles ? tile_count[i] : -1;  // padding ranks behind everything
     __syncthreads();
@@ -653,14 +693,21 @@ __global__ __launch_bounds__(256) void tile_order_kernel(const int* __restrict__
 }
 
 int launch_ds_entries(const uint8_t* fine, int64_t fine_sb, int64_t fine_ss, int B, int Sq, int Sk, int* entry,
-                      int64_t entry_sb, int* tile_base, int* count, int* tile_count, int* tile_order, hipStream_t stream) {
-    const int slots = 4 * ((Sq + BLOCK_M - 1) / BLOCK_M), nkt = (Sk + 127) / 128, num_n = (Sk + BLOCK_N - 1) / BLOCK_N;
-    const int n_tiles = nkt * B;
+                      int64_t entry_sb, int* tile_base, int* count, int* tile_count, int* tile_order, const int* order,
+                      int64_t order_sb, int* group_count, int* group_order, hipStream_t stream) {
+    const int num_m = (Sq + BLOCK_M - 1) / BLOCK_M;
+    const int slots = 4 * num_m, nkt = (Sk + 127) / 128, num_n = (Sk + BLOCK_N - 1) / BLOCK_N;
+    const int n_tiles = nkt * B, n_groups = num_m * B;
     if (n_tiles > DS_MAX_ORDERED_TILES || tile_count == nullptr) tile_order = nullptr;
-    hipLaunchKernelGGL(ds_entries_kernel, dim3(nkt, B), dim3(DS_NUM_THREADS), 0, stream, fine, fine_sb, fine_ss, slots, nkt,
-                       num_n, entry, entry_sb, tile_base, count, tile_order != nullptr ? tile_count : nullptr);
-    if (tile_order != nullptr)
-        hipLaunchKernelGGL(tile_order_kernel, dim3((n_tiles + 63) / 64), dim3(256), 0, stream, tile_count, n_tiles, tile_order);
+    if (n_groups > DS_MAX_ORDERED_TILES || group_count == nullptr || order == nullptr) group_order = nullptr;
+    hipLaunchKernelGGL(ds_entries_kernel, dim3(nkt + (group_order != nullptr ? num_m : 0), B), dim3(DS_NUM_THREADS), 0,
+                       stream, fine, fine_sb, fine_ss, slots, nkt, num_n, entry, entry_sb, tile_base, count,
+                       tile_order != nullptr ? tile_count : nullptr, order, order_sb, group_count);
+    if (tile_order != nullptr || group_order != nullptr) {
+        const int nt = tile_order != nullptr ? n_tiles : 0, ng = group_order != nullptr ? n_groups : 0;
+        hipLaunchKernelGGL(tile_order_kernel, dim3((max(nt, ng) + 63) / 64, group_order != nullptr ? 2 : 1), dim3(256), 0,
+                           stream, tile_count, nt, tile_order, group_count, ng, group_order);
+    }
     return (int)hipGetLastError();
 }
 

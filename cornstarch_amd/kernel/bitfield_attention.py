@@ -187,6 +187,17 @@ class _TilePlan:
                                 (st.order - ws.data_ptr()) // 4)
 
 
+    def group_order(self) -> Optional[torch.Tensor]:
+        """int32 (B * ceil(S/128),) view, or None (more than 1024 groups): the groups of four slices of
+        ``slice_order()``, as codes ``b * ceil(S/128) + group``, by falling number of 64-key tiles they visit -- the
+        order in which the forward / dQ kernels take their workgroups."""
+        st, ws = self.struct, self.workspace
+        if not st.group_order:
+            return None
+        return torch.as_strided(ws.view(torch.int32), (st.B * (-(-st.Sq // BLOCK_M)),), (1,),
+                                (st.group_order - ws.data_ptr()) // 4)
+
+
 def _plan_arg(plan: Optional["_TilePlan"]):
     return plan.byref() if plan is not None else None
 

@@ -119,6 +119,10 @@ typedef struct bam_plan {
     const int32_t* ds_tile_order; /* device, B * ceil(Sk/128) ints, or null (more than 1024 key tiles): the key tiles
                                      (code b * ceil(Sk/128) + t) by falling number of pairs, the order in which the
                                      dK/dV kernel takes its workgroups so that the longest start first */
+    const int32_t* group_order; /* device, B * ceil(Sq/128) ints, or null (more than 1024 groups): the groups of four
+                                   slices of `order` (code b * ceil(Sq/128) + group) by falling number of 64-key tiles
+                                   they visit, the order in which the forward and dQ kernels take their workgroups, so
+                                   that the longest start first whatever the sequences of a batch look like */
     void* ds_workspace;        /* device, at least bam_ds_workspace_bytes(Hq, pairs) bytes, 16-byte aligned */
     int64_t ds_capacity;       /* pairs the workspace has room for: at least *ds_count */
     /* Materialized masks only (bam_mask_tile_plan; null otherwise): the mask packed to bits, once per orientation, so

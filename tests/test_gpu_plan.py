@@ -106,6 +106,26 @@ def test_classes_when_the_bitfield_changes_every_few_rows(S, max_run):
         assert sorted(o[:n]) == list(range(n)) and all(x == -1 for x in o[n:])
 
 
+@pytest.mark.parametrize("B,S", [(1, 1000), (3, 700), (8, 4096), (5, 129)])
+def test_groups_of_slices_are_ranked_by_the_length_of_their_tile_lists(B, S):
+    # group_order: codes b * num_m + group of ALL sequences, by falling number of 64-key tiles the group's four
+    # slices visit together (ties: lower code first)
+    bf = random_bitfield(B, S, seed=7 * B + S, pad=S // 9)
+    _, fine, order, plan = build_plan(bf.to(dev()))
+    got = plan.group_order()
+    num_m, n64 = -(-S // 128), -(-S // 64)
+    assert got is not None and got.shape == (B * num_m,)
+    fine, order = fine.cpu(), order.cpu()
+    weight = []
+    for b in range(B):
+        cls = F.pad(fine[b], (0, 2 * n64 - fine.shape[2])).view(fine.shape[1], n64, 2).amax(dim=2) > 0
+        for grp in range(num_m):
+            rows = [int(s) for s in order[b, 4 * grp : 4 * grp + 4] if s >= 0]
+            weight.append(int(cls[rows].any(dim=0).sum()) if rows else 0)
+    want = sorted(range(B * num_m), key=lambda c: (-weight[c], c))
+    assert got.cpu().tolist() == want
+
+
 @pytest.mark.parametrize("name", ["C1", "C2", "C4"])
 def test_fine_classes_on_the_benchmark_workloads(name):
     bf = W.make_bitfields(name).to(dev())
