@@ -12,6 +12,7 @@ module (cornstarch/kernel/attention.py:51-52, cornstarch/shardformer/layers/util
 
 from __future__ import annotations
 
+import atexit
 import math
 from typing import Optional
 
@@ -96,6 +97,9 @@ class _MaskPlan:
     @classmethod
     def forget(cls):
         cls._last = None
+
+
+atexit.register(_MaskPlan.forget)  # (runs before the release of the bitfield module's state, registered earlier)
 
 
 def _checked_mask(mask, batch, seqlen_q, seqlen_k):

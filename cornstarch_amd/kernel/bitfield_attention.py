@@ -10,6 +10,7 @@ live on the GPU and the HIP library must be built.
 
 from __future__ import annotations
 
+import atexit
 import math
 import os
 from typing import Optional
@@ -108,6 +109,24 @@ class _PinnedInts:
         if key not in cls._streams:
             cls._streams[key] = torch.cuda.Stream(device=device)
         return cls._streams[key]
+
+
+def _release_device_state() -> None:
+    """Drops what this module keeps alive between calls (cached flags and plans, the pinned counter slots, the side
+    stream) while the GPU runtime is still up: left to interpreter shutdown, pinned memory and streams would be
+    released in no particular order after it."""
+    try:
+        if torch.cuda.is_available() and torch.cuda.is_initialized():
+            torch.cuda.synchronize()
+    except Exception:  # the runtime is already gone: nothing left to wait for
+        pass
+    BitfieldUtils.clear_cache()
+    _IndexView.forget()
+    _PinnedInts._buf = None
+    _PinnedInts._streams.clear()
+
+
+atexit.register(_release_device_state)
 
 
 class _TilePlan:
