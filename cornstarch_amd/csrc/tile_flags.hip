@@ -552,15 +552,100 @@ __global__ __launch_bounds__(256) void mask_tile_plan_kernel(const uint8_t* __re
     }
 }
 
+// The same for masks whose rows are 4-byte aligned (Sk a multiple of four): a lane takes FOUR key columns and reads
+// them as one word per row, a wave takes one 32-row slice, so a workgroup reads 1 KiB per load instruction instead of
+// 256 bytes.  The bytes are reduced to one bit each in the word; the four column words of the lane collect them row
+// by row, the row word of a 32-key block is the OR of the nibbles of its eight lanes (DPP), staged in LDS and stored
+// as runs of 32 rows.
+__device__ __forceinline__ unsigned oct_or(unsigned x) {  // OR over groups of eight lanes, result in every lane
+    x |= (unsigned)__builtin_amdgcn_mov_dpp((int)x, 0xB1, 0xF, 0xF, false);   // quad_perm [1,0,3,2]
+    x |= (unsigned)__builtin_amdgcn_mov_dpp((int)x, 0x4E, 0xF, 0xF, false);   // quad_perm [2,3,0,1]
+    x |= (unsigned)__builtin_amdgcn_mov_dpp((int)x, 0x141, 0xF, 0xF, false);  // row_half_mirror
+    return x;
+}
+__global__ __launch_bounds__(256) void mask_tile_plan_words_kernel(
+    const uint8_t* __restrict__ mask, int8_t* __restrict__ flags, int64_t flags_stride_b, int64_t flags_stride_m, int Sq,
+    int Sk, int num_n, uint8_t* __restrict__ fine, int64_t fine_sb, int64_t fine_ss, int* __restrict__ order,
+    int64_t order_sb, int* __restrict__ pair_count, unsigned* __restrict__ row_bits, int64_t row_bits_sb,
+    int64_t row_bits_sn, unsigned* __restrict__ col_bits, int64_t col_bits_sb, int64_t col_bits_ss) {
+    __shared__ unsigned s_rows[4][8][32];  // [slice][32-key block][row]: row words of this workgroup
+    __shared__ int s_cnt[4][8];
+    const int b = blockIdx.z, m = blockIdx.y, tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+    if (pair_count != nullptr && blockIdx.x == 0 && m == 0 && b == 0 && tid == 0) *pair_count = 0;
+    if (blockIdx.x == 0 && tid < 4) {
+        const int ns = (Sq + 31) / 32, slot = 4 * m + tid;
+        order[(int64_t)b * order_sb + slot] = slot < ns ? ns - 1 - slot : -1;
+    }
+    const int col0 = blockIdx.x * 256 + 4 * lane;  // first of this lane's four columns (all inside or all outside)
+    const int ra = m * BLOCK_M + 32 * w;           // first row of this wave's slice
+    const int nb = lane >> 3, n = blockIdx.x * 8 + nb;
+    const int num_n_bits = (num_n + 1) & ~1, sk_pad = ((Sk + 127) >> 7) << 7;
+    const uint8_t* prow = mask + ((int64_t)b * Sq + ra) * Sk + (col0 < Sk ? col0 : 0);
+    unsigned v[32];
+#pragma unroll
+    for (int r = 0; r < 32; ++r) v[r] = (col0 < Sk && ra + r < Sq) ? *(const unsigned*)(prow + (int64_t)r * Sk) : 0u;
+    unsigned cw[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int r = 0; r < 32; ++r) {
+        unsigned t = v[r] | (v[r] >> 4);  // any bit of a byte -> its bit 0
+        t |= t >> 2;
+        t |= t >> 1;
+        t &= 0x01010101u;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) cw[c] |= ((t >> (8 * c)) & 1u) << r;
+        const unsigned nib = (t | (t >> 7) | (t >> 14) | (t >> 21)) & 0xFu;  // the four bits side by side
+        const unsigned word = oct_or(nib << (4 * (lane & 7)));
+        if ((lane & 7) == 0) s_rows[w][nb][r] = word;
+    }
+    if (col0 < sk_pad) {
+        u32x4 out = {cw[0], cw[1], cw[2], cw[3]};
+        *(u32x4*)(col_bits + (int64_t)b * col_bits_sb + (int64_t)(4 * m + w) * col_bits_ss + col0) = out;
+    }
+    // this wave's row words: 8 blocks x 32 rows, each block a run of 32 consecutive words
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const int idx = 64 * k + lane, nb2 = idx >> 5, rr = idx & 31, n2 = blockIdx.x * 8 + nb2;
+        if (n2 < num_n_bits)
+            row_bits[(int64_t)b * row_bits_sb + (int64_t)n2 * row_bits_sn + ra + rr] = s_rows[w][nb2][rr];
+    }
+    int cnt = __popc(cw[0]) + __popc(cw[1]) + __popc(cw[2]) + __popc(cw[3]);
+    cnt += __shfl_xor(cnt, 1);
+    cnt += __shfl_xor(cnt, 2);
+    cnt += __shfl_xor(cnt, 4);
+    if ((lane & 7) == 0) {
+        s_cnt[w][nb] = cnt;
+        if (n < num_n) {
+            const int cols = min(BLOCK_N, Sk - n * BLOCK_N), rows = max(0, min(32, Sq - ra));
+            fine[(int64_t)b * fine_sb + (int64_t)(4 * m + w) * fine_ss + n] = (uint8_t)(cnt == 0 ? 0 : cnt == rows * cols ? 2 : 1);
+        }
+    }
+    __syncthreads();
+    if (tid < 8 && blockIdx.x * 8 + tid < num_n) {
+        const int nn = blockIdx.x * 8 + tid, cols = min(BLOCK_N, Sk - nn * BLOCK_N);
+        int total = 0, cells = 0;
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+            total += s_cnt[x][tid];
+            cells += max(0, min(32, Sq - (m * BLOCK_M + 32 * x))) * cols;
+        }
+        flags[(int64_t)b * flags_stride_b + (int64_t)m * flags_stride_m + nn] = total == 0 ? 0 : total == cells ? 2 : 1;
+    }
+}
+
 int launch_mask_tile_plan(const uint8_t* mask, int8_t* flags, int64_t flags_stride_b, int64_t flags_stride_m,
                           uint8_t* fine, int64_t fine_sb, int64_t fine_ss, int* order, int64_t order_sb, int* pair_count,
                           unsigned* row_bits, int64_t row_bits_sb, int64_t row_bits_sn, unsigned* col_bits,
                           int64_t col_bits_sb, int64_t col_bits_ss, int B, int Sq, int Sk, hipStream_t stream) {
     const int num_m = (Sq + BLOCK_M - 1) / BLOCK_M, num_n = (Sk + BLOCK_N - 1) / BLOCK_N;
     dim3 grid((num_n + 7) / 8, num_m, B);
-    hipLaunchKernelGGL(mask_tile_plan_kernel, grid, dim3(256), 0, stream, mask, flags, flags_stride_b, flags_stride_m, Sq,
-                       Sk, num_n, fine, fine_sb, fine_ss, order, order_sb, pair_count, row_bits, row_bits_sb, row_bits_sn,
-                       col_bits, col_bits_sb, col_bits_ss);
+    if (row_bits != nullptr && col_bits != nullptr && (Sk & 3) == 0 && (reinterpret_cast<uintptr_t>(mask) & 3u) == 0)
+        hipLaunchKernelGGL(mask_tile_plan_words_kernel, grid, dim3(256), 0, stream, mask, flags, flags_stride_b,
+                           flags_stride_m, Sq, Sk, num_n, fine, fine_sb, fine_ss, order, order_sb, pair_count, row_bits,
+                           row_bits_sb, row_bits_sn, col_bits, col_bits_sb, col_bits_ss);
+    else
+        hipLaunchKernelGGL(mask_tile_plan_kernel, grid, dim3(256), 0, stream, mask, flags, flags_stride_b, flags_stride_m,
+                           Sq, Sk, num_n, fine, fine_sb, fine_ss, order, order_sb, pair_count, row_bits, row_bits_sb,
+                           row_bits_sn, col_bits, col_bits_sb, col_bits_ss);
     return (int)hipGetLastError();
 }
 
