@@ -8,8 +8,9 @@
 // Work decomposition: as the forward -- a workgroup is four 32-row slices of one (batch, q head), one per wave (taken
 // from the plan's slice order), and walks the 64-key tiles any of them needs; K tiles are shared through LDS (double
 // buffered), every wave copies its own dS blocks (two 2 KiB blocks per tile, one per 32-key half) into a wave-private
-// LDS area, two tiles ahead: a buffer is refilled as soon as its operands are in registers.  Both MFMA operands come from transposing LDS reads: K^T (d x keys) from the row-major K tile, dS^T
-// (keys x rows) from the block, which the dK/dV lanes wrote key by key.
+// LDS area, two tiles ahead: a buffer is refilled as soon as its operands are in registers.  Both MFMA operands come
+// from transposing LDS reads: K^T (d x keys) from the row-major K tile, dS^T (keys x rows) from the block, which the
+// dK/dV lanes wrote key by key.
 #pragma once
 #include "bam_common.h"
 #include "bam_launch.h"
