@@ -260,6 +260,28 @@ __device__ __forceinline__ void sched_pipeline_mfma_lds() {
     for (int i = 0; i < AHEAD; ++i) __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
 }
 
+// x as the sum of three values of the 16-bit type (for bf16: x to its full fp32 precision), packed into the first three
+// of a lane's eight k-slots of an MFMA operand; the other slots are zero.  Multiplied by ones in the same slots of the
+// other operand, an MFMA adds x to a whole row or column of its accumulator.  An infinite x stays infinite (one slot).
+template <typename T>
+__device__ __forceinline__ u32x4 split3_operand(float x) {
+    const unsigned h = T::pack2(x, 0.f) & 0xFFFFu;
+    const float fh = T::to_float((unsigned short)h);
+    const float r1 = fabsf(fh) < INFINITY ? x - fh : 0.f;  // exact
+    const unsigned l = T::pack2(r1, 0.f) & 0xFFFFu;
+    const float r2 = r1 - T::to_float((unsigned short)l);
+    const unsigned l2 = T::pack2(r2, 0.f) & 0xFFFFu;
+    u32x4 r = {h | (l << 16), l2, 0u, 0u};
+    return r;
+}
+// The matching operand of ones (1.0 in the 16-bit type, three slots).
+template <typename T>
+__device__ __forceinline__ u32x4 ones3_operand() {
+    const unsigned one = T::pack2(1.f, 0.f) & 0xFFFFu;
+    u32x4 r = {one | (one << 16), one, 0u, 0u};
+    return r;
+}
+
 // Workgroups are dealt round-robin to the 8 XCDs.  Map a linear block id onto
 // (unit, member) so that the `G` members of one unit land on the same XCD back to back
 // (they share K/V through that XCD's L2) while consecutive units spread over all XCDs.

@@ -101,7 +101,15 @@ __global__ __launch_bounds__(FWD_THREADS, D == 128 ? 2 : 3) void fwd_kernel(cons
     float m_i = -INFINITY, l_i = 0.f, nb = 0.f;  // nb = -m_i * c2 (0 while m_i is -inf)
     // with a bias the scores are turned into scale * s + bias right after the S phase, and only log2(e) is left
     // to fold into the exponent
-    const float c2 = BIAS ? LOG2E : p.scale * LOG2E;
+    // A per-key bias whose groups of four keys are aligned, in-range accesses travels with the tile copies: 64 values
+    // per tile, one word per lane (16-bit elements: lanes 32..63 repeat lanes 0..31).
+    const bool bias_lds = BIAS && p.bias_sm == 0 && p.bias_vec != 0;
+    // ... and with bf16 operands it is added by the matrix cores: bias / scale, split into three bf16 values, rides in
+    // one more MFMA of the S phase against an operand of ones, so that the scores come out as q.k + bias / scale and
+    // the exponent is taken exactly as without a bias (no multiply-add per score, no bias reads per score).
+    const bool bias_fold = bias_lds && std::is_same<T, BF16>::value;
+    const float c2 = (BIAS && !bias_fold) ? LOG2E : p.scale * LOG2E;
+    const float inv_scale = 1.f / p.scale;
     const char* bias_row = nullptr;  // this lane's row of the bias
     if (BIAS)
         bias_row = (const char*)p.bias + (p.bias_f32 ? 4 : 2) * ((int64_t)b * p.bias_sb + (int64_t)h * p.bias_sh +
@@ -127,9 +135,6 @@ __global__ __launch_bounds__(FWD_THREADS, D == 128 ? 2 : 3) void fwd_kernel(cons
     stV.setup(2 * p.v.ss, tid);
     const unsigned ldsK = lds_addr(sK), ldsV = lds_addr(sV), ldsB = lds_addr(sKbf), ldsP = lds_addr(sKpos);
     const unsigned ldsR = lds_addr(sRowBits);
-    // A per-key bias whose groups of four keys are aligned, in-range accesses travels with the tile copies: 64 values
-    // per tile, one word per lane (16-bit elements: lanes 32..63 repeat lanes 0..31).
-    const bool bias_lds = BIAS && p.bias_sm == 0 && p.bias_vec != 0;
     const char* bias_head = BIAS ? (const char*)p.bias + (p.bias_f32 ? 4 : 2) * ((int64_t)b * p.bias_sb + (int64_t)h * p.bias_sh) : nullptr;
     const unsigned bias_voff = (unsigned)((p.bias_f32 ? lane : (lane & 31)) * 4);
     const int bias_tile_bytes = FWD_KT * (p.bias_f32 ? 4 : 2);
@@ -184,6 +189,16 @@ __global__ __launch_bounds__(FWD_THREADS, D == 128 ? 2 : 3) void fwd_kernel(cons
         // (the MFMA phases run at raised wave priority: when the SIMD's other wave is in its softmax phase, this
         // wave's next MFMA is picked first and the MFMA pipe does not idle behind a queue of VALU instructions)
         f32x16 s[2];
+        u32x4 bias_a[2];  // bias_fold: this lane's key of either 32-key block, as an operand (keys are the rows of S^T)
+        if (BIAS && PREFETCH && bias_fold) {
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb) {
+                const float bv = p.bias_f32 ? ((const float*)sBias[cur])[32 * kb + l32]
+                                            : T::to_float(((const unsigned short*)sBias[cur])[32 * kb + l32]);
+                const u32x4 z = {0u, 0u, 0u, 0u};
+                bias_a[kb] = hi == 0 ? split3_operand<T>(bv * inv_scale) : z;
+            }
+        }
         __builtin_amdgcn_s_setprio(1);
         {
             constexpr int NOP = 2 * KK, AHEAD = 4;
@@ -202,11 +217,19 @@ __global__ __launch_bounds__(FWD_THREADS, D == 128 ? 2 : 3) void fwd_kernel(cons
 #pragma unroll
                 for (int j = NOP; j < NLOADS; ++j) issue_copy(j, kt_next, cur ^ 1);
             }
+            if (BIAS && PREFETCH && bias_fold) {
+                const u32x4 z = {0u, 0u, 0u, 0u};
+                const u32x4 ones = hi == 0 ? ones3_operand<T>() : z;
+                s[0] = T::mfma(bias_a[0], ones, s[0]);
+                s[1] = T::mfma(bias_a[1], ones, s[1]);
+            }
             __builtin_amdgcn_sched_barrier(0);
         }
         __builtin_amdgcn_s_setprio(0);
 
-        if (BIAS && PREFETCH && bias_lds) {  // (the ragged last tile is staged without the bias)
+        if (BIAS && PREFETCH && bias_fold) {
+            // (added by the MFMA above)
+        } else if (BIAS && PREFETCH && bias_lds) {  // (the ragged last tile is staged without the bias)
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
@@ -232,7 +255,9 @@ __global__ __launch_bounds__(FWD_THREADS, D == 128 ? 2 : 3) void fwd_kernel(cons
                 for (int grp = 0; grp < 4; ++grp) {
                     const f32x4 b4 = load_bias4<T>(bias_row, kt * FWD_KT + 32 * kb + 8 * grp + 4 * hi, Sk, p.bias_f32 != 0, p.bias_vec != 0);
 #pragma unroll
-                    for (int x = 0; x < 4; ++x) s[kb][4 * grp + x] = fmaf(s[kb][4 * grp + x], p.scale, b4[x]);
+                    for (int x = 0; x < 4; ++x)
+                        s[kb][4 * grp + x] = bias_fold ? fmaf(b4[x], inv_scale, s[kb][4 * grp + x])  // (c2 holds the scale)
+                                                       : fmaf(s[kb][4 * grp + x], p.scale, b4[x]);
                 }
         }
 
