@@ -192,6 +192,33 @@ def test_results_do_not_depend_on_the_plan(B, S, Hq, Hkv, D):
     BA.BitfieldUtils.clear_cache()
 
 
+def test_batches_with_more_than_1024_groups_or_key_tiles_run_without_the_rankings():
+    # 1100 sequences of 130 rows: 2200 groups of slices and 2200 key tiles, more than the rankings cover; the kernels
+    # then walk them in their natural order and the results are what they are without a plan
+    d = dev()
+    B, S, Hq, Hkv, D = 1100, 130, 2, 1, 32
+    bf = random_bitfield(B, S, seed=5, pad=3).to(d)
+    g = torch.Generator().manual_seed(5)
+    q = (torch.randn(B, S, Hq, D, generator=g) * 0.5).bfloat16().to(d)
+    k = (torch.randn(B, S, Hkv, D, generator=g) * 0.5).bfloat16().to(d)
+    v = (torch.randn(B, S, Hkv, D, generator=g) * 0.5).bfloat16().to(d)
+    do = torch.randn(B, S, Hq, D, generator=g).bfloat16().to(d)
+    flags, _, _, plan = build_plan(bf)
+    assert plan.group_order() is None and not plan.struct.ds_tile_order
+    scale = 1.0 / math.sqrt(D)
+    with_plan = _run(q, k, v, do, bf, flags, plan, scale)
+    without = _run(q, k, v, do, bf, flags, None, scale)
+    for name, a, b in zip(("o", "lse", "dq", "dk", "dv"), with_plan, without):
+        if name in ("dk", "dv"):
+            assert rel_l2(a.float(), b.float()) <= 2e-3, name
+        else:
+            assert torch.equal(a, b), name
+    sub = slice(0, 16)  # the oracle on a few of the sequences
+    o_ref, _ = O.attention_forward(q[sub], k[sub], v[sub], bf[sub])
+    assert (with_plan[0][sub].float() - o_ref).abs().max().item() <= 2e-2
+    BA.BitfieldUtils.clear_cache()
+
+
 def test_a_plan_of_another_problem_is_refused():
     d = dev()
     bf = random_bitfield(1, 256, seed=1).to(d)
