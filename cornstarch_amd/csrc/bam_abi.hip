@@ -397,8 +397,8 @@ int place_plan(const char* who, void* workspace, int64_t workspace_bytes, int B,
     plan->ds_entry_stride_b = l.entry_sb;
     plan->ds_tile_base = (const int32_t*)(w + l.base_off);
     plan->ds_count = (const int32_t*)(w + l.count_off);
-    plan->ds_tile_order = (int64_t)B * ((Sk + 127) / 128) <= 1024 ? (const int32_t*)(w + l.tile_order_off) : nullptr;
-    plan->group_order = (int64_t)B * ((Sq + 127) / 128) <= 1024 ? (const int32_t*)(w + l.group_order_off) : nullptr;
+    plan->ds_tile_order = (int64_t)B * ((Sk + 127) / 128) <= bam::MAX_RANKED ? (const int32_t*)(w + l.tile_order_off) : nullptr;
+    plan->group_order = (int64_t)B * ((Sq + 127) / 128) <= bam::MAX_RANKED ? (const int32_t*)(w + l.group_order_off) : nullptr;
     plan->ds_workspace = nullptr;
     plan->ds_capacity = 0;
     plan->row_bits = with_bits ? (const uint32_t*)(w + l.row_off) : nullptr;

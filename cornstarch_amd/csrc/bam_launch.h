@@ -13,6 +13,7 @@ constexpr int MASK_DENSE = 2;     // a materialized bool mask (B, Sq, Sk), one b
 // A workgroup lists its 64-key tiles (forward, dQ) or its 32-row slices (dK/dV) in LDS, this many at a time;
 // sequences beyond 131072 tokens take several passes.
 constexpr int MAX_LIST = 2048;         // 64-key tiles per pass
+constexpr int MAX_RANKED = 8192;       // key tiles / groups of slices of a batch that the plan ranks by their work
 constexpr int MAX_SLICE_LIST = 4096;   // 32-row slices per pass
 // Longest sequence the entry points accept (tile numbers are packed with eight class bits into 32-bit list entries,
 // positions are 32-bit; the bound leaves a wide margin to both).
@@ -132,7 +133,7 @@ int launch_mask_tile_plan(const uint8_t* mask, int8_t* flags, int64_t flags_stri
 // tile_base (B, ceil(Sk/128)) ints: number of the first pair of each key tile (pairs are numbered tile by tile).
 // *count must be zero when the kernel starts (the plan kernels reset it).  tile_count (B, ceil(Sk/128)) scratch and
 // tile_order (B * ceil(Sk/128)): the key tiles by falling number of pairs, written by a second small launch; both may
-// be null, and no order is written beyond 1024 tiles.  The same for the groups of four slices in the plan's slice
+// be null, and no order is written beyond MAX_RANKED tiles.  The same for the groups of four slices in the plan's slice
 // order (order, order_sb): group_count (B * num_m) scratch, group_order (B * num_m) = the groups by falling number of
 // 64-key tiles they visit.
 int launch_ds_entries(const uint8_t* fine, int64_t fine_sb, int64_t fine_ss, int B, int Sq, int Sk, int* entry,

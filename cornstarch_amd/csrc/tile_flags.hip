@@ -660,7 +660,7 @@ int launch_mask_tile_plan(const uint8_t* mask, int8_t* flags, int64_t flags_stri
 // tile_count[b][t] (optional) = number of pairs of key tile (b, t): what tile_order_kernel ranks the tiles by.
 // One workgroup per (key tile, batch); thread = slice, 256 slices per sweep.
 constexpr int DS_NUM_THREADS = 256;
-constexpr int DS_MAX_ORDERED_TILES = 1024;
+constexpr int DS_MAX_ORDERED_TILES = MAX_RANKED;  // counts staged in LDS: 32 KiB
 __global__ __launch_bounds__(DS_NUM_THREADS) void ds_entries_kernel(const uint8_t* __restrict__ fine, int64_t fine_sb,
                                                                    int64_t fine_ss, int slots, int nkt, int num_n,
                                                                    int* __restrict__ entry, int64_t entry_sb,

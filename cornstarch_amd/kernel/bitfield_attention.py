@@ -207,7 +207,7 @@ class _TilePlan:
 
 
     def group_order(self) -> Optional[torch.Tensor]:
-        """int32 (B * ceil(S/128),) view, or None (more than 1024 groups): the groups of four slices of
+        """int32 (B * ceil(S/128),) view, or None (more than 8192 groups): the groups of four slices of
         ``slice_order()``, as codes ``b * ceil(S/128) + group``, by falling number of 64-key tiles they visit -- the
         order in which the forward / dQ kernels take their workgroups."""
         st, ws = self.struct, self.workspace

@@ -116,10 +116,10 @@ typedef struct bam_plan {
     int64_t ds_entry_stride_b;
     const int32_t* ds_tile_base; /* device, (B, ceil(Sk/128)): number of the first pair of each key tile */
     const int32_t* ds_count;   /* device, one int: how many such pairs there are */
-    const int32_t* ds_tile_order; /* device, B * ceil(Sk/128) ints, or null (more than 1024 key tiles): the key tiles
+    const int32_t* ds_tile_order; /* device, B * ceil(Sk/128) ints, or null (more than 8192 key tiles): the key tiles
                                      (code b * ceil(Sk/128) + t) by falling number of pairs, the order in which the
                                      dK/dV kernel takes its workgroups so that the longest start first */
-    const int32_t* group_order; /* device, B * ceil(Sq/128) ints, or null (more than 1024 groups): the groups of four
+    const int32_t* group_order; /* device, B * ceil(Sq/128) ints, or null (more than 8192 groups): the groups of four
                                    slices of `order` (code b * ceil(Sq/128) + group) by falling number of 64-key tiles
                                    they visit, the order in which the forward and dQ kernels take their workgroups, so
                                    that the longest start first whatever the sequences of a batch look like */

@@ -106,7 +106,7 @@ def test_classes_when_the_bitfield_changes_every_few_rows(S, max_run):
         assert sorted(o[:n]) == list(range(n)) and all(x == -1 for x in o[n:])
 
 
-@pytest.mark.parametrize("B,S", [(1, 1000), (3, 700), (8, 4096), (5, 129)])
+@pytest.mark.parametrize("B,S", [(1, 1000), (3, 700), (8, 4096), (5, 129), (700, 300)])  # up to 2100 groups / tiles
 def test_groups_of_slices_are_ranked_by_the_length_of_their_tile_lists(B, S):
     # group_order: codes b * num_m + group of ALL sequences, by falling number of 64-key tiles the group's four
     # slices visit together (ties: lower code first)
@@ -124,6 +124,13 @@ def test_groups_of_slices_are_ranked_by_the_length_of_their_tile_lists(B, S):
             weight.append(int(cls[rows].any(dim=0).sum()) if rows else 0)
     want = sorted(range(B * num_m), key=lambda c: (-weight[c], c))
     assert got.cpu().tolist() == want
+    # the key tiles of the same plan, ranked by the number of slices that list them (what dK/dV goes by)
+    nkt = -(-S // 128)
+    has = (F.pad(fine, (0, 4 * nkt - fine.shape[2])).view(B, fine.shape[1], nkt, 4) != 0).any(dim=3)
+    counts = has.sum(dim=1).reshape(-1).tolist()
+    st, ws = plan.struct, plan.workspace
+    tile_order = torch.as_strided(ws.view(torch.int32), (B * nkt,), (1,), (st.ds_tile_order - ws.data_ptr()) // 4)
+    assert tile_order.cpu().tolist() == sorted(range(B * nkt), key=lambda c: (-counts[c], c))
 
 
 @pytest.mark.parametrize("name", ["C1", "C2", "C4"])
@@ -192,11 +199,11 @@ def test_results_do_not_depend_on_the_plan(B, S, Hq, Hkv, D):
     BA.BitfieldUtils.clear_cache()
 
 
-def test_batches_with_more_than_1024_groups_or_key_tiles_run_without_the_rankings():
-    # 1100 sequences of 130 rows: 2200 groups of slices and 2200 key tiles, more than the rankings cover; the kernels
-    # then walk them in their natural order and the results are what they are without a plan
+def test_batches_with_more_groups_or_key_tiles_than_are_ranked_run_without_the_rankings():
+    # 4200 sequences of 130 rows: 8400 groups of slices and 8400 key tiles, more than the rankings cover (8192); the
+    # kernels then walk them in their natural order and the results are what they are without a plan
     d = dev()
-    B, S, Hq, Hkv, D = 1100, 130, 2, 1, 32
+    B, S, Hq, Hkv, D = 4200, 130, 2, 1, 32
     bf = random_bitfield(B, S, seed=5, pad=3).to(d)
     g = torch.Generator().manual_seed(5)
     q = (torch.randn(B, S, Hq, D, generator=g) * 0.5).bfloat16().to(d)
