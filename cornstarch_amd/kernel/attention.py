@@ -13,6 +13,7 @@ module (cornstarch/kernel/attention.py:51-52, cornstarch/shardformer/layers/util
 from __future__ import annotations
 
 import atexit
+import contextlib
 import math
 from typing import Optional
 
@@ -21,6 +22,7 @@ import torch.nn.functional as F
 
 from . import _bam_hip
 from .bitfield_attention import (
+    _CACHE_LOCK,
     _bias_arg,
     _BiasView,
     _plan_arg,
@@ -67,6 +69,11 @@ class _MaskPlan:
         """-> (flags int8 (B, ceil(Sq/128), ceil(Sk/32)), plan or None)"""
         if mask is None:
             return mask_tile_flags(None, batch, seqlen_q, seqlen_k, device), None
+        with _CACHE_LOCK:
+            return cls._get_locked(mask, batch, seqlen_q, seqlen_k, device)
+
+    @classmethod
+    def _get_locked(cls, mask: torch.Tensor, batch: int, seqlen_q: int, seqlen_k: int, device):
         key = (mask.data_ptr(), tuple(mask.shape), tuple(mask.stride()), mask._version, mask.device)
         if cls._last is not None and cls._last[0] == key:
             return cls._last[1], cls._last[2]
@@ -203,8 +210,8 @@ def _flash_attn_backward(
     _launch_bwd_preprocess(ok, gk, delta)
     mask_ptr = mask.data_ptr() if mask is not None else None
     wq, wk, wv = work
-    ds_ws = plan.attach_ds_workspace(nheads, dp, seqlen_k) if plan is not None else None  # noqa: F841 (kept alive)
-    with torch.cuda.device(q.device):
+    handover = plan.ds_handover(nheads, dp, seqlen_k) if plan is not None else contextlib.nullcontext()
+    with handover, torch.cuda.device(q.device):
         _bam_hip.call(
             "bam_bwd_dkdv_masked",
             qk.data_ptr(), kk.data_ptr(), vk.data_ptr(), gk.data_ptr(), lse.data_ptr(), delta.data_ptr(),
@@ -221,8 +228,6 @@ def _flash_attn_backward(
             batch, seqlen_q, seqlen_k, nheads, nheads_k, dp, float(softmax_scale), _dtype_code(q.dtype), 0,
             _bias_arg(bias_view), _plan_arg(plan), _stream_ptr(q.device),
         )
-    if plan is not None:
-        plan.detach_ds_workspace()
     if not direct:
         for dst, w in zip(outs, work):
             dst.copy_(w[..., :d])

@@ -11,8 +11,10 @@ live on the GPU and the HIP library must be built.
 from __future__ import annotations
 
 import atexit
+import contextlib
 import math
 import os
+import threading
 from typing import Optional
 
 import torch
@@ -111,6 +113,11 @@ class _PinnedInts:
         return cls._streams[key]
 
 
+# The caches below (flags + plan of the last bitfield mask, index view, mask plan) are per process, as in the
+# reference; host threads that share them take this lock while they look an entry up or replace it.
+_CACHE_LOCK = threading.RLock()
+
+
 def _release_device_state() -> None:
     """Drops what this module keeps alive between calls (cached flags and plans, the pinned counter slots, the side
     stream) while the GPU runtime is still up: left to interpreter shutdown, pinned memory and streams would be
@@ -141,6 +148,7 @@ class _TilePlan:
         # The number of (slice, 128-key tile) pairs that have work is device data; it sizes the dS workspace of the
         # backward.  Its copy to the host is enqueued here, right behind the kernels that compute it, and awaited
         # only when a backward asks for it -- by then it has long arrived.
+        self._lock = threading.Lock()  # held while a backward has its dS workspace named in the struct
         self._pairs: Optional[int] = None
         self._pairs_host = _PinnedInts.slot()
         count = torch.as_strided(workspace.view(torch.int32), (1,), (1,), (struct.ds_count - workspace.data_ptr()) // 4)
@@ -187,6 +195,18 @@ class _TilePlan:
     def detach_ds_workspace(self) -> None:
         self.struct.ds_workspace = None
         self.struct.ds_capacity = 0
+
+    @contextlib.contextmanager
+    def ds_handover(self, nheads: int, head_dim: int, seqlen_k: int):
+        """The launches of one backward: the dS workspace (if any) is attached on entry and detached on exit, and
+        other host threads that run a backward with the same plan wait meanwhile (the struct is shared; the
+        launches only enqueue work, so the wait is short)."""
+        with self._lock:
+            ws = self.attach_ds_workspace(nheads, head_dim, seqlen_k)
+            try:
+                yield ws
+            finally:
+                self.detach_ds_workspace()
 
     def byref(self):
         import ctypes
@@ -242,11 +262,12 @@ class BitfieldUtils:
 
     @classmethod
     def clear_cache(cls):
-        cls.compressed_mask_cache = None
-        cls._cache_key = None
-        cls._cache_owner = None
-        cls._plan = None
-        _IndexView.forget()
+        with _CACHE_LOCK:
+            cls.compressed_mask_cache = None
+            cls._cache_key = None
+            cls._cache_owner = None
+            cls._plan = None
+            _IndexView.forget()
 
     @classmethod
     def plan_for(cls, compressed_mask: torch.Tensor, bitfield_mask: torch.Tensor) -> Optional[_TilePlan]:
@@ -254,14 +275,15 @@ class BitfieldUtils:
         itself and ``bitfield_mask`` is still the (unchanged) mask they were computed from.  Callers that bring
         their own flags (re-indexed context-parallel shards, for instance) get None and the kernels work from
         the flags alone."""
-        plan = cls._plan
-        if plan is None or plan.flags is not cls.compressed_mask_cache:
+        with _CACHE_LOCK:
+            plan, cached, key = cls._plan, cls.compressed_mask_cache, cls._cache_key
+        if plan is None or plan.flags is not cached:
             return None
         # the cache keeps its flags tensor alive, so equal address and shape mean "that tensor" (autograd may hand
         # saved tensors back as new Python objects)
         if compressed_mask.data_ptr() != plan.flags.data_ptr() or compressed_mask.shape != plan.flags.shape:
             return None
-        if cls._cache_key != cls._key_of(bitfield_mask):
+        if key != cls._key_of(bitfield_mask):
             return None
         return plan
 
@@ -277,6 +299,11 @@ class BitfieldUtils:
 
     @classmethod
     def materialize_compressed_mask_from_bitfield_mask(cls, bitfield_mask: torch.Tensor) -> torch.Tensor:
+        with _CACHE_LOCK:
+            return cls._materialize_locked(bitfield_mask)
+
+    @classmethod
+    def _materialize_locked(cls, bitfield_mask: torch.Tensor) -> torch.Tensor:
         key = cls._key_of(bitfield_mask)
         if cls.compressed_mask_cache is not None and cls._cache_key == key:
             # _cache_owner is alive, so this address still belongs to the tensor (or a view of the
@@ -439,11 +466,12 @@ class _IndexView:
         if offsets_q is None or offsets_k is None:
             raise ValueError("offsets_q and offsets_k must be given together")
         key = tuple(cls._tensor_key(t) for t in (bitfield_mask, offsets_q, offsets_k))
-        if cls._last is not None and cls._last[0] == key:
-            return cls._last[1]
-        view = cls(bitfield_mask, offsets_q, offsets_k)
-        cls._last = (key, view, (bitfield_mask, offsets_q, offsets_k))
-        return view
+        with _CACHE_LOCK:
+            if cls._last is not None and cls._last[0] == key:
+                return cls._last[1]
+            view = cls(bitfield_mask, offsets_q, offsets_k)
+            cls._last = (key, view, (bitfield_mask, offsets_q, offsets_k))
+            return view
 
     @classmethod
     def forget(cls):
@@ -613,13 +641,9 @@ def _bitfield_attn_backward_overwrite(do, q, k, v, o, bitfield_mask, compressed_
     batch, seqlen_q, nheads, _ = q.shape
     bias_view = _BiasView(bias, q, batch, nheads, seqlen_q, k.shape[1], may_copy=False) if bias is not None else None
     _launch_bwd_preprocess(o, do, delta)
-    ds_ws = plan.attach_ds_workspace(nheads, d, k.shape[1]) if plan is not None else None  # noqa: F841 (kept alive)
-    try:
+    with plan.ds_handover(nheads, d, k.shape[1]) if plan is not None else contextlib.nullcontext():
         _launch_bwd_dkdv(q, k, v, do, lse, delta, dk, dv, bf, flags, softmax_scale, accumulate=False, bias=bias_view, plan=plan)
         _launch_bwd_dq(q, k, v, do, lse, delta, dq, bf, flags, softmax_scale, accumulate=False, bias=bias_view, plan=plan)
-    finally:
-        if plan is not None:
-            plan.detach_ds_workspace()
     return dq, dk, dv
 
 
@@ -681,13 +705,9 @@ def _bitfield_attn_backward(
     wq, wk, wv = work
     _launch_bwd_preprocess(ok, gk, delta)
     the_plan = plan if view is None else view.plan
-    ds_ws = the_plan.attach_ds_workspace(nheads, dp, seqlen_k) if the_plan is not None else None  # noqa: F841
-    try:
+    with the_plan.ds_handover(nheads, dp, seqlen_k) if the_plan is not None else contextlib.nullcontext():
         _launch_bwd_dkdv(qk, kk, vk, gk, lse, delta, wk, wv, bf, flags, softmax_scale, bias=bias_view, plan=plan)
         _launch_bwd_dq(qk, kk, vk, gk, lse, delta, wq, bf, flags, softmax_scale, bias=bias_view, plan=plan)
-    finally:
-        if the_plan is not None:
-            the_plan.detach_ds_workspace()
     # the kernels accumulated into `work`; hand the sums back if those were copies
     for dst, mid, w in zip((dq, dk, dv), acc, work):
         if dp != d:
