@@ -378,9 +378,10 @@ __global__ __launch_bounds__(DKDV_THREADS, 2) void bwd_dkdv_kernel(const AttnPar
         }
         if (DENSE) {
             if (cls == 1 && col_bits_on) {
-                const unsigned w = sColBits[cur][st][32 * kg + l32];
+                // (shifted by this lane's first row, 4 hi, once: the bit numbers tested are then constants)
+                const unsigned w = sColBits[cur][st][32 * kg + l32] >> (4 * hi);
 #pragma unroll
-                for (int i = 0; i < 16; ++i) s[i] = ((w >> (8 * (i >> 2) + 4 * hi + (i & 3))) & 1u) ? s[i] : 0.f;
+                for (int i = 0; i < 16; ++i) s[i] = ((w >> (8 * (i >> 2) + (i & 3))) & 1u) ? s[i] : 0.f;
             } else if (cls == 1) {
                 // mask bytes of this lane's key column, one per row of the C fragment
                 const uint8_t* mcol = p.mask + ((int64_t)b * Sq + myrow0) * Sk + key;
@@ -826,7 +827,9 @@ __global__ __launch_bounds__(DQ_THREADS, D == 128 ? 2 : 3) void bwd_dq_kernel(co
                 uniform &= rel0 == kt0;
             }
             uniform_keys = __all(uniform);
-            rel = allow_bits(qb, flo, fhi) ? qb.lim - kt0 : -1;  // last allowed key, relative to the tile
+            // last allowed key, relative to the first key this lane holds (4 hi): what it is compared with are then
+            // compile-time constants, which occupy no registers
+            rel = allow_bits(qb, flo, fhi) ? qb.lim - kt0 - 4 * hi : -1;
         }
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) {
@@ -865,9 +868,10 @@ __global__ __launch_bounds__(DQ_THREADS, D == 128 ? 2 : 3) void bwd_dq_kernel(co
             }
             if (DENSE) {
                 if (cls == 1 && row_bits_w != nullptr) {
-                    const unsigned w = sRowBits[cur][wave][32 * kb + l32];
+                    // (shifted by this lane's first key, 4 hi, once: the bit numbers tested are then constants)
+                    const unsigned w = sRowBits[cur][wave][32 * kb + l32] >> (4 * hi);
 #pragma unroll
-                    for (int i = 0; i < 16; ++i) dp[i] = ((w >> (8 * (i >> 2) + 4 * hi + (i & 3))) & 1u) ? dp[i] : 0.f;
+                    for (int i = 0; i < 16; ++i) dp[i] = ((w >> (8 * (i >> 2) + (i & 3))) & 1u) ? dp[i] : 0.f;
                 } else if (cls == 1) {
                     const int kt0 = kt * DQ_KT;
                     const uint8_t* mrow = p.mask + ((int64_t)b * Sq + (qvalid ? qrow : 0)) * Sk + kt0;
@@ -897,12 +901,10 @@ __global__ __launch_bounds__(DQ_THREADS, D == 128 ? 2 : 3) void bwd_dq_kernel(co
             } else if (cls == 1) {
                 if (uniform_keys) {
 #pragma unroll
-                    for (int i = 0; i < 16; ++i) {
-                        const int koff = 32 * kb + 8 * (i >> 2) + 4 * hi + (i & 3);
-                        dp[i] = (koff <= rel) ? dp[i] : 0.f;
-                    }
+                    for (int i = 0; i < 16; ++i) dp[i] = (32 * kb + 8 * (i >> 2) + (i & 3) <= rel) ? dp[i] : 0.f;
                 } else {
-                    const int kt0 = kt * DQ_KT;
+                    // natural positions: the row's limit relative to the first key this lane holds
+                    const int lim_rel = qb.lim - (kt * DQ_KT + 4 * hi);
 #pragma unroll
                     for (int grp = 0; grp < 4; ++grp) {
                         const int koff = 32 * kb + 8 * grp + 4 * hi;
@@ -910,15 +912,13 @@ __global__ __launch_bounds__(DQ_THREADS, D == 128 ? 2 : 3) void bwd_dq_kernel(co
                         const u32x4 k23 = *(const u32x4*)&sKbf[cur][koff + 2];  // lo2 hi2 lo3 hi3
                         const unsigned klo[4] = {k01[0], k01[2], k23[0], k23[2]};
                         const unsigned khi[4] = {k01[1], k01[3], k23[1], k23[3]};
-                        int kpos[4] = {kt0 + koff, kt0 + koff + 1, kt0 + koff + 2, kt0 + koff + 3};
-                        if (IDX) {
-                            const u32x4 kp = *(const u32x4*)&sKpos[cur][koff];
+                        u32x4 kp = {0u, 0u, 0u, 0u};
+                        if (IDX) kp = *(const u32x4*)&sKpos[cur][koff];
 #pragma unroll
-                            for (int x = 0; x < 4; ++x) kpos[x] = (int)kp[x];
+                        for (int x = 0; x < 4; ++x) {
+                            const bool pos_ok = IDX ? (int)kp[x] <= qb.lim : 32 * kb + 8 * grp + x <= lim_rel;
+                            dp[4 * grp + x] = (allow_bits(qb, klo[x], khi[x]) & pos_ok) ? dp[4 * grp + x] : 0.f;
                         }
-#pragma unroll
-                        for (int x = 0; x < 4; ++x)
-                            dp[4 * grp + x] = allow_pair(qb, klo[x], khi[x], kpos[x]) ? dp[4 * grp + x] : 0.f;
                     }
                 }
             }

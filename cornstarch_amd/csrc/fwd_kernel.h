@@ -264,14 +264,13 @@ __global__ __launch_bounds__(FWD_THREADS, D == 128 ? 2 : 3) void fwd_kernel(cons
         // ---- bitfield rule in registers (partial tiles only) ------------------------------
         if (DENSE) {
             if (cls == 1 && row_bits_w != nullptr) {
-                const unsigned w01[2] = {sRowBits[cur][wave][l32], sRowBits[cur][wave][32 + l32]};
+                // (shifted by this lane's first key, 4 hi, once: the bit numbers tested are then constants)
+                const unsigned w01[2] = {sRowBits[cur][wave][l32] >> (4 * hi), sRowBits[cur][wave][32 + l32] >> (4 * hi)};
 #pragma unroll
                 for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-                    for (int i = 0; i < 16; ++i) {
-                        const int bit = 8 * (i >> 2) + 4 * hi + (i & 3);
-                        s[kb][i] = ((w01[kb] >> bit) & 1u) ? s[kb][i] : -INFINITY;
-                    }
+                    for (int i = 0; i < 16; ++i)
+                        s[kb][i] = ((w01[kb] >> (8 * (i >> 2) + (i & 3))) & 1u) ? s[kb][i] : -INFINITY;
             } else if (cls == 1) {
                 // mask bytes of this lane's query row: 4 consecutive keys per C-fragment group
                 const int kt0 = kt * FWD_KT;
@@ -316,15 +315,18 @@ __global__ __launch_bounds__(FWD_THREADS, D == 128 ? 2 : 3) void fwd_kernel(cons
                 uniform &= rel0 == kt0;
             }
             if (__all(uniform)) {
-                const int rel = allow_bits(qb, flo, fhi) ? qb.lim - kt0 : -1;  // last allowed key, relative to the tile
+                // last allowed key, relative to the first key this lane holds (4 hi): what it is compared with are
+                // then compile-time constants, which occupy no registers
+                const int rel = allow_bits(qb, flo, fhi) ? qb.lim - kt0 - 4 * hi : -1;
 #pragma unroll
                 for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-                    for (int i = 0; i < 16; ++i) {
-                        const int koff = 32 * kb + 8 * (i >> 2) + 4 * hi + (i & 3);
-                        s[kb][i] = (koff <= rel) ? s[kb][i] : -INFINITY;
-                    }
+                    for (int i = 0; i < 16; ++i)
+                        s[kb][i] = (32 * kb + 8 * (i >> 2) + (i & 3) <= rel) ? s[kb][i] : -INFINITY;
             } else {
+                // natural positions: the row's limit relative to the first key this lane holds, so that the position
+                // test compares with compile-time constants
+                const int lim_rel = qb.lim - (kt * FWD_KT + 4 * hi);
 #pragma unroll
                 for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
@@ -334,15 +336,12 @@ __global__ __launch_bounds__(FWD_THREADS, D == 128 ? 2 : 3) void fwd_kernel(cons
                         const u32x4 k23 = *(const u32x4*)&sKbf[cur][koff + 2];  // lo2 hi2 lo3 hi3
                         const unsigned klo[4] = {k01[0], k01[2], k23[0], k23[2]};
                         const unsigned khi[4] = {k01[1], k01[3], k23[1], k23[3]};
-                        int kpos[4] = {kt * FWD_KT + koff, kt * FWD_KT + koff + 1, kt * FWD_KT + koff + 2, kt * FWD_KT + koff + 3};
-                        if (IDX) {
-                            const u32x4 kp = *(const u32x4*)&sKpos[cur][koff];
-#pragma unroll
-                            for (int x = 0; x < 4; ++x) kpos[x] = (int)kp[x];
-                        }
+                        u32x4 kp = {0u, 0u, 0u, 0u};
+                        if (IDX) kp = *(const u32x4*)&sKpos[cur][koff];
 #pragma unroll
                         for (int x = 0; x < 4; ++x) {
-                            const bool a = allow_pair(qb, klo[x], khi[x], kpos[x]);
+                            const bool pos_ok = IDX ? (int)kp[x] <= qb.lim : 32 * kb + 8 * grp + x <= lim_rel;
+                            const bool a = allow_bits(qb, klo[x], khi[x]) & pos_ok;
                             s[kb][4 * grp + x] = a ? s[kb][4 * grp + x] : -INFINITY;
                         }
                     }
