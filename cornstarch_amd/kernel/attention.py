@@ -13,7 +13,6 @@ module (cornstarch/kernel/attention.py:51-52, cornstarch/shardformer/layers/util
 from __future__ import annotations
 
 import atexit
-import contextlib
 import math
 from typing import Optional
 
@@ -27,6 +26,7 @@ from .bitfield_attention import (
     _BiasView,
     _plan_arg,
     _TilePlan,
+    _backward_in_head_runs,
     _dtype_code,
     _is_kernel_ready,
     _kernel_ready,
@@ -210,24 +210,29 @@ def _flash_attn_backward(
     _launch_bwd_preprocess(ok, gk, delta)
     mask_ptr = mask.data_ptr() if mask is not None else None
     wq, wk, wv = work
-    handover = plan.ds_handover(nheads, dp, seqlen_k) if plan is not None else contextlib.nullcontext()
-    with handover, torch.cuda.device(q.device):
-        _bam_hip.call(
-            "bam_bwd_dkdv_masked",
-            qk.data_ptr(), kk.data_ptr(), vk.data_ptr(), gk.data_ptr(), lse.data_ptr(), delta.data_ptr(),
-            wk.data_ptr(), wv.data_ptr(), mask_ptr, flags.data_ptr(),
-            *_strides3(qk, kk, vk, gk, wk, wv), flags.stride(0), flags.stride(1),
-            batch, seqlen_q, seqlen_k, nheads, nheads_k, dp, float(softmax_scale), _dtype_code(q.dtype), 0,
-            _bias_arg(bias_view), _plan_arg(plan), _stream_ptr(q.device),
-        )
-        _bam_hip.call(
-            "bam_bwd_dq_masked",
-            qk.data_ptr(), kk.data_ptr(), vk.data_ptr(), gk.data_ptr(), lse.data_ptr(), delta.data_ptr(),
-            wq.data_ptr(), mask_ptr, flags.data_ptr(),
-            *_strides3(qk, kk, vk, gk, wq), flags.stride(0), flags.stride(1),
-            batch, seqlen_q, seqlen_k, nheads, nheads_k, dp, float(softmax_scale), _dtype_code(q.dtype), 0,
-            _bias_arg(bias_view), _plan_arg(plan), _stream_ptr(q.device),
-        )
+
+    def launch(q, k, v, do, lse, delta, dq, dk, dv):
+        heads, heads_k = q.shape[2], k.shape[2]
+        with torch.cuda.device(q.device):
+            _bam_hip.call(
+                "bam_bwd_dkdv_masked",
+                q.data_ptr(), k.data_ptr(), v.data_ptr(), do.data_ptr(), lse.data_ptr(), delta.data_ptr(),
+                dk.data_ptr(), dv.data_ptr(), mask_ptr, flags.data_ptr(),
+                *_strides3(q, k, v, do, dk, dv), flags.stride(0), flags.stride(1),
+                batch, seqlen_q, seqlen_k, heads, heads_k, dp, float(softmax_scale), _dtype_code(q.dtype), 0,
+                _bias_arg(bias_view), _plan_arg(plan), _stream_ptr(q.device),
+            )
+            _bam_hip.call(
+                "bam_bwd_dq_masked",
+                q.data_ptr(), k.data_ptr(), v.data_ptr(), do.data_ptr(), lse.data_ptr(), delta.data_ptr(),
+                dq.data_ptr(), mask_ptr, flags.data_ptr(),
+                *_strides3(q, k, v, do, dq), flags.stride(0), flags.stride(1),
+                batch, seqlen_q, seqlen_k, heads, heads_k, dp, float(softmax_scale), _dtype_code(q.dtype), 0,
+                _bias_arg(bias_view), _plan_arg(plan), _stream_ptr(q.device),
+            )
+
+    # (a bias is indexed by absolute head: with one, the heads stay in one run)
+    _backward_in_head_runs(plan, launch, qk, kk, vk, gk, lse, delta, wq, wk, wv, dp, splittable=bias_view is None)
     if not direct:
         for dst, w in zip(outs, work):
             dst.copy_(w[..., :d])

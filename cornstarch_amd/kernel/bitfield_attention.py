@@ -74,10 +74,20 @@ def materialize_bitfield_mask(bitfield_mask: torch.Tensor) -> torch.Tensor:
     return out.bool()
 
 
-# Largest dS workspace the backward allocates for the hand-over of dS from the dK/dV kernel to the dQ kernel; beyond it
-# the dQ kernel recomputes S and dP instead.  BAM_DS_WORKSPACE_LIMIT_GB overrides the default (a quarter of the
-# device's memory, at most 64 GiB); 0 switches the hand-over off.
+# Largest dS workspace the backward allocates for the hand-over of dS from the dK/dV kernel to the dQ kernel.  Where
+# the workspace for all heads would be larger, the backward takes the heads in runs of whole kv heads, one launch pair
+# per run through the same, smaller workspace; where even one kv head's q heads need more, the dQ kernel recomputes S
+# and dP instead.  BAM_DS_WORKSPACE_LIMIT_GB overrides the default (a quarter of the device's memory, at most
+# 64 GiB); 0 switches the hand-over off.
 _DS_LIMIT_ENV = os.environ.get("BAM_DS_WORKSPACE_LIMIT_GB")
+
+
+# Below the limit, a backward whose dS workspace for all heads would exceed this size still prefers runs of kv heads
+# as long as the dK/dV launch of a run keeps this many workgroups (128-key tiles x batch x kv heads of the run: four
+# rounds of the chip's 256 compute units).  One sequence of 65536 tokens with 32 q heads and 8 kv heads: 47 GiB in
+# one run, 12 GiB in four runs, the same 41.9 ms either way (and 46.6 ms in eight runs of one kv head each).
+_DS_RUN_TARGET = 16 << 30
+_DS_RUN_MIN_WORKGROUPS = 1024
 
 
 def _ds_workspace_limit(device) -> int:
@@ -187,6 +197,28 @@ class _TilePlan:
         self.struct.ds_workspace = ws.data_ptr()
         self.struct.ds_capacity = pairs
         return ws
+
+    def ds_head_runs(self, batch: int, nheads: int, nheads_k: int, head_dim: int, seqlen_k: int) -> int:
+        """Into how many runs of whole kv heads a backward splits: the smallest divisor of ``nheads_k`` for which the
+        dS workspace of one run stays within the limit, and beyond that more runs while a run's workspace is above
+        ``_DS_RUN_TARGET`` and its dK/dV launch keeps ``_DS_RUN_MIN_WORKGROUPS`` workgroups.  1: all heads at once
+        (also where the hand-over does not apply or no split helps: ``attach_ds_workspace`` then decides)."""
+        if head_dim != 128 or seqlen_k > 131072 or nheads % nheads_k != 0:
+            return 1
+        pairs = self.ds_pairs()
+        limit = _ds_workspace_limit(self.workspace.device)
+        lib = _bam_hip.load()
+        nbytes = {r: lib.bam_ds_workspace_bytes(nheads // r, pairs) for r in range(1, nheads_k + 1) if nheads_k % r == 0}
+        fits = [r for r, n in nbytes.items() if 0 < n <= limit and (nheads // r) * pairs < 1 << 31]
+        if not fits:
+            return 1
+        runs = fits[0]
+        key_tiles = batch * ((seqlen_k + 127) // 128)
+        for r in fits[1:]:
+            if nbytes[runs] <= _DS_RUN_TARGET or key_tiles * (nheads_k // r) < _DS_RUN_MIN_WORKGROUPS:
+                break
+            runs = r
+        return runs
 
     @staticmethod
     def _allocate(nbytes: int, device) -> torch.Tensor:
@@ -618,6 +650,28 @@ def _is_kernel_ready(x: torch.Tensor, elems_per_16b: int = 8) -> bool:
     return _kernel_ready(x, elems_per_16b) is x
 
 
+def _backward_in_head_runs(plan, launch, q, k, v, do, lse, delta, dq, dk, dv, head_dim, splittable=True):
+    """The dK/dV and dQ launches of a backward, ``launch(q, k, v, do, lse, delta, dq, dk, dv)``, under the plan's
+    dS hand-over.  When the dS workspace for all heads exceeds the limit, the heads are taken in runs of whole kv
+    heads (views of the tensors along the head dimension; lse and delta of a run are made contiguous), every run
+    through the same workspace: the launches of a stream run in order, so a run's dQ kernel has read the workspace
+    before the next run's dK/dV kernel writes it.  Per head the arithmetic is that of a single launch pair."""
+    if plan is None:
+        launch(q, k, v, do, lse, delta, dq, dk, dv)
+        return
+    nheads, nheads_k, seqlen_k = q.shape[2], k.shape[2], k.shape[1]
+    runs = plan.ds_head_runs(q.shape[0], nheads, nheads_k, head_dim, seqlen_k) if splittable else 1
+    hq, hk = nheads // runs, nheads_k // runs
+    with plan.ds_handover(hq, head_dim, seqlen_k):
+        if runs == 1:
+            launch(q, k, v, do, lse, delta, dq, dk, dv)
+            return
+        for r in range(runs):
+            qs, ks = slice(r * hq, (r + 1) * hq), slice(r * hk, (r + 1) * hk)
+            launch(q[:, :, qs], k[:, :, ks], v[:, :, ks], do[:, :, qs], lse[:, qs].contiguous(),
+                   delta[:, qs].contiguous(), dq[:, :, qs], dk[:, :, ks], dv[:, :, ks])
+
+
 def _bitfield_attn_backward_overwrite(do, q, k, v, o, bitfield_mask, compressed_mask, lse, softmax_scale, bias=None):
     """Gradients in the input dtype, written (not accumulated) by the kernels: what
     ``BitfieldAttentionFunction.backward`` needs, without the reference's zero-filled fp32
@@ -641,9 +695,13 @@ def _bitfield_attn_backward_overwrite(do, q, k, v, o, bitfield_mask, compressed_
     batch, seqlen_q, nheads, _ = q.shape
     bias_view = _BiasView(bias, q, batch, nheads, seqlen_q, k.shape[1], may_copy=False) if bias is not None else None
     _launch_bwd_preprocess(o, do, delta)
-    with plan.ds_handover(nheads, d, k.shape[1]) if plan is not None else contextlib.nullcontext():
+
+    def launch(q, k, v, do, lse, delta, dq, dk, dv):
         _launch_bwd_dkdv(q, k, v, do, lse, delta, dk, dv, bf, flags, softmax_scale, accumulate=False, bias=bias_view, plan=plan)
         _launch_bwd_dq(q, k, v, do, lse, delta, dq, bf, flags, softmax_scale, accumulate=False, bias=bias_view, plan=plan)
+
+    # (a bias is indexed by absolute head: with one, the heads stay in one run)
+    _backward_in_head_runs(plan, launch, q, k, v, do, lse, delta, dq, dk, dv, d, splittable=bias_view is None)
     return dq, dk, dv
 
 
@@ -705,9 +763,13 @@ def _bitfield_attn_backward(
     wq, wk, wv = work
     _launch_bwd_preprocess(ok, gk, delta)
     the_plan = plan if view is None else view.plan
-    with the_plan.ds_handover(nheads, dp, seqlen_k) if the_plan is not None else contextlib.nullcontext():
-        _launch_bwd_dkdv(qk, kk, vk, gk, lse, delta, wk, wv, bf, flags, softmax_scale, bias=bias_view, plan=plan)
-        _launch_bwd_dq(qk, kk, vk, gk, lse, delta, wq, bf, flags, softmax_scale, bias=bias_view, plan=plan)
+
+    def launch(q, k, v, do, lse, delta, dq, dk, dv):
+        _launch_bwd_dkdv(q, k, v, do, lse, delta, dk, dv, bf, flags, softmax_scale, bias=bias_view, plan=plan)
+        _launch_bwd_dq(q, k, v, do, lse, delta, dq, bf, flags, softmax_scale, bias=bias_view, plan=plan)
+
+    # (a bias is indexed by absolute head: with one, the heads stay in one run)
+    _backward_in_head_runs(the_plan, launch, qk, kk, vk, gk, lse, delta, wq, wk, wv, dp, splittable=bias_view is None)
     # the kernels accumulated into `work`; hand the sums back if those were copies
     for dst, mid, w in zip((dq, dk, dv), acc, work):
         if dp != d:

@@ -223,3 +223,103 @@ def test_a_workspace_that_cannot_be_allocated_means_recomputation(monkeypatch):
         assert rel_l2(a.float(), b.float()) <= 2e-3
         assert rel_l2(b.float().cpu(), w) <= GRAD_REL_L2
     BA.BitfieldUtils.clear_cache()
+
+
+@pytest.mark.parametrize("runs", [2, 4])
+@pytest.mark.parametrize("accumulate", [False, True], ids=["typed", "fp32"])
+def test_heads_in_runs_under_a_small_workspace_limit(runs, accumulate, monkeypatch):
+    # a limit that holds the dS of Hq / runs heads only: the backward takes the kv heads in `runs` runs through one
+    # workspace of that size, and every gradient comes out bit for bit as with one launch pair for all heads
+    from cornstarch_amd.kernel import _bam_hip
+
+    d = dev()
+    B, S, Hq, Hkv = 2, 640, 8, 4
+    bf = random_bitfield(B, S, seed=21, pad=6).to(d)
+    q, k, v, do = (t.to(d) for t in inputs(B, S, Hq, Hkv, 128, torch.bfloat16, seed=8))
+    whole = run_backward(q, k, v, do, bf, True, monkeypatch, accumulate)
+
+    flags, plan = build(bf)
+    limit = _bam_hip.load().bam_ds_workspace_bytes(Hq // runs, plan.ds_pairs())
+    monkeypatch.setattr(BA, "_ds_workspace_limit", lambda device: limit)
+    assert plan.ds_head_runs(B, Hq, Hkv, 128, S) == runs
+    assert plan.ds_head_runs(B, Hq, Hkv, 64, S) == 1  # no hand-over at head dim 64: nothing to split for
+    allocated = []
+    real = BA._TilePlan._allocate
+    monkeypatch.setattr(BA._TilePlan, "_allocate",
+                        staticmethod(lambda nbytes, device: allocated.append(nbytes) or real(nbytes, device)))
+    o, lse, scale = BA._bitfield_attn_forward(q, k, v, bf, flags)
+    if accumulate:
+        grads = [torch.zeros_like(t, dtype=torch.float32) for t in (q, k, v)]
+        BA._bitfield_attn_backward(do, q, k, v, o, bf, flags, lse, *grads, softmax_scale=scale)
+    else:
+        grads = BA._bitfield_attn_backward_overwrite(do, q, k, v, o, bf, flags, lse, scale)
+    torch.cuda.synchronize()
+    assert allocated == [limit] and plan.struct.ds_workspace is None
+    for got, want in zip(grads, whole):
+        assert torch.equal(got, want)
+    BA.BitfieldUtils.clear_cache()
+
+
+def test_heads_in_runs_with_index_tensors_and_dense_masks(monkeypatch):
+    d = dev()
+    B, S, Hq, Hkv = 1, 512, 4, 2
+    bf_cpu = random_bitfield(B, S, seed=5, pad=4)
+    q, k, v, do = inputs(B, S, Hq, Hkv, 128, torch.bfloat16, seed=2)
+    chunks = torch.arange(S).chunk(4)
+    idx_q = torch.cat([chunks[1], chunks[2]])
+    idx_k = torch.cat([chunks[1], chunks[2], chunks[0], chunks[3]])
+    flags = O.tile_flags_indexed(bf_cpu, idx_q, idx_k).to(d)
+    ql, dol = q[:, idx_q].contiguous().to(d), do[:, idx_q].contiguous().to(d)
+    kl, vl = k[:, idx_k].contiguous().to(d), v[:, idx_k].contiguous().to(d)
+    bfg, oq, ok = bf_cpu.to(d), idx_q.to(d), idx_k.to(d)
+    mask = O.materialize_mask(bf_cpu).to(d)
+    qd, kd, vd, dod = (t.to(d) for t in (q, k, v, do))
+    results = {}
+    for limit in (1 << 40, None):  # None: room for one kv head's q heads
+        if limit is None:
+            per_run = []
+            # the limit follows the plan in use: the dS of Hq / Hkv heads
+            monkeypatch.setattr(BA, "_ds_workspace_limit", lambda device: per_run[-1])
+            real_runs = BA._TilePlan.ds_head_runs
+
+            def runs_with_limit(self, batch, nheads, nheads_k, head_dim, seqlen_k):
+                from cornstarch_amd.kernel import _bam_hip
+                per_run.append(_bam_hip.load().bam_ds_workspace_bytes(nheads // nheads_k, self.ds_pairs()))
+                n = real_runs(self, batch, nheads, nheads_k, head_dim, seqlen_k)
+                assert n == nheads_k
+                return n
+
+            monkeypatch.setattr(BA._TilePlan, "ds_head_runs", runs_with_limit)
+        else:
+            monkeypatch.setattr(BA, "_ds_workspace_limit", lambda device: limit)
+        BA.BitfieldUtils.clear_cache()
+        A._MaskPlan.forget()
+        o, lse, scale = BA._bitfield_attn_forward(ql, kl, vl, bfg, flags, oq, ok)
+        g1 = [torch.zeros_like(t, dtype=torch.float32) for t in (ql, kl, vl)]
+        BA._bitfield_attn_backward(dol, ql, kl, vl, o, bfg, flags, lse, *g1, offsets_q=oq, offsets_k=ok, softmax_scale=scale)
+        o, lse, scale = A._flash_attn_forward(qd, kd, vd, mask=mask)
+        g2 = [torch.empty_like(t) for t in (qd, kd, vd)]
+        A._flash_attn_backward(dod, qd, kd, vd, o, lse, *g2, mask=mask, softmax_scale=scale)
+        torch.cuda.synchronize()
+        results[limit] = g1 + g2
+    for a, b in zip(results[1 << 40], results[None]):
+        assert torch.equal(a, b)
+    A._MaskPlan.forget()
+    BA.BitfieldUtils.clear_cache()
+
+
+def test_runs_of_heads_below_the_limit_when_the_workspace_is_large(monkeypatch):
+    # within the limit, a workspace above the preferred size is still split while a run keeps enough workgroups
+    d = dev()
+    B, S, Hq, Hkv = 2, 640, 16, 8
+    bf = random_bitfield(B, S, seed=2, pad=3).to(d)
+    flags, plan = build(bf)
+    key_tiles = B * 5
+    monkeypatch.setattr(BA, "_ds_workspace_limit", lambda device: 1 << 40)
+    assert plan.ds_head_runs(B, Hq, Hkv, 128, S) == 1                    # small workspace: one run
+    monkeypatch.setattr(BA, "_DS_RUN_TARGET", 1)
+    monkeypatch.setattr(BA, "_DS_RUN_MIN_WORKGROUPS", 2 * key_tiles)     # a run keeps at least two kv heads
+    assert plan.ds_head_runs(B, Hq, Hkv, 128, S) == 4
+    monkeypatch.setattr(BA, "_DS_RUN_MIN_WORKGROUPS", 8 * key_tiles + 1)  # no run is large enough: not split
+    assert plan.ds_head_runs(B, Hq, Hkv, 128, S) == 1
+    BA.BitfieldUtils.clear_cache()
