@@ -29,6 +29,14 @@ __device__ __forceinline__ void dma_b128(const void* sbase, unsigned voff, unsig
                  "n"(SITE)
                  : "memory");
 }
+// The same with the non-temporal hint: data that is read once (it should not displace what other workgroups re-read
+// from the L2).
+template <int SITE = 0>
+__device__ __forceinline__ void dma_b128_stream(const void* sbase, unsigned voff, unsigned lds_base) {
+    asm volatile("s_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 nt ; site %3" ::"v"(voff), "s"(sbase), "{m0}"(lds_base),
+                 "n"(SITE)
+                 : "memory");
+}
 template <int SITE = 0>
 __device__ __forceinline__ void dma_b32(const void* sbase, unsigned voff, unsigned lds_base) {
     asm volatile("s_nop 0\n\tglobal_load_lds_dword %0, %1 ; site %3" ::"v"(voff), "s"(sbase), "{m0}"(lds_base),

@@ -146,8 +146,8 @@ __global__ __launch_bounds__(DQS_THREADS, 2) void bwd_dq_saved_kernel(const Attn
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb)
             if ((c >> (2 * kb)) & 3) {
-                dma_b128<1>(rec + kb * 2048, (unsigned)(lane * 16), ldsDS + buf * 4096u + kb * 2048u);
-                dma_b128<2>(rec + kb * 2048, (unsigned)(lane * 16 + 1024), ldsDS + buf * 4096u + kb * 2048u + 1024u);
+                dma_b128_stream<1>(rec + kb * 2048, (unsigned)(lane * 16), ldsDS + buf * 4096u + kb * 2048u);
+                dma_b128_stream<2>(rec + kb * 2048, (unsigned)(lane * 16 + 1024), ldsDS + buf * 4096u + kb * 2048u + 1024u);
                 issued += 2;
             }
         return issued;

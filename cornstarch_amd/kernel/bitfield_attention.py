@@ -86,7 +86,8 @@ _DS_LIMIT_ENV = os.environ.get("BAM_DS_WORKSPACE_LIMIT_GB")
 # as long as the dK/dV launch of a run keeps this many workgroups (128-key tiles x batch x kv heads of the run: four
 # rounds of the chip's 256 compute units).  One sequence of 65536 tokens with 32 q heads and 8 kv heads: 47 GiB in
 # one run, 12 GiB in four runs, the same 41.9 ms either way (and 46.6 ms in eight runs of one kv head each).
-_DS_RUN_TARGET = 16 << 30
+# BAM_DS_WORKSPACE_TARGET_GB overrides the size (a value at or above the limit means: one run whenever it fits).
+_DS_RUN_TARGET = int(float(os.environ.get("BAM_DS_WORKSPACE_TARGET_GB", "16")) * (1 << 30))
 _DS_RUN_MIN_WORKGROUPS = 1024
 
 
