@@ -312,7 +312,7 @@ extern "C" {
 
 const char* bam_last_error(void) { return g_error; }
 
-int bam_abi_version(void) { return 9; }
+int bam_abi_version(void) { return 10; }
 
 int bam_tile_flags(const int64_t* bf, int64_t bf_stride_b, int8_t* flags, int64_t flags_stride_b,
                    int64_t flags_stride_m, int B, int S, void* stream) {
@@ -330,7 +330,7 @@ namespace {
 struct PlanLayout {
     int64_t fine_ss, fine_sb, order_sb, entry_sb, fine_off, order_off, entry_off, base_off, count_off, bytes;
     int64_t row_sn, row_sb, col_ss, col_sb, row_off, col_off, bytes_with_bits, tile_count_off, tile_order_off;
-    int64_t group_count_off, group_order_off;
+    int64_t group_count_off, group_order_off, row_workloads_off;
 };
 PlanLayout plan_layout(int B, int Sq, int Sk) {
     const int64_t num_m = (Sq + 127) / 128, num_n = (Sk + 31) / 32, slots = 4 * num_m;
@@ -349,7 +349,8 @@ PlanLayout plan_layout(int B, int Sq, int Sk) {
     l.tile_order_off = l.tile_count_off + up(B * ((Sk + 127) / 128) * 4, 256);
     l.group_count_off = l.tile_order_off + up(B * ((Sk + 127) / 128) * 4, 256);
     l.group_order_off = l.group_count_off + up(B * num_m * 4, 256);
-    l.bytes = l.group_order_off + up(B * num_m * 4, 256);
+    l.row_workloads_off = l.group_order_off + up(B * num_m * 4, 256);
+    l.bytes = l.row_workloads_off + up(num_m * 8, 256);
     // the packed mask of bam_mask_tile_plan: rows padded to 128, keys to 128, 32-key blocks to an even number
     l.row_sn = num_m * 128;
     l.row_sb = ((num_n + 1) & ~(int64_t)1) * l.row_sn;
@@ -399,6 +400,7 @@ int place_plan(const char* who, void* workspace, int64_t workspace_bytes, int B,
     plan->ds_count = (const int32_t*)(w + l.count_off);
     plan->ds_tile_order = (int64_t)B * ((Sk + 127) / 128) <= bam::MAX_RANKED ? (const int32_t*)(w + l.tile_order_off) : nullptr;
     plan->group_order = (int64_t)B * ((Sq + 127) / 128) <= bam::MAX_RANKED ? (const int32_t*)(w + l.group_order_off) : nullptr;
+    plan->row_workloads = (const int64_t*)(w + l.row_workloads_off);
     plan->ds_workspace = nullptr;
     plan->ds_capacity = 0;
     plan->row_bits = with_bits ? (const uint32_t*)(w + l.row_off) : nullptr;
@@ -423,7 +425,8 @@ int number_pairs(const char* who, const bam_plan* plan, const PlanLayout& l, voi
                                            (int*)((char*)workspace + l.tile_count_off),
                                            const_cast<int*>(plan->ds_tile_order), plan->order, plan->order_stride_b,
                                            (int*)((char*)workspace + l.group_count_off),
-                                           const_cast<int*>(plan->group_order), (hipStream_t)stream),
+                                           const_cast<int*>(plan->group_order),
+                                           const_cast<int64_t*>(plan->row_workloads), (hipStream_t)stream),
                     who);
 }
 }  // namespace

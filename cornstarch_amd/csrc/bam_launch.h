@@ -135,10 +135,11 @@ int launch_mask_tile_plan(const uint8_t* mask, int8_t* flags, int64_t flags_stri
 // tile_order (B * ceil(Sk/128)): the key tiles by falling number of pairs, written by a second small launch; both may
 // be null, and no order is written beyond MAX_RANKED tiles.  The same for the groups of four slices in the plan's slice
 // order (order, order_sb): group_count (B * num_m) scratch, group_order (B * num_m) = the groups by falling number of
-// 64-key tiles they visit.
+// 64-key tiles they visit.  row_workloads (num_m int64, or null): per 128-row block, the number of its 128 x 32 tiles
+// with an allowed pair, summed over the batch.
 int launch_ds_entries(const uint8_t* fine, int64_t fine_sb, int64_t fine_ss, int B, int Sq, int Sk, int* entry,
                       int64_t entry_sb, int* tile_base, int* count, int* tile_count, int* tile_order, const int* order,
-                      int64_t order_sb, int* group_count, int* group_order, hipStream_t stream);
+                      int64_t order_sb, int* group_count, int* group_order, int64_t* row_workloads, hipStream_t stream);
 int launch_fwd(const AttnParams& p, int dtype, hipStream_t stream);
 int launch_bwd_preprocess(const AttnParams& p, int dtype, hipStream_t stream);
 int launch_bwd_dkdv(const AttnParams& p, int dtype, hipStream_t stream);

@@ -667,11 +667,36 @@ __global__ __launch_bounds__(DS_NUM_THREADS) void ds_entries_kernel(const uint8_
                                                                    int* __restrict__ tile_base, int* __restrict__ count,
                                                                    int* __restrict__ tile_count,
                                                                    const int* __restrict__ order, int64_t order_sb,
-                                                                   int* __restrict__ group_count) {
+                                                                   int* __restrict__ group_count, int group_blocks,
+                                                                   long long* __restrict__ row_workloads) {
     __shared__ int wave_sum[DS_NUM_THREADS / 64];
     __shared__ int s_base;
     const int b = blockIdx.y;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    if ((int)blockIdx.x >= nkt + group_blocks) {
+        // Extra workgroups, one per 128-row block m (those of batch entry 0 do the work): in how many of the block's
+        // 128 x 32 tiles, over the whole batch, some pair is allowed -- the sum of (flags > 0) over batch and key
+        // columns (reference shardformer/layers/utils.py:161-166).  A 128 x 32 flag is non-zero exactly when one of the
+        // classes of its four 32 x 32 tiles is.
+        if (b != 0) return;
+        const int m = blockIdx.x - nkt - group_blocks, nb = gridDim.y;
+        int tiles = 0;
+        for (int bb = 0; bb < nb; ++bb) {
+            const uint8_t* rows = fine + (int64_t)bb * fine_sb + (int64_t)(4 * m) * fine_ss;
+            for (int n = tid; n < num_n; n += DS_NUM_THREADS)
+                tiles += (rows[n] | rows[fine_ss + n] | rows[2 * fine_ss + n] | rows[3 * fine_ss + n]) != 0 ? 1 : 0;
+        }
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) tiles += __shfl_xor(tiles, off);
+        if (lane == 0) wave_sum[wave] = tiles;
+        __syncthreads();
+        if (tid == 0) {
+            long long total = 0;
+            for (int w = 0; w < DS_NUM_THREADS / 64; ++w) total += wave_sum[w];
+            row_workloads[m] = total;
+        }
+        return;
+    }
     if ((int)blockIdx.x >= nkt) {
         // Extra workgroups, one per group of four slices of the slice order: how many 64-key tiles the forward / dQ
         // workgroup of that group visits (the union over its slices), which is what group_order ranks the groups by.
@@ -779,15 +804,17 @@ __global__ __launch_bounds__(256) void tile_order_kernel(const int* __restrict__
 
 int launch_ds_entries(const uint8_t* fine, int64_t fine_sb, int64_t fine_ss, int B, int Sq, int Sk, int* entry,
                       int64_t entry_sb, int* tile_base, int* count, int* tile_count, int* tile_order, const int* order,
-                      int64_t order_sb, int* group_count, int* group_order, hipStream_t stream) {
+                      int64_t order_sb, int* group_count, int* group_order, int64_t* row_workloads, hipStream_t stream) {
     const int num_m = (Sq + BLOCK_M - 1) / BLOCK_M;
     const int slots = 4 * num_m, nkt = (Sk + 127) / 128, num_n = (Sk + BLOCK_N - 1) / BLOCK_N;
     const int n_tiles = nkt * B, n_groups = num_m * B;
     if (n_tiles > DS_MAX_ORDERED_TILES || tile_count == nullptr) tile_order = nullptr;
     if (n_groups > DS_MAX_ORDERED_TILES || group_count == nullptr || order == nullptr) group_order = nullptr;
-    hipLaunchKernelGGL(ds_entries_kernel, dim3(nkt + (group_order != nullptr ? num_m : 0), B), dim3(DS_NUM_THREADS), 0,
-                       stream, fine, fine_sb, fine_ss, slots, nkt, num_n, entry, entry_sb, tile_base, count,
-                       tile_order != nullptr ? tile_count : nullptr, order, order_sb, group_count);
+    const int group_blocks = group_order != nullptr ? num_m : 0;
+    hipLaunchKernelGGL(ds_entries_kernel, dim3(nkt + group_blocks + (row_workloads != nullptr ? num_m : 0), B),
+                       dim3(DS_NUM_THREADS), 0, stream, fine, fine_sb, fine_ss, slots, nkt, num_n, entry, entry_sb,
+                       tile_base, count, tile_order != nullptr ? tile_count : nullptr, order, order_sb, group_count,
+                       group_blocks, (long long*)row_workloads);
     if (tile_order != nullptr || group_order != nullptr) {
         const int nt = tile_order != nullptr ? n_tiles : 0, ng = group_order != nullptr ? n_groups : 0;
         hipLaunchKernelGGL(tile_order_kernel, dim3((max(nt, ng) + 63) / 64, group_order != nullptr ? 2 : 1), dim3(256), 0,

@@ -15,7 +15,7 @@ BAM_DTYPE_F16 = 0
 BAM_DTYPE_BF16 = 1
 BAM_MAX_SEQLEN = 4194304
 BAM_STATIC_PLAN_BYTES = 8 << 20
-ABI_VERSION = 9
+ABI_VERSION = 10
 
 _i64 = ctypes.c_int64
 _int = ctypes.c_int
@@ -64,6 +64,7 @@ class Plan(ctypes.Structure):
         ("ds_count", ctypes.c_void_p),
         ("ds_tile_order", ctypes.c_void_p),
         ("group_order", ctypes.c_void_p),
+        ("row_workloads", ctypes.c_void_p),
         ("ds_workspace", ctypes.c_void_p),
         ("ds_capacity", ctypes.c_int64),
         ("row_bits", ctypes.c_void_p),

@@ -156,6 +156,7 @@ class _TilePlan:
         self.workspace = workspace  # keeps the device memory alive
         self.struct = struct
         self.flags = flags  # None for plans that are not tied to a flags tensor (index-tensor attention)
+        self.flags_version = flags._version if flags is not None else -1  # (the builder wrote through raw pointers)
         # The number of (slice, 128-key tile) pairs that have work is device data; it sizes the dS workspace of the
         # backward.  Its copy to the host is enqueued here, right behind the kernels that compute it, and awaited
         # only when a backward asks for it -- by then it has long arrived.
@@ -173,6 +174,13 @@ class _TilePlan:
         workspace.record_stream(side)
         self._pairs_event = torch.cuda.Event()
         self._pairs_event.record(side)
+
+    def row_workloads(self) -> torch.Tensor:
+        """int64 (ceil(Sq/128),): non-empty 128 x 32 tiles of each row block, summed over the batch; a view into the
+        plan's workspace, written by the plan builder's numbering launch."""
+        num_m = -(-self.struct.Sq // 128)
+        ws = self.workspace
+        return torch.as_strided(ws.view(torch.int64), (num_m,), (1,), (self.struct.row_workloads - ws.data_ptr()) // 8)
 
     def ds_pairs(self) -> int:
         """How many (32-row slice, 128-key tile) pairs have work (waits for the asynchronous copy on first use)."""
@@ -383,6 +391,14 @@ class BitfieldUtils:
         sequence split sorts by (reference shardformer/layers/utils.py:161-171), computed on the GPU so that
         only this small vector has to travel to the host."""
         assert compressed_mask.is_cuda and compressed_mask.dtype == torch.int8 and compressed_mask.dim() == 3
+        with _CACHE_LOCK:
+            plan, cached = cls._plan, cls.compressed_mask_cache
+        # the cached flags tensor itself, unwritten since it was built: its plan already holds the sums, so nothing is
+        # launched; the result is a view into the plan's workspace (read it, do not write it)
+        if (plan is not None and cached is not None and plan.flags is cached and plan.struct.row_workloads
+                and compressed_mask.data_ptr() == cached.data_ptr() and compressed_mask.shape == cached.shape
+                and compressed_mask.stride() == cached.stride() and compressed_mask._version == plan.flags_version):
+            return plan.row_workloads()
         flags = compressed_mask if compressed_mask.stride(-1) == 1 else compressed_mask.contiguous()
         batch_size, num_m, num_n = flags.shape
         out = torch.empty((num_m,), dtype=torch.int32, device=flags.device)

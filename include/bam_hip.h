@@ -123,6 +123,11 @@ typedef struct bam_plan {
                                    slices of `order` (code b * ceil(Sq/128) + group) by falling number of 64-key tiles
                                    they visit, the order in which the forward and dQ kernels take their workgroups, so
                                    that the longest start first whatever the sequences of a batch look like */
+    const int64_t* row_workloads; /* device, ceil(Sq/128) int64: per 128-row block, the number of its 128 x 32 tiles in
+                                     which some pair is allowed, summed over the batch -- sum(flags > 0) over batch and
+                                     key columns, the workloads the reference's makespan-minimizing sequence split sorts
+                                     by (shardformer/layers/utils.py:161-166); written by the plan builders' numbering
+                                     launch, so a caller that builds a plan needs no bam_flag_row_workloads call */
     void* ds_workspace;        /* device, at least bam_ds_workspace_bytes(Hq, pairs) bytes, 16-byte aligned */
     int64_t ds_capacity;       /* pairs the workspace has room for: at least *ds_count */
     /* Materialized masks only (bam_mask_tile_plan; null otherwise): the mask packed to bits, once per orientation, so

@@ -158,6 +158,7 @@ def test_mask_plan_classes_and_results_do_not_depend_on_the_plan(Sq, Sk, D, monk
     want = torch.where(cnt == 0, 0, torch.where(cnt == tot, 2, 1)).to(torch.uint8)
     fine = plan.fine_classes().cpu()
     assert torch.equal(fine[:, :n_q], want) and (fine[:, n_q:] == 0).all()
+    assert torch.equal(plan.row_workloads().cpu(), torch.sum(flags.cpu() > 0, dim=(0, 2)))  # per 128-row block
     for b in range(2):
         order = plan.slice_order()[b].cpu().tolist()
         assert order[:n_q] == list(range(n_q - 1, -1, -1)) and all(x == -1 for x in order[n_q:])

@@ -117,6 +117,27 @@ def test_row_block_workloads_for_the_makespan_split(S):
     assert torch.equal(BA.BitfieldUtils.nonempty_tiles_per_row_block(flags), torch.sum(flags > 0, dim=(0, 2)))
 
 
+@pytest.mark.parametrize("B,S", [(1, 57), (3, 335), (2, 1024), (2, 3712), (5, 2049)])
+def test_row_block_workloads_come_with_the_plan(B, S):
+    # the plan builder's numbering launch leaves the same sums in the plan: the flags tensor the cache holds gets them
+    # from there (no launch), any other flags tensor -- a copy, a re-indexed one, one written since -- from the kernel
+    bf = random_bitfield(B, S, seed=S + B, pad=min(5, S - 1)).to(dev())
+    BA.BitfieldUtils.clear_cache()
+    flags = BA.BitfieldUtils.materialize_compressed_mask_from_bitfield_mask(bf)
+    plan = BA.BitfieldUtils.plan_for(flags, bf)
+    assert plan is not None and plan.struct.row_workloads
+    want = torch.sum(flags > 0, dim=(0, 2))
+    from_plan = BA.BitfieldUtils.nonempty_tiles_per_row_block(flags)
+    assert from_plan.dtype == torch.int64 and from_plan.data_ptr() == plan.row_workloads().data_ptr()
+    assert torch.equal(from_plan, want)
+    copy = flags.clone()
+    from_kernel = BA.BitfieldUtils.nonempty_tiles_per_row_block(copy)
+    assert from_kernel.data_ptr() != plan.row_workloads().data_ptr() and torch.equal(from_kernel, want)
+    flags[:, 0, 0] = 0  # written since the plan was built: counted again
+    assert torch.equal(BA.BitfieldUtils.nonempty_tiles_per_row_block(flags), torch.sum(flags > 0, dim=(0, 2)))
+    BA.BitfieldUtils.clear_cache()
+
+
 def test_flags_of_a_strided_bitfield_row_view():
     base = random_bitfield(4, 600, seed=11)
     big = torch.zeros((4, 1000), dtype=torch.int64)
